@@ -1,0 +1,161 @@
+/*
+ * C ABI of libmoe_hip.so: the FP8 fused-MoE inference path for AMD MI355X (gfx950).
+ *
+ * Plain C, no torch types.  Every pointer is a DEVICE pointer unless the comment says
+ * otherwise; every entry point enqueues its kernels on `stream` (a hipStream_t passed as
+ * void*) and returns without synchronising.  Nothing here allocates: outputs, scratch and
+ * the workspace are the caller's (the reference's ops follow the same rule: the caller of
+ * torch_tpu/csrc/ops/my_ops/fusedMoE.cpp:117-236 allocates output and all scratch).
+ *
+ * Return value: 0 = enqueued; < 0 = invalid argument (MOE_E_*); > 0 = a hipError_t raised
+ * by a launch.  Never throws.  This mirrors the reference's inner launcher convention
+ * (`int moe_multi_core_bf16_fp8e4m3(stream, addrs..., ints...)` returning 0 or an error
+ * code, torch_tpu/csrc/ops/my_ops/fusedMoE.cpp:27-37) and its status enum
+ * (third_party/tpuDNN/include/tpuDNN.h:8-12).
+ *
+ * Data formats
+ *   fp8      OCP e4m3fn bytes (gfx950's native FP8), saturating encode at +-448.
+ *   W13      [E, 2*I, H] fp8, rows 0..I-1 = gate projection, rows I..2I-1 = up projection,
+ *            fp32 scales [E, 2*I/128, H/128]  (one per 128x128 block).
+ *   W2       [E, H, I] fp8, fp32 scales [E, H/128, I/128].
+ *   acts     bf16 [T, H]; quantised per token per 128 columns: scale = max(amax,1e-10)/448.
+ *   ids      int32 [T, K], the K experts of a token are distinct.
+ *   H and I must be multiples of 128.
+ */
+#ifndef MOE_HIP_H
+#define MOE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MOE_OK                0
+#define MOE_E_NULL           -1   /* a required pointer is NULL                          */
+#define MOE_E_SHAPE          -2   /* a dimension is out of the supported range           */
+#define MOE_E_ALIGN          -3   /* H or I not a multiple of 128, or pointer misaligned */
+#define MOE_E_WORKSPACE      -4   /* workspace smaller than moe_workspace_bytes()        */
+#define MOE_E_MODE           -5   /* unknown mode / dtype selector                       */
+
+#define MOE_DTYPE_F32   0
+#define MOE_DTYPE_BF16  1
+
+#define MOE_ROUTE_SOFTMAX 0   /* select on logits; weights = softmax over all experts      */
+#define MOE_ROUTE_SIGMOID 1   /* scores = sigmoid(logit); select on scores + bias          */
+#define MOE_ROUTE_SCORES  2   /* the input already holds scores; select on scores + bias   */
+
+#define MOE_MAX_EXPERTS 1024
+#define MOE_MAX_TOPK    32
+
+/* Library version (major*10000 + minor*100 + patch) and the gfx target it was built for. */
+int moe_hip_version(void);
+const char *moe_hip_arch(void);
+/* Text for a code returned by any entry point (static storage). */
+const char *moe_hip_strerror(int code);
+
+/*
+ * Group-limited top-k.  Replaces at::noaux_tc_topk -> tpudnnNoauxTcTopkAsync
+ * (torch_tpu/csrc/ops/my_ops/NoauxTcTopk.cpp:9-67, third_party/tpuDNN/include/tpuDNNTensor.h:728-737).
+ * scores [T, E] viewed [T, n_groups, E/n_groups]; group score = sum of the group's two best
+ * scores, rounded to the scores' dtype; the `topk_groups` best groups stay, the others
+ * count as -inf; `top_k` best of the row follow, descending.  Equal values: lower index wins.
+ * values_out [T, top_k] in the scores' dtype, indices_out [T, top_k] int32.
+ */
+int moe_noaux_tc_topk(void *stream, const void *scores, int scores_dtype, int T, int E,
+                      int n_groups, int topk_groups, int top_k,
+                      void *values_out, int32_t *indices_out);
+
+/*
+ * Router selection + weights from logits (or scores).  Replaces the aten recipe the
+ * reference's callers run (python/regression/test_llm/test_torch_ops.py:441-456:
+ * sigmoid -> topk -> sum -> div -> mul) and the softmax/top-k variant
+ * (torch_tpu/csrc/ops/native_ops/Topk.cpp:91-205).
+ * logits [T, E] (dtype selector), bias [E] fp32 or NULL (added for selection only).
+ * n_groups <= 1 disables group limiting.  renorm != 0 divides by the sum of the selected
+ * weights; the result is multiplied by `scale`.
+ * weights_out [T, K] fp32, ids_out [T, K] int32 (descending selection order),
+ * scores_out [T, E] fp32 or NULL (the scores selection ran on, before the bias).
+ */
+int moe_route_topk(void *stream, const void *logits, int logits_dtype, const float *bias,
+                   int T, int E, int K, int mode, int n_groups, int topk_groups,
+                   int renorm, float scale,
+                   float *weights_out, int32_t *ids_out, float *scores_out);
+
+/*
+ * Token permutation = stable counting sort of the flattened ids.  Replaces the index
+ * building phases of the reference kernel (torch_tpu/csrc/ops/my_ops/fusedMoE.pl:624-756:
+ * per expert, ascending token ids / ascending flat slot ids).
+ * sorted_slot [T*K]: flat slot ids t*K+k grouped by expert, ascending inside an expert.
+ * expert_offsets [E+1]: rows of expert e are sorted_slot[expert_offsets[e] .. expert_offsets[e+1]).
+ * slot_to_row [T*K]: inverse permutation.
+ * Ids outside [0, E) are dropped: they get no row, slot_to_row = -1.
+ * workspace: moe_permute_workspace_bytes(T, K, E) bytes.
+ */
+size_t moe_permute_workspace_bytes(int T, int K, int E);
+/* Rows of one expert that a grouped-GEMM workgroup owns for this problem shape (16..128); the
+ * permutation leaves the matching tile list in its workspace.  The reference's launcher picks
+ * its token slice per core the same way, on the host (fusedMoE.cpp:60-78). */
+int moe_tile_rows(int T, int K, int E);
+int moe_permute(void *stream, const int32_t *ids, int T, int K, int E,
+                int32_t *sorted_slot, int32_t *expert_offsets, int32_t *slot_to_row,
+                void *workspace, size_t workspace_bytes);
+
+/*
+ * Per-token, per-128-column dynamic quantisation of bf16 activations.
+ * x [R, C] bf16 -> q [R, C] fp8, s [R, C/128] fp32.  No counterpart in the open part of the
+ * reference (its W8A8 sibling is closed: torch_tpu/csrc/ops/my_ops/MlpW8A8Quant.cpp:34-46).
+ */
+int moe_act_quant(void *stream, const void *x_bf16, int R, int C, uint8_t *q, float *s);
+
+/*
+ * The expert computation.  Replaces at::fused_moe_fused_experts ->
+ * tpudnnFusedMoEFusedExpertsMultiCoreAsync (torch_tpu/csrc/ops/my_ops/fusedMoE.cpp:117-236,
+ * third_party/tpuDNN/include/tpuDNNTensor.h:1585-1610) and its _v2 twin (fusedMoE.cpp:237-318):
+ *   permute -> quantise x -> grouped FP8 GEMM with W13 + SwiGLU + re-quantise
+ *           -> grouped FP8 GEMM with W2 -> un-permute.
+ * out_mode 0: out is bf16 [T, K, H], un-weighted per-slot results (the reference's form;
+ *             routing_weights may be NULL).
+ * out_mode 1: out is bf16 [T, H] = sum_k routing_weights[t,k] * slot result (fp32 sum).
+ *             If the shared_* pointers are non-NULL a shared expert (W13 [1,2*I_sh,H],
+ *             W2 [1,H,I_sh]) is applied to every token and added with weight 1.
+ * workspace: moe_fused_experts_workspace_bytes(...) bytes, 256-byte aligned.
+ */
+size_t moe_fused_experts_workspace_bytes(int T, int H, int I, int E, int K, int I_shared);
+int moe_fused_experts_fp8(void *stream,
+                          const void *x_bf16, int T, int H,
+                          const uint8_t *w13, const float *w13_scale,
+                          const uint8_t *w2, const float *w2_scale, int I, int E,
+                          const int32_t *ids, const float *routing_weights, int K,
+                          const uint8_t *shared_w13, const float *shared_w13_scale,
+                          const uint8_t *shared_w2, const float *shared_w2_scale, int I_shared,
+                          void *out_bf16, int out_mode,
+                          void *workspace, size_t workspace_bytes);
+
+/*
+ * Stages of the above, exposed for tests and for timing one kernel at a time.  All take
+ * the permutation produced by moe_permute() and the tile list it leaves in its workspace.
+ *
+ * moe_gemm1_swiglu:  hq [T*K, I] fp8 / hs [T*K, I/128] fp32 (rows in permuted order)
+ *                    = requant(silu(x W_gate^T) * (x W_up^T)) with xq/xs from moe_act_quant.
+ * moe_gemm2:         y [T*K, H] bf16, row of slot s at y[s] (slot order, i.e. [T, K, H]).
+ * moe_weighted_reduce: out [T, H] bf16 = sum_k w[t,k] * y[t,k,:] (+ shared_y[t,:] if given).
+ */
+int moe_gemm1_swiglu(void *stream, const uint8_t *xq, const float *xs, int T, int H,
+                     const uint8_t *w13, const float *w13_scale, int I, int E, int K,
+                     const int32_t *sorted_slot, const int32_t *expert_offsets,
+                     const void *permute_workspace,
+                     uint8_t *hq, float *hs);
+int moe_gemm2(void *stream, const uint8_t *hq, const float *hs, int T, int H,
+              const uint8_t *w2, const float *w2_scale, int I, int E, int K,
+              const int32_t *sorted_slot, const int32_t *expert_offsets,
+              const void *permute_workspace,
+              void *y_bf16);
+int moe_weighted_reduce(void *stream, const void *y_bf16, const float *routing_weights,
+                        const void *shared_y_bf16, int T, int K, int H, void *out_bf16);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOE_HIP_H */

@@ -1,0 +1,40 @@
+import json
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+import __graft_entry__ as entry  # noqa: E402
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a ROCm GPU (run with -m gpu on an MI355X)")
+
+
+@pytest.fixture(scope="session")
+def oracle():
+    return entry.load_oracle()
+
+
+@pytest.fixture(scope="session")
+def pkg():
+    """The package under test; importing it loads libmoe_hip.so and fails loudly if absent."""
+    return entry.load_package()
+
+
+@pytest.fixture(scope="session")
+def ref_fixtures():
+    with open(os.path.join(ROOT, "tests", "golden", "reference_fixtures.json")) as f:
+        return json.load(f)
+
+
+@pytest.fixture(scope="session")
+def dev():
+    import torch
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return "cuda:0"

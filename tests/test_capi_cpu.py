@@ -1,0 +1,110 @@
+"""The C-ABI library without a GPU: it loads, exports every symbol the header declares, and
+rejects bad arguments before touching a device."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "moe_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(moe_\w+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    syms = declared_symbols()
+    for s in ["moe_fused_experts_fp8", "moe_noaux_tc_topk", "moe_route_topk", "moe_permute", "moe_act_quant",
+              "moe_gemm1_swiglu", "moe_gemm2", "moe_weighted_reduce", "moe_hip_version"]:
+        assert s in syms
+
+
+def test_library_exports_every_declared_symbol(pkg):
+    lib = ctypes.CDLL(os.path.join(ROOT, "torch-tpu_amd", "libmoe_hip.so"))
+    for s in declared_symbols():
+        assert hasattr(lib, s), f"{s} is declared in include/moe_hip.h but not exported"
+
+
+def test_binding_table_covers_the_header(pkg):
+    from torch_tpu_amd import _lib
+    assert sorted(_lib.SIGNATURES) == declared_symbols()
+
+
+def test_version_and_arch(pkg):
+    from torch_tpu_amd._lib import lib
+    assert lib.moe_hip_version() >= 100
+    assert lib.moe_hip_arch() == b"gfx950"
+    assert lib.moe_hip_strerror(0) == b"ok"
+    assert b"NULL" in lib.moe_hip_strerror(-1)
+
+
+def test_argument_errors_are_codes_not_crashes(pkg):
+    from torch_tpu_amd._lib import lib
+    E_NULL, E_SHAPE, E_ALIGN, E_WS, E_MODE = -1, -2, -3, -4, -5
+    fake = ctypes.c_void_p(0x1000)          # never dereferenced: validation fails first
+    assert lib.moe_act_quant(None, None, 4, 128, fake, fake) == E_NULL
+    assert lib.moe_act_quant(None, fake, 4, 100, fake, fake) == E_ALIGN
+    assert lib.moe_noaux_tc_topk(None, fake, 7, 1, 256, 8, 4, 8, fake, fake) == E_MODE
+    assert lib.moe_noaux_tc_topk(None, fake, 0, 1, 250, 8, 4, 8, fake, fake) == E_SHAPE      # 250 % 8 != 0
+    assert lib.moe_noaux_tc_topk(None, fake, 0, 1, 4096, 8, 4, 8, fake, fake) == E_SHAPE     # too many experts
+    assert lib.moe_route_topk(None, fake, 0, None, 1, 8, 9, 0, 1, 1, 1, 1.0, fake, fake, None) == E_SHAPE
+    assert lib.moe_route_topk(None, fake, 0, None, 1, 8, 2, 9, 1, 1, 1, 1.0, fake, fake, None) == E_MODE
+    assert lib.moe_permute(None, fake, 4, 2, 8, fake, fake, fake, fake, 16) == E_WS
+    assert lib.moe_permute(None, fake, 4, 2, 5000, fake, fake, fake, fake, 1 << 20) == E_SHAPE
+    ws = lib.moe_fused_experts_workspace_bytes(4, 256, 512, 8, 2, 0)
+    assert ws > 0 and ws % 256 == 0
+    args = dict(T=4, H=256, I=512, E=8, K=2)
+
+    def fused(x=fake, H=256, I=512, out_mode=0, wsb=ws, rw=None, workspace=fake):
+        return lib.moe_fused_experts_fp8(None, x, 4, H, fake, fake, fake, fake, I, 8, fake, rw, 2,
+                                         None, None, None, None, 0, fake, out_mode, workspace, wsb)
+    assert fused(x=None) == E_NULL
+    assert fused(H=200) == E_ALIGN
+    assert fused(I=100) == E_ALIGN
+    assert fused(out_mode=3) == E_MODE
+    assert fused(out_mode=1) == E_NULL            # weighted output needs routing weights
+    assert fused(wsb=ws - 1) == E_WS
+    assert fused(workspace=ctypes.c_void_p(0x1004)) == E_ALIGN
+    del args
+
+
+def test_workspace_sizes_grow_with_the_problem(pkg):
+    from torch_tpu_amd._lib import lib
+    small = lib.moe_fused_experts_workspace_bytes(16, 256, 512, 8, 2, 0)
+    big = lib.moe_fused_experts_workspace_bytes(4096, 7168, 2048, 256, 8, 2048)
+    assert 0 < small < big
+    # the big pieces: y [T*K, H] bf16 + hq [T*K, I] + xq [T, H]
+    assert big >= 4096 * 8 * 7168 * 2 + 4096 * 8 * 2048 + 4096 * 7168
+    assert lib.moe_permute_workspace_bytes(4096, 8, 256) >= (4096 * 8 // 256) * 256 * 4
+    for T in (1, 16, 17, 32, 33, 64, 65, 4096):
+        assert lib.moe_tile_rows(T, 8, 256) in (16, 32, 64, 128)
+
+
+def test_python_wrappers_validate_before_launch(pkg):
+    import torch
+    x = torch.zeros(4, 256, dtype=torch.bfloat16)          # CPU tensor: must be refused
+    with pytest.raises(RuntimeError, match="GPU"):
+        pkg.act_quant(x)
+    with pytest.raises(RuntimeError, match="int32"):
+        pkg.noaux_tc_topk(torch.zeros(1, 8), torch.zeros(1, 8, dtype=torch.int64), torch.zeros(1, 256), 8, 4, 8)
+    with pytest.raises(RuntimeError, match="same dtype"):
+        pkg.noaux_tc_topk(torch.zeros(1, 8, dtype=torch.bfloat16), torch.zeros(1, 8, dtype=torch.int32),
+                          torch.zeros(1, 256), 8, 4, 8)
+
+
+def test_my_ops_are_registered_with_reference_arity(pkg):
+    import torch
+    ops = torch.ops.my_ops
+    assert len(ops.fused_moe_fused_experts.default._schema.arguments) == 25
+    assert len(ops.fused_moe_fused_experts_v2.default._schema.arguments) == 27
+    assert len(ops.noaux_tc_topk.default._schema.arguments) == 6
+    assert len(ops.fused_moe_grouped_topk.default._schema.arguments) == 10
+    with pytest.raises(RuntimeError, match="closed-source"):
+        ops.fused_moe_grouped_topk(*[torch.zeros(1)] * 10)
+    z = torch.zeros(1, 1, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="int32"):
+        ops.fused_moe_fused_experts(z, z[0], None, None, z, z, z, z, z, z, torch.zeros(1, 1, dtype=torch.int64),
+                                    z[0], None, None, None, 128, 1, 1, True, 8, 4, None, None, None, False)

@@ -1,0 +1,308 @@
+"""Parity of the HIP path with the CPU oracle, through the C ABI, on a real MI355X.
+
+Integer results (routing ids, permutation, e4m3 codes of the activation quantiser) must be
+bit-exact; bf16 outputs must be within rtol 2e-2 / atol 1e-2 of the oracle's fp32 computation
+on the same quantised operands.
+"""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 2e-2, 1e-2
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def distinct_ids(T, E, K, seed, gen_weights=True):
+    g = torch.Generator().manual_seed(seed)
+    ids = torch.argsort(torch.rand(T, E, generator=g), dim=-1)[:, :K].to(torch.int32).contiguous()
+    w = torch.rand(T, K, generator=g) + 0.1
+    w = (w / w.sum(-1, keepdim=True)).float()
+    return ids, w
+
+
+# ----------------------------------------------------------------------------- quantiser
+@pytest.mark.parametrize("R,C", [(1, 128), (16, 256), (33, 7168), (257, 2048)])
+def test_act_quant_bit_exact(pkg, oracle, dev, R, C):
+    say("act_quant", R, C)
+    g = torch.Generator().manual_seed(R * 1000 + C)
+    x = torch.randn(R, C, generator=g)
+    x[0, :128] = 0.0                                     # an all-zero group
+    if R > 1:
+        x[1, :128] *= 1e4                                # large magnitudes
+        x[1, 128:] *= 1e-6 if C > 128 else 1             # tiny magnitudes
+    x = x.to(torch.bfloat16)
+    q_ref, s_ref = oracle.act_quant_group128(x)
+    q, s = pkg.act_quant(x.to(dev))
+    torch.cuda.synchronize()
+    assert torch.equal(s.cpu(), s_ref)
+    assert torch.equal(q.cpu().view(torch.uint8), q_ref.view(torch.uint8))
+
+
+# ----------------------------------------------------------------------------- routing
+@pytest.mark.parametrize("batch", [1, 8, 16, 64, 128])
+def test_noaux_tc_topk_reference_cases(pkg, oracle, dev, batch):
+    say("noaux reference case", batch)
+    torch.manual_seed(42)
+    scores = torch.stack([torch.randperm(256, dtype=torch.float32)]).reshape(1, -1).to(torch.bfloat16).repeat(batch, 1)
+    v_ref, i_ref = oracle.noaux_tc_topk(scores.clone(), 8, 4, 8)
+    values = torch.empty(batch, 8, dtype=torch.bfloat16, device=dev)
+    indices = torch.empty(batch, 8, dtype=torch.int32, device=dev)
+    ret = torch.ops.my_ops.noaux_tc_topk(values, indices, scores.to(dev), 8, 4, 8)
+    torch.cuda.synchronize()
+    assert ret.data_ptr() == values.data_ptr()
+    assert torch.equal(indices.cpu(), i_ref)
+    assert torch.allclose(values.cpu().float(), v_ref.float(), rtol=1e-5, atol=1e-6)
+    assert all(len({i // 32 for i in row}) <= 4 for row in indices.cpu().tolist())
+
+
+def test_noaux_tc_topk_err_data(pkg, oracle, dev, ref_fixtures):
+    say("noaux err_data")
+    row = ref_fixtures["noaux_tc_topk_err_data"]
+    for dtype in (torch.float32, torch.bfloat16):
+        scores = torch.tensor([row], dtype=torch.float32).to(dtype)
+        v_ref, i_ref = oracle.noaux_tc_topk(scores, 8, 4, 8)
+        values = torch.empty(1, 8, dtype=dtype, device=dev)
+        indices = torch.empty(1, 8, dtype=torch.int32, device=dev)
+        pkg.noaux_tc_topk(values, indices, scores.to(dev), 8, 4, 8)
+        torch.cuda.synchronize()
+        assert torch.equal(indices.cpu(), i_ref) and torch.equal(values.cpu(), v_ref)
+
+
+@pytest.mark.parametrize("T,E,G,TG,K,dtype", [
+    (300, 256, 8, 4, 8, torch.float32), (300, 256, 8, 4, 8, torch.bfloat16), (64, 64, 4, 2, 6, torch.float32),
+    (17, 16, 8, 3, 2, torch.float32), (5, 1024, 16, 5, 32, torch.float32), (40, 128, 1, 1, 8, torch.float32),
+    (9, 96, 3, 2, 7, torch.bfloat16),
+])
+def test_noaux_tc_topk_random_with_ties(pkg, oracle, dev, T, E, G, TG, K, dtype):
+    say("noaux random", T, E, G, TG, K, dtype)
+    g = torch.Generator().manual_seed(T + E)
+    scores = torch.randn(T, E, generator=g)
+    scores[::3] = torch.round(scores[::3] * 2) / 2          # many exact ties
+    scores = scores.to(dtype)
+    v_ref, i_ref = oracle.noaux_tc_topk(scores, G, TG, K)
+    values = torch.empty(T, K, dtype=dtype, device=dev)
+    indices = torch.empty(T, K, dtype=torch.int32, device=dev)
+    pkg.noaux_tc_topk(values, indices, scores.to(dev), G, TG, K)
+    torch.cuda.synchronize()
+    assert torch.equal(indices.cpu(), i_ref)
+    assert torch.equal(values.cpu(), v_ref)
+
+
+@pytest.mark.parametrize("T,E,K", [(16, 8, 2), (4096, 8, 2), (1000, 128, 8), (7, 64, 6)])
+def test_route_softmax(pkg, oracle, dev, T, E, K):
+    say("route softmax", T, E, K)
+    g = torch.Generator().manual_seed(E * 7 + T)
+    logits = torch.randn(T, E, generator=g) * 2
+    w_ref, i_ref = oracle.route_softmax_topk(logits, K, renorm=True)
+    w, ids, scores = pkg.moe_route(logits.to(dev), K, "softmax", return_scores=True)
+    torch.cuda.synchronize()
+    assert torch.equal(ids.cpu(), i_ref)
+    assert torch.allclose(w.cpu(), w_ref, rtol=1e-5, atol=1e-7)
+    assert torch.allclose(scores.cpu(), torch.softmax(logits, -1), rtol=1e-5, atol=1e-8)
+    w2, ids2 = pkg.moe_route(logits.to(dev), K, "softmax", renorm=False)
+    w2_ref, _ = oracle.route_softmax_topk(logits, K, renorm=False)
+    assert torch.equal(ids2.cpu(), i_ref) and torch.allclose(w2.cpu(), w2_ref, rtol=1e-5, atol=1e-8)
+    # bf16 logits are widened exactly
+    wb, idb = pkg.moe_route(logits.to(torch.bfloat16).to(dev), K, "softmax")
+    wb_ref, idb_ref = oracle.route_softmax_topk(logits.to(torch.bfloat16), K)
+    assert torch.equal(idb.cpu(), idb_ref) and torch.allclose(wb.cpu(), wb_ref, rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.parametrize("T,E,K,G,TG,with_bias", [(4096, 256, 8, 8, 4, True), (32, 256, 8, 8, 4, False),
+                                                  (16, 128, 4, 1, 1, False), (100, 64, 6, 4, 2, True)])
+def test_route_sigmoid_grouped(pkg, oracle, dev, T, E, K, G, TG, with_bias):
+    say("route sigmoid", T, E, K, G, TG, with_bias)
+    g = torch.Generator().manual_seed(E + T)
+    logits = torch.randn(T, E, generator=g)
+    bias = (torch.randn(E, generator=g) * 0.1) if with_bias else None
+    w, ids, scores = pkg.moe_route(logits.to(dev), K, "sigmoid", bias=None if bias is None else bias.to(dev),
+                                   n_groups=G, topk_groups=TG, renorm=True, scale=2.5, return_scores=True)
+    torch.cuda.synchronize()
+    scores = scores.cpu()
+    assert torch.allclose(scores, torch.sigmoid(logits), rtol=1e-6, atol=1e-7)
+    # selection is exact GIVEN the scores the device computed (sigmoid may differ in the last ulp)
+    w_ref, i_ref = oracle.select_sigmoid_grouped(scores, bias, K, G, TG, 2.5, True)
+    assert torch.equal(ids.cpu(), i_ref)
+    assert torch.allclose(w.cpu(), w_ref, rtol=1e-5, atol=1e-7)
+    # and identical when the same scores are handed in directly
+    w3, ids3 = pkg.moe_route(scores.to(dev), K, "scores", bias=None if bias is None else bias.to(dev), n_groups=G,
+                             topk_groups=TG, renorm=True, scale=2.5)
+    assert torch.equal(ids3.cpu(), i_ref) and torch.allclose(w3.cpu(), w_ref, rtol=1e-5, atol=1e-7)
+
+
+# ----------------------------------------------------------------------------- permutation
+def check_permutation(pkg, oracle, dev, sel, E):
+    ss_ref, off_ref, s2r_ref = oracle.permute_counting_sort(sel, E)
+    ss, off, s2r = pkg.moe_permute(sel.to(dev), E)
+    torch.cuda.synchronize()
+    assert torch.equal(off.cpu(), off_ref)
+    assert torch.equal(ss.cpu(), ss_ref)
+    assert torch.equal(s2r.cpu(), s2r_ref)
+
+
+@pytest.mark.parametrize("name", ["SELECTED_EXPERTS_B8_E256", "SELECTED_EXPERTS_B22_E256"])
+def test_permutation_reference_tables(pkg, oracle, dev, ref_fixtures, name):
+    say("permute table", name)
+    sel = torch.tensor(ref_fixtures[name], dtype=torch.int32)
+    check_permutation(pkg, oracle, dev, sel, 256)
+    gather, scatter = oracle.permute_literal(sel, 256)
+    ss, off, _ = pkg.moe_permute(sel.to(dev), 256)
+    ss, off = ss.cpu(), off.cpu()
+    for e in range(256):
+        assert ss[off[e]:off[e + 1]].tolist() == scatter[e]
+
+
+@pytest.mark.parametrize("T,E,K", [(1, 1, 1), (1, 256, 8), (32, 256, 8), (33, 8, 2), (4096, 256, 8), (1000, 1024, 32),
+                                   (5000, 3, 2), (16384, 128, 8)])
+def test_permutation_random(pkg, oracle, dev, T, E, K):
+    say("permute random", T, E, K)
+    sel, _ = distinct_ids(T, E, K, seed=T + E + K)
+    check_permutation(pkg, oracle, dev, sel, E)
+
+
+def test_permutation_skewed_with_empty_experts(pkg, oracle, dev):
+    say("permute zipf")
+    T, E, K = 16384, 128, 8
+    g = torch.Generator().manual_seed(5)
+    bias = -1.2 * torch.log(torch.arange(1, E + 1).float())
+    bias[torch.randperm(E, generator=g)[:13]] = -1e9
+    logits = torch.randn(T, E, generator=g) + bias
+    _, sel = oracle.route_softmax_topk(logits, K)
+    counts = torch.bincount(sel.flatten().long(), minlength=E)
+    assert (counts == 0).sum() >= 13
+    check_permutation(pkg, oracle, dev, sel, E)
+
+
+# ----------------------------------------------------------------------------- experts
+def run_layer(pkg, dev, x, layer, ids, w, out_shape, shared=None):
+    w13q, w13s, w2q, w2s = (t.to(dev) for t in layer)
+    sh = None if shared is None else tuple(t.to(dev) for t in shared)
+    out = torch.full(out_shape, float("nan"), dtype=torch.bfloat16, device=dev)
+    pkg.fused_experts_fp8(x.to(dev), w13q, w13s, w2q, w2s, ids.to(dev), None if w is None else w.to(dev), out=out,
+                          shared=sh)
+    torch.cuda.synchronize()
+    return out.float().cpu()
+
+
+@pytest.mark.parametrize("T,H,I,E,K", [
+    (16, 256, 512, 8, 2),        # the toy configuration
+    (1, 256, 128, 1, 1), (1, 7168, 256, 2, 2), (1, 7168, 256, 16, 8), (8, 7168, 256, 256, 8),   # reference grid
+    (17, 512, 384, 8, 2), (33, 512, 256, 4, 2), (64, 1024, 256, 16, 4), (65, 256, 256, 8, 2),
+    (200, 512, 256, 8, 2), (300, 256, 128, 3, 2), (256, 7168, 256, 256, 8),
+])
+def test_fused_experts_per_slot_and_weighted(pkg, oracle, dev, T, H, I, E, K):
+    say("fused experts", T, H, I, E, K)
+    layer = oracle.make_layer(E, H, I, seed=H + I + E)
+    g = torch.Generator().manual_seed(T)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    ids, w = distinct_ids(T, E, K, seed=T * 3 + E)
+    ref = oracle.experts_w8a8_fp32(x, ids, *layer)
+    out = run_layer(pkg, dev, x, layer, ids, None, (T, K, H))
+    torch.testing.assert_close(out, ref, rtol=RTOL, atol=ATOL)
+    out2 = run_layer(pkg, dev, x, layer, ids, w, (T, H))
+    torch.testing.assert_close(out2, oracle.weighted_reduce(ref, w), rtol=RTOL, atol=ATOL)
+    cd, _, _ = oracle.cal_diff(ref, out)
+    assert oracle.cos_sim(ref.numpy(), out.numpy()) > 0.9999 and cd < 1e-4
+
+
+def test_fused_experts_stage_outputs(pkg, oracle, dev):
+    say("stage outputs")
+    T, H, I, E, K = 150, 512, 256, 8, 2
+    layer = oracle.make_layer(E, H, I, seed=3)
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    ids, w = distinct_ids(T, E, K, seed=5)
+    ref, (xq_ref, xs_ref, hq_ref, hs_ref) = oracle.experts_w8a8_fp32(x, ids, *layer, return_mid=True)
+    w13q, w13s, w2q, w2s = (t.to(dev) for t in layer)
+    xq, xs = pkg.act_quant(x.to(dev))
+    ss, off, s2r, ws = pkg.moe_permute(ids.to(dev), E, return_workspace=True)
+    hq, hs = pkg.gemm1_swiglu(xq, xs, w13q, w13s, (T, K), ss, off, ws)
+    y = pkg.gemm2(hq, hs, w2q, w2s, (T, K), ss, off, ws)
+    torch.cuda.synchronize()
+    # rows of hq are in permuted order: row r belongs to slot sorted_slot[r]
+    slot = ss.cpu().long()
+    h_dev = hq.cpu().float() * hs.cpu().repeat_interleave(128, -1)
+    h_ref = (hq_ref.view(torch.float8_e4m3fn).float() * hs_ref.repeat_interleave(128, -1)).reshape(T * K, I)[slot]
+    assert torch.allclose(hs.cpu(), hs_ref.reshape(T * K, -1)[slot], rtol=1e-4)
+    same = (hq.cpu().view(torch.uint8) == hq_ref.reshape(T * K, I)[slot]).float().mean().item()
+    assert same > 0.995, same
+    torch.testing.assert_close(h_dev, h_ref, rtol=0.13, atol=1e-3)      # a flipped code moves one e4m3 step
+    torch.testing.assert_close(y.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+    out = pkg.weighted_reduce(y, w.to(dev))
+    torch.testing.assert_close(out.float().cpu(), oracle.weighted_reduce(ref, w), rtol=RTOL, atol=ATOL)
+
+
+def test_fused_experts_with_shared_expert_and_empty_experts(pkg, oracle, dev):
+    say("shared expert")
+    T, H, I, E, K = 70, 512, 256, 16, 4
+    layer = oracle.make_layer(E, H, I, seed=6)
+    shared = oracle.make_layer(1, H, 384, seed=7)
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    ids, w = distinct_ids(T, 8, K, seed=9)               # experts 8..15 never chosen
+    ref = oracle.moe_w8a8_fp32(x, ids, w, *layer, shared=shared)
+    out = run_layer(pkg, dev, x, layer, ids, w, (T, H), shared=shared)
+    torch.testing.assert_close(out, ref, rtol=RTOL, atol=ATOL)
+
+
+def test_my_ops_drop_in_reference_layout(pkg, oracle, dev):
+    """The reference's call, argument for argument (python/regression/test_llm/test_moe.py:119-140):
+    separate gate/up weights, pre-transposed down, bf16 scales, [T,K,H] output."""
+    say("my_ops drop-in")
+    T, H, I, E, K = 8, 7168, 256, 256, 8
+    g = torch.Generator().manual_seed(1000)
+    rnd = random.Random(1000)
+    sel = torch.tensor([rnd.sample(range(E), K) for _ in range(T)], dtype=torch.int32)
+    w0 = (torch.randn(E, I, H, generator=g) * 0.1).to(torch.float8_e4m3fn)
+    w1 = (torch.randn(E, I, H, generator=g) * 0.1).to(torch.float8_e4m3fn)
+    w2 = (torch.randn(E, H, I, generator=g) * 0.1).to(torch.float8_e4m3fn)
+    s0 = (torch.randn(E, I // 128, H // 128, generator=g) * 0.1).to(torch.bfloat16)
+    s1 = (torch.randn(E, I // 128, H // 128, generator=g) * 0.1).to(torch.bfloat16)
+    s2 = (torch.randn(E, H // 128, I // 128, generator=g) * 0.1).to(torch.bfloat16)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    rw = torch.randn(T, K, generator=g).to(torch.bfloat16)
+    ref_bf16 = oracle.experts_ref_bf16(x, sel, w0, w1, w2, s0, s1, s2).float()
+    ref_w8a8 = oracle.experts_w8a8_fp32(x, sel, torch.cat([w0, w1], 1), torch.cat([s0, s1], 1).float(), w2, s2.float())
+    out = torch.empty(T, K, H, dtype=torch.bfloat16, device=dev)
+    scratch = [torch.empty(E, T, dtype=torch.int32, device=dev) for _ in range(3)]
+    scratch.append(torch.empty(E, T, K, dtype=torch.int32, device=dev))
+    args = [out, x.to(dev), None, None, w0.to(dev), w1.to(dev), w2.transpose(1, 2).contiguous().to(dev),
+            s0.to(dev), s1.to(dev), s2.transpose(1, 2).contiguous().to(dev), sel.to(dev), rw.to(dev), None]
+    tail = [128, E, K, True, 8, 4, None, None, None, False]
+    ret = torch.ops.my_ops.fused_moe_fused_experts(*args, scratch[0], scratch[1], *tail)
+    torch.cuda.synchronize()
+    assert ret.data_ptr() == out.data_ptr()
+    got = out.float().cpu()
+    scale = ref_w8a8.abs().max().item()
+    torch.testing.assert_close(got / scale, ref_w8a8 / scale, rtol=RTOL, atol=ATOL)
+    assert oracle.cos_sim(ref_bf16.numpy(), got.numpy()) > 0.99
+    out.zero_()
+    torch.ops.my_ops.fused_moe_fused_experts_v2(*args, scratch[0], scratch[1], scratch[2], scratch[3], *tail)
+    torch.cuda.synchronize()
+    assert torch.equal(out.float().cpu(), got)
+
+
+def test_layer_module_end_to_end_toy_config(pkg, oracle, dev):
+    say("toy config end to end")
+    T, H, I, E, K = 16, 256, 512, 8, 2
+    layer = oracle.make_layer(E, H, I, seed=0)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    wr = (torch.randn(E, H, generator=g) * 0.02).to(torch.bfloat16)
+    moe = pkg.FusedMoE(wr.to(dev), *(t.to(dev) for t in layer), top_k=K, mode="softmax")
+    xd = x.to(dev)
+    w, ids = moe.route(xd)
+    out = moe.experts(xd, w, ids)
+    torch.cuda.synchronize()
+    logits_dev = torch.matmul(xd, wr.to(dev).t()).float().cpu()
+    w_ref, ids_ref = oracle.route_softmax_topk(logits_dev, K)
+    assert torch.equal(ids.cpu(), ids_ref)
+    ref = oracle.moe_w8a8_fp32(x, ids_ref, w_ref, *layer)
+    torch.testing.assert_close(out.float().cpu(), ref, rtol=RTOL, atol=ATOL)

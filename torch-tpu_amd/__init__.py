@@ -1,0 +1,15 @@
+"""MI355X-native FP8 fused-MoE inference path behind torch-tpu's `my_ops` operator surface.
+
+Importing the package loads libmoe_hip.so (hand-written gfx950 kernels behind a C ABI) and
+registers `torch.ops.my_ops.{fused_moe_fused_experts, fused_moe_fused_experts_v2, noaux_tc_topk,
+fused_moe_grouped_topk}`.  There is no CPU fallback: without the built library the import fails.
+"""
+from . import _lib                      # noqa: F401  (raises if the library is missing)
+from . import my_ops as _my_ops         # noqa: F401  (registers torch.ops.my_ops.*)
+from .layer import FusedMoE, pack_expert_weights
+from .ops import (MoeHipError, act_quant, fused_experts_fp8, fused_experts_workspace_bytes, gemm1_swiglu, gemm2,
+                  moe_permute, moe_route, noaux_tc_topk, tile_rows, weighted_reduce)
+
+__all__ = ["FusedMoE", "pack_expert_weights", "MoeHipError", "act_quant", "fused_experts_fp8",
+           "fused_experts_workspace_bytes", "gemm1_swiglu", "gemm2", "moe_permute", "moe_route", "noaux_tc_topk",
+           "tile_rows", "weighted_reduce"]

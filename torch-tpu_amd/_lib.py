@@ -1,0 +1,59 @@
+"""ctypes binding of libmoe_hip.so (the C ABI declared in include/moe_hip.h).
+
+There is no fallback: if the library is missing or a symbol is absent, importing this
+module raises, and every op built on it is unavailable.
+"""
+import ctypes
+import os
+from ctypes import c_char_p, c_float, c_int, c_size_t, c_void_p
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libmoe_hip.so")
+
+# name -> (restype, argtypes); the single source for both binding and the symbol test
+SIGNATURES = {
+    "moe_hip_version": (c_int, []),
+    "moe_hip_arch": (c_char_p, []),
+    "moe_hip_strerror": (c_char_p, [c_int]),
+    "moe_tile_rows": (c_int, [c_int, c_int, c_int]),
+    "moe_noaux_tc_topk": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "moe_route_topk": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                               c_int, c_float, c_void_p, c_void_p, c_void_p]),
+    "moe_permute_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "moe_permute": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t]),
+    "moe_act_quant": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p]),
+    "moe_fused_experts_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
+    "moe_fused_experts_fp8": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                      c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                                      c_void_p, c_int, c_void_p, c_int, c_void_p, c_size_t]),
+    "moe_gemm1_swiglu": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
+                                 c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "moe_gemm2": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
+                          c_void_p, c_void_p, c_void_p, c_void_p]),
+    "moe_weighted_reduce": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+}
+
+
+class MoeHipError(RuntimeError):
+    pass
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python {os.path.join(HERE, 'build.py')}` "
+            "(hipcc, gfx950). There is no CPU fallback.")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)          # AttributeError if the symbol is absent
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+lib = _load()
+
+
+def check(rc: int, what: str):
+    if rc != 0:
+        raise MoeHipError(f"{what}: {lib.moe_hip_strerror(rc).decode()} (code {rc})")

@@ -1,0 +1,130 @@
+// The whole-path entry point and the library's housekeeping calls.
+#include "moe_common.h"
+#include "moe_layout.h"
+#include "../../include/moe_hip.h"
+
+namespace moe {
+
+int permute_launch(hipStream_t st, const int32_t *ids, int T, int K, int E, int tile_m, int32_t *sorted_slot,
+                   int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &ws);
+int gemm1_launch(hipStream_t st, const uint8_t *xq, const float *xs, int T, int H, const uint8_t *w13,
+                 const float *w13s, int I, int E, int K, const int32_t *sorted_slot, const int32_t *expert_offsets,
+                 const PermuteWs *pw, int fixed_expert, uint8_t *hq, float *hs);
+int gemm2_launch(hipStream_t st, const uint8_t *hq, const float *hs, int rows_a, int T, int H, const uint8_t *w2,
+                 const float *w2s, int I, int E, int K, const int32_t *sorted_slot, const int32_t *expert_offsets,
+                 const PermuteWs *pw, int fixed_expert, uint16_t *y);
+
+// Carves the caller's workspace.  Every piece starts on a 256-byte boundary.
+struct FusedWs {
+  void *permute;
+  int32_t *sorted_slot, *expert_offsets, *slot_to_row;
+  uint8_t *xq;
+  float *xs;
+  uint8_t *hq;
+  float *hs;
+  uint16_t *y;
+  uint8_t *sh_hq;
+  float *sh_hs;
+  uint16_t *sh_y;
+  size_t bytes;
+};
+
+static FusedWs fused_layout(void *base, int T, int H, int I, int E, int K, int I_sh) {
+  FusedWs w{};
+  size_t off = 0;
+  auto take = [&](size_t n) {
+    void *p = base ? (void *)((uint8_t *)base + off) : nullptr;
+    off += align_up(n ? n : 1, 256);
+    return p;
+  };
+  const size_t TK = (size_t)T * K;
+  w.permute = take(permute_ws_bytes(T, K, E));
+  w.sorted_slot = (int32_t *)take(TK * 4);
+  w.expert_offsets = (int32_t *)take((size_t)(E + 1) * 4);
+  w.slot_to_row = (int32_t *)take(TK * 4);
+  w.xq = (uint8_t *)take((size_t)T * H);
+  w.xs = (float *)take((size_t)T * (H / kBlock) * 4);
+  w.hq = (uint8_t *)take(TK * I);
+  w.hs = (float *)take(TK * (I / kBlock) * 4);
+  w.y = (uint16_t *)take(TK * H * 2);
+  if (I_sh > 0) {
+    w.sh_hq = (uint8_t *)take((size_t)T * I_sh);
+    w.sh_hs = (float *)take((size_t)T * (I_sh / kBlock) * 4);
+    w.sh_y = (uint16_t *)take((size_t)T * H * 2);
+  }
+  w.bytes = off;
+  return w;
+}
+
+}  // namespace moe
+
+extern "C" int moe_hip_version(void) { return 100; }
+extern "C" const char *moe_hip_arch(void) { return "gfx950"; }
+
+extern "C" const char *moe_hip_strerror(int code) {
+  switch (code) {
+    case MOE_OK: return "ok";
+    case MOE_E_NULL: return "a required pointer is NULL";
+    case MOE_E_SHAPE: return "a dimension is out of the supported range";
+    case MOE_E_ALIGN: return "H or I is not a multiple of 128, or a pointer is misaligned";
+    case MOE_E_WORKSPACE: return "workspace too small";
+    case MOE_E_MODE: return "unknown mode or dtype selector";
+    default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
+  }
+}
+
+extern "C" size_t moe_fused_experts_workspace_bytes(int T, int H, int I, int E, int K, int I_shared) {
+  if (T < 0 || H < 1 || I < 1 || E < 1 || K < 1 || I_shared < 0) return 0;
+  return moe::fused_layout(nullptr, T, H, I, E, K, I_shared).bytes;
+}
+
+extern "C" int moe_fused_experts_fp8(void *stream, const void *x_bf16, int T, int H, const uint8_t *w13,
+                                     const float *w13_scale, const uint8_t *w2, const float *w2_scale, int I, int E,
+                                     const int32_t *ids, const float *routing_weights, int K,
+                                     const uint8_t *shared_w13, const float *shared_w13_scale,
+                                     const uint8_t *shared_w2, const float *shared_w2_scale, int I_shared,
+                                     void *out_bf16, int out_mode, void *workspace, size_t workspace_bytes) {
+  using namespace moe;
+  if (!x_bf16 || !w13 || !w13_scale || !w2 || !w2_scale || !ids || !out_bf16 || !workspace) return MOE_E_NULL;
+  if (out_mode != 0 && out_mode != 1) return MOE_E_MODE;
+  if (out_mode == 1 && !routing_weights) return MOE_E_NULL;
+  if (T < 0 || H < 1 || I < 1 || E < 1 || E > MOE_MAX_EXPERTS || K < 1 || K > MOE_MAX_TOPK || K > E) return MOE_E_SHAPE;
+  if ((long)T * K > (1l << 30)) return MOE_E_SHAPE;
+  if (H % kBlock || I % kBlock) return MOE_E_ALIGN;
+  const bool has_shared = shared_w13 != nullptr;
+  if (has_shared) {
+    if (out_mode != 1) return MOE_E_MODE;
+    if (!shared_w13_scale || !shared_w2 || !shared_w2_scale) return MOE_E_NULL;
+    if (I_shared < 1) return MOE_E_SHAPE;
+    if (I_shared % kBlock) return MOE_E_ALIGN;
+  }
+  const int I_sh = has_shared ? I_shared : 0;
+  if (((uintptr_t)workspace % 256) || ((uintptr_t)x_bf16 % 16) || ((uintptr_t)out_bf16 % 16) ||
+      ((uintptr_t)w13 % 16) || ((uintptr_t)w2 % 16))
+    return MOE_E_ALIGN;
+  FusedWs w = fused_layout(workspace, T, H, I, E, K, I_sh);
+  if (workspace_bytes < w.bytes) return MOE_E_WORKSPACE;
+  if (T == 0) return MOE_OK;
+
+  hipStream_t st = (hipStream_t)stream;
+  PermuteWs pw = permute_ws_layout(w.permute, T, K, E);
+  int rc = permute_launch(st, ids, T, K, E, choose_tile_m(T, K, E), w.sorted_slot, w.expert_offsets, w.slot_to_row, pw);
+  if (rc) return rc;
+  rc = moe_act_quant(stream, x_bf16, T, H, w.xq, w.xs);
+  if (rc) return rc;
+  rc = gemm1_launch(st, w.xq, w.xs, T, H, w13, w13_scale, I, E, K, w.sorted_slot, w.expert_offsets, &pw, -1, w.hq, w.hs);
+  if (rc) return rc;
+  uint16_t *y = out_mode == 0 ? (uint16_t *)out_bf16 : w.y;
+  rc = gemm2_launch(st, w.hq, w.hs, T * K, T, H, w2, w2_scale, I, E, K, w.sorted_slot, w.expert_offsets, &pw, -1, y);
+  if (rc) return rc;
+  if (out_mode == 0) return MOE_OK;
+  if (has_shared) {
+    rc = gemm1_launch(st, w.xq, w.xs, T, H, shared_w13, shared_w13_scale, I_sh, 1, 1, nullptr, nullptr, nullptr, 0,
+                      w.sh_hq, w.sh_hs);
+    if (rc) return rc;
+    rc = gemm2_launch(st, w.sh_hq, w.sh_hs, T, T, H, shared_w2, shared_w2_scale, I_sh, 1, 1, nullptr, nullptr, nullptr,
+                      0, w.sh_y);
+    if (rc) return rc;
+  }
+  return moe_weighted_reduce(stream, y, routing_weights, has_shared ? w.sh_y : nullptr, T, K, H, out_bf16);
+}

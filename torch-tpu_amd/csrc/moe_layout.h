@@ -1,0 +1,61 @@
+// Host-side layout of the caller-provided workspaces (shared by the launchers).
+#pragma once
+#include <stddef.h>
+#include <stdint.h>
+
+namespace moe {
+
+constexpr int kChunk = 256;   // slots ranked by one wavefront in the permutation kernels
+
+static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// Rows of one expert that a grouped-GEMM workgroup owns.  A pure function of the problem
+// shape so that the permutation (which builds the tile list) and the GEMM launchers agree
+// without passing it around.  A token's K experts are distinct, so no expert ever holds
+// more than T rows: small T gets small tiles.
+static inline int choose_tile_m(int T, int K, int E) {
+  (void)K; (void)E;
+  if (T <= 16) return 16;
+  if (T <= 32) return 32;
+  if (T <= 64) return 64;
+  return 128;
+}
+
+struct PermuteWs {
+  int32_t *chunk_counts;   // [n_chunks, E]
+  int32_t *tile_prefix;    // [E + 1] first tile of each expert; [E] = number of tiles
+  int32_t *tile_expert;    // [max_tiles]
+  int n_chunks;
+  int max_tiles;
+};
+
+static inline int permute_max_tiles(int T, int K, int E) {
+  const int tm = choose_tile_m(T, K, E);
+  long tk = (long)T * K;
+  long a = tk / tm + E;           // sum_e ceil(n_e / tm) <= TK/tm + (#non-empty experts)
+  long b = tk;                    // and never more than one tile per row
+  long m = a < b ? a : b;
+  return (int)(m < 1 ? 1 : m);
+}
+
+static inline size_t permute_ws_bytes(int T, int K, int E) {
+  long tk = (long)T * K;
+  size_t n_chunks = (size_t)((tk + kChunk - 1) / kChunk);
+  if (n_chunks == 0) n_chunks = 1;
+  size_t ints = n_chunks * (size_t)E + (size_t)(E + 1) + (size_t)permute_max_tiles(T, K, E);
+  return align_up(ints * 4, 256);
+}
+
+static inline PermuteWs permute_ws_layout(void *ws, int T, int K, int E) {
+  PermuteWs p;
+  long tk = (long)T * K;
+  p.n_chunks = (int)((tk + kChunk - 1) / kChunk);
+  if (p.n_chunks == 0) p.n_chunks = 1;
+  p.max_tiles = permute_max_tiles(T, K, E);
+  p.chunk_counts = (int32_t *)ws;
+  p.tile_prefix = p.chunk_counts + (size_t)p.n_chunks * E;
+  p.tile_expert = p.tile_prefix + (E + 1);
+  return p;
+}
+
+}  // namespace moe

@@ -1,0 +1,237 @@
+// Token permutation: a stable counting sort of the flattened [T*K] expert ids.
+//
+// Three small kernels, no host round trip (the grouped GEMMs that follow read the expert
+// offsets and the tile list from device memory):
+//   count    one wavefront per chunk of kChunk consecutive slots: per-chunk histogram in LDS.
+//   scan     one workgroup: per expert, running sum over the chunks (turns the histogram into
+//            the chunk's starting rank inside its expert), then an exclusive scan over the
+//            experts -> expert_offsets, and the list of row tiles the GEMMs walk.
+//   scatter  one wavefront per chunk again: ranks its slots in slot order with a ballot
+//            "match-any" loop, so equal experts keep their original order (stable), and writes
+//            sorted_slot / slot_to_row.
+// A problem of at most kChunk slots is done by one wavefront in a single launch.
+#include "moe_common.h"
+#include "moe_layout.h"
+#include "../../include/moe_hip.h"
+
+namespace moe {
+
+// rank of each lane among the lanes holding the same expert id, in lane order; also the
+// size of that set and whether the lane is the last of it.
+__device__ __forceinline__ void match_rank(int v, bool valid, int lane, int &rank, int &cnt, bool &is_last) {
+  uint64_t todo = __ballot(valid);
+  rank = 0; cnt = 0; is_last = false;
+  const uint64_t lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  while (todo) {
+    int leader = __ffsll((unsigned long long)todo) - 1;
+    int lv = __shfl(v, leader, 64);
+    uint64_t m = __ballot(valid && v == lv);
+    if (valid && v == lv) {
+      rank = __popcll(m & lt);
+      cnt = __popcll(m);
+      is_last = (lane == 63 - __clzll((long long)m));
+    }
+    todo &= ~m;
+  }
+}
+
+__global__ __launch_bounds__(64) void permute_count_kernel(const int32_t *__restrict__ ids, int TK, int E,
+                                                           int32_t *__restrict__ chunk_counts) {
+  __shared__ int hist[MOE_MAX_EXPERTS];
+  const int lane = threadIdx.x, c = blockIdx.x;
+  for (int e = lane; e < E; e += 64) hist[e] = 0;
+  __syncthreads();
+  const int lo = c * kChunk;
+  for (int s = lo + lane; s < min(lo + kChunk, TK); s += 64) {
+    int v = ids[s];
+    if (v >= 0 && v < E) atomicAdd(&hist[v], 1);
+  }
+  __syncthreads();
+  for (int e = lane; e < E; e += 64) chunk_counts[(size_t)c * E + e] = hist[e];
+}
+
+// exclusive scan of one value per thread over a 1024-thread workgroup
+__device__ __forceinline__ int block_exclusive_scan(int x, int *lds_wave_sums, int &total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int inc = x;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    int y = __shfl_up(inc, off, 64);
+    if (lane >= off) inc += y;
+  }
+  if (lane == 63) lds_wave_sums[wave] = inc;
+  __syncthreads();
+  int base = 0, tot = 0;
+  for (int w = 0; w < (int)(blockDim.x >> 6); w++) {
+    int s = lds_wave_sums[w];
+    if (w < wave) base += s;
+    tot += s;
+  }
+  __syncthreads();
+  total = tot;
+  return base + inc - x;
+}
+
+__device__ __forceinline__ void write_tiles(int e, int count, int first_tile, int tile_m, int32_t *tile_expert,
+                                            int max_tiles) {
+  int nt = (count + tile_m - 1) / tile_m;
+  for (int j = 0; j < nt; j++)
+    if (first_tile + j < max_tiles) tile_expert[first_tile + j] = e;
+}
+
+__global__ __launch_bounds__(1024) void permute_scan_kernel(int32_t *__restrict__ chunk_counts, int n_chunks, int E,
+                                                            int tile_m, int max_tiles,
+                                                            int32_t *__restrict__ expert_offsets,
+                                                            int32_t *__restrict__ tile_prefix,
+                                                            int32_t *__restrict__ tile_expert) {
+  __shared__ int wave_sums[16];
+  const int e = threadIdx.x;
+  int count = 0;
+  if (e < E) {
+    for (int c = 0; c < n_chunks; c++) {
+      int x = chunk_counts[(size_t)c * E + e];
+      chunk_counts[(size_t)c * E + e] = count;   // rank of the chunk's first slot inside expert e
+      count += x;
+    }
+  }
+  int total;
+  int off = block_exclusive_scan(count, wave_sums, total);
+  int tiles = (count + tile_m - 1) / tile_m;
+  int total_tiles;
+  int first_tile = block_exclusive_scan(tiles, wave_sums, total_tiles);
+  if (e < E) {
+    expert_offsets[e] = off;
+    tile_prefix[e] = first_tile;
+    write_tiles(e, count, first_tile, tile_m, tile_expert, max_tiles);
+  }
+  if (e == 0) {
+    expert_offsets[E] = total;
+    tile_prefix[E] = total_tiles;
+  }
+}
+
+__global__ __launch_bounds__(64) void permute_scatter_kernel(const int32_t *__restrict__ ids, int TK, int E,
+                                                             const int32_t *__restrict__ chunk_counts,
+                                                             const int32_t *__restrict__ expert_offsets,
+                                                             int32_t *__restrict__ sorted_slot,
+                                                             int32_t *__restrict__ slot_to_row) {
+  __shared__ int base[MOE_MAX_EXPERTS];
+  const int lane = threadIdx.x, c = blockIdx.x;
+  for (int e = lane; e < E; e += 64) base[e] = expert_offsets[e] + chunk_counts[(size_t)c * E + e];
+  __syncthreads();
+  const int lo = c * kChunk;
+  const int hi = min(lo + kChunk, TK);
+  for (int s0 = lo; s0 < hi; s0 += 64) {
+    const int s = s0 + lane;
+    int v = (s < hi) ? ids[s] : -1;
+    const bool valid = (s < hi) && v >= 0 && v < E;
+    int rank, cnt;
+    bool is_last;
+    match_rank(v, valid, lane, rank, cnt, is_last);
+    int row = valid ? base[v] + rank : -1;
+    __syncthreads();
+    if (valid && is_last) base[v] += cnt;
+    __syncthreads();
+    if (valid && row < TK) sorted_slot[row] = s;
+    if (s < hi) slot_to_row[s] = row;
+  }
+}
+
+// whole permutation of at most kChunk slots by one wavefront
+__global__ __launch_bounds__(64) void permute_small_kernel(const int32_t *__restrict__ ids, int TK, int E, int tile_m,
+                                                           int max_tiles, int32_t *__restrict__ sorted_slot,
+                                                           int32_t *__restrict__ expert_offsets,
+                                                           int32_t *__restrict__ slot_to_row,
+                                                           int32_t *__restrict__ tile_prefix,
+                                                           int32_t *__restrict__ tile_expert) {
+  __shared__ int hist[MOE_MAX_EXPERTS];
+  __shared__ int base[MOE_MAX_EXPERTS];
+  const int lane = threadIdx.x;
+  for (int e = lane; e < E; e += 64) hist[e] = 0;
+  __syncthreads();
+  for (int s = lane; s < TK; s += 64) {
+    int v = ids[s];
+    if (v >= 0 && v < E) atomicAdd(&hist[v], 1);
+  }
+  __syncthreads();
+  // lane owns experts [lane*per, lane*per+per)
+  const int per = (E + 63) / 64;
+  int sum = 0, tsum = 0;
+  for (int j = 0; j < per; j++) {
+    int e = lane * per + j;
+    if (e < E) { sum += hist[e]; tsum += (hist[e] + tile_m - 1) / tile_m; }
+  }
+  int inc = sum, tinc = tsum;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    int y = __shfl_up(inc, off, 64), ty = __shfl_up(tinc, off, 64);
+    if (lane >= off) { inc += y; tinc += ty; }
+  }
+  int run = inc - sum, trun = tinc - tsum;
+  for (int j = 0; j < per; j++) {
+    int e = lane * per + j;
+    if (e < E) {
+      int cnt = hist[e];
+      expert_offsets[e] = run;
+      base[e] = run;
+      tile_prefix[e] = trun;
+      write_tiles(e, cnt, trun, tile_m, tile_expert, max_tiles);
+      run += cnt;
+      trun += (cnt + tile_m - 1) / tile_m;
+    }
+  }
+  if (lane == 63) { expert_offsets[E] = inc; tile_prefix[E] = tinc; }
+  __syncthreads();
+  for (int s0 = 0; s0 < TK; s0 += 64) {
+    const int s = s0 + lane;
+    int v = (s < TK) ? ids[s] : -1;
+    const bool valid = (s < TK) && v >= 0 && v < E;
+    int rank, cnt;
+    bool is_last;
+    match_rank(v, valid, lane, rank, cnt, is_last);
+    int row = valid ? base[v] + rank : -1;
+    __syncthreads();
+    if (valid && is_last) base[v] += cnt;
+    __syncthreads();
+    if (valid && row < TK) sorted_slot[row] = s;
+    if (s < TK) slot_to_row[s] = row;
+  }
+}
+
+int permute_launch(hipStream_t st, const int32_t *ids, int T, int K, int E, int tile_m, int32_t *sorted_slot,
+                   int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &ws) {
+  const int TK = T * K;
+  if (TK <= kChunk) {
+    permute_small_kernel<<<1, 64, 0, st>>>(ids, TK, E, tile_m, ws.max_tiles, sorted_slot, expert_offsets, slot_to_row,
+                                           ws.tile_prefix, ws.tile_expert);
+    return (int)hipGetLastError();
+  }
+  permute_count_kernel<<<ws.n_chunks, 64, 0, st>>>(ids, TK, E, ws.chunk_counts);
+  permute_scan_kernel<<<1, 1024, 0, st>>>(ws.chunk_counts, ws.n_chunks, E, tile_m, ws.max_tiles, expert_offsets,
+                                          ws.tile_prefix, ws.tile_expert);
+  permute_scatter_kernel<<<ws.n_chunks, 64, 0, st>>>(ids, TK, E, ws.chunk_counts, expert_offsets, sorted_slot,
+                                                     slot_to_row);
+  return (int)hipGetLastError();
+}
+
+}  // namespace moe
+
+extern "C" size_t moe_permute_workspace_bytes(int T, int K, int E) {
+  if (T < 0 || K < 1 || E < 1) return 0;
+  return moe::permute_ws_bytes(T, K, E);
+}
+
+extern "C" int moe_tile_rows(int T, int K, int E) { return moe::choose_tile_m(T, K, E); }
+
+extern "C" int moe_permute(void *stream, const int32_t *ids, int T, int K, int E, int32_t *sorted_slot,
+                           int32_t *expert_offsets, int32_t *slot_to_row, void *workspace, size_t workspace_bytes) {
+  using namespace moe;
+  if (!ids || !sorted_slot || !expert_offsets || !slot_to_row || !workspace) return MOE_E_NULL;
+  if (T < 0 || K < 1 || K > MOE_MAX_TOPK || E < 1 || E > MOE_MAX_EXPERTS) return MOE_E_SHAPE;
+  if ((long)T * K > (1l << 30)) return MOE_E_SHAPE;
+  if (workspace_bytes < permute_ws_bytes(T, K, E)) return MOE_E_WORKSPACE;
+  if ((uintptr_t)workspace % 4) return MOE_E_ALIGN;
+  PermuteWs ws = permute_ws_layout(workspace, T, K, E);
+  return permute_launch((hipStream_t)stream, ids, T, K, E, choose_tile_m(T, K, E), sorted_slot, expert_offsets,
+                        slot_to_row, ws);
+}

@@ -1,0 +1,108 @@
+// The two bandwidth-bound elementwise stages around the grouped GEMMs:
+//   act_quant        bf16 [R, C] -> e4m3fn [R, C] + fp32 scale per row per 128 columns
+//   weighted_reduce  bf16 [T, K, H] per-slot results -> bf16 [T, H], fp32 weighted sum
+// Both move 16 bytes per lane per access; rows are contiguous so every access is coalesced.
+#include "moe_common.h"
+#include "../../include/moe_hip.h"
+
+namespace moe {
+
+// 16 lanes share one 128-column group: 8 bf16 per lane.
+__global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t *__restrict__ x, size_t n_groups,
+                                                        uint8_t *__restrict__ q, float *__restrict__ s) {
+  const size_t g = ((size_t)blockIdx.x * 256 + threadIdx.x) >> 4;
+  const int sub = threadIdx.x & 15;
+  const bool live = g < n_groups;
+  float f[8];
+  float amax = 0.f;
+  if (live) {
+    v4i raw = *(const v4i *)(x + g * kBlock + sub * 8);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      uint32_t w = (uint32_t)raw[i];
+      f[2 * i] = bf16_to_f32((uint16_t)(w & 0xffff));
+      f[2 * i + 1] = bf16_to_f32((uint16_t)(w >> 16));
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(f[i]));
+  }
+  amax = max_over_row16(amax);
+  if (!live) return;
+  const float sc = group_scale(amax);
+  v2i out;
+  out[0] = (int)pack4_fp8(f[0] / sc, f[1] / sc, f[2] / sc, f[3] / sc);
+  out[1] = (int)pack4_fp8(f[4] / sc, f[5] / sc, f[6] / sc, f[7] / sc);
+  *(v2i *)(q + g * kBlock + sub * 8) = out;
+  if (sub == 0) s[g] = sc;
+}
+
+// One lane produces 8 consecutive columns of one token.
+__global__ __launch_bounds__(256) void weighted_reduce_kernel(const uint16_t *__restrict__ y,
+                                                              const float *__restrict__ w,
+                                                              const uint16_t *__restrict__ shared_y, int T, int K,
+                                                              int H, uint16_t *__restrict__ out) {
+  const int hv = H >> 3;   // 16-byte vectors per row
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (size_t)T * hv) return;
+  const int t = (int)(idx / hv), c = (int)(idx % hv) * 8;
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) acc[i] = 0.f;
+  for (int k = 0; k < K; k++) {
+    const float wk = w[(size_t)t * K + k];
+    v4i raw = *(const v4i *)(y + ((size_t)t * K + k) * H + c);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      uint32_t u = (uint32_t)raw[i];
+      acc[2 * i] += wk * bf16_to_f32((uint16_t)(u & 0xffff));
+      acc[2 * i + 1] += wk * bf16_to_f32((uint16_t)(u >> 16));
+    }
+  }
+  if (shared_y != nullptr) {
+    v4i raw = *(const v4i *)(shared_y + (size_t)t * H + c);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      uint32_t u = (uint32_t)raw[i];
+      acc[2 * i] += bf16_to_f32((uint16_t)(u & 0xffff));
+      acc[2 * i + 1] += bf16_to_f32((uint16_t)(u >> 16));
+    }
+  }
+  v4i o;
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+    o[i] = (int)((uint32_t)f32_to_bf16(acc[2 * i]) | ((uint32_t)f32_to_bf16(acc[2 * i + 1]) << 16));
+  *(v4i *)(out + (size_t)t * H + c) = o;
+}
+
+}  // namespace moe
+
+extern "C" int moe_act_quant(void *stream, const void *x_bf16, int R, int C, uint8_t *q, float *s) {
+  using namespace moe;
+  if (!x_bf16 || !q || !s) return MOE_E_NULL;
+  if (R < 0 || C < 1) return MOE_E_SHAPE;
+  if (C % kBlock) return MOE_E_ALIGN;
+  if (((uintptr_t)x_bf16 % 16) || ((uintptr_t)q % 8) || ((uintptr_t)s % 4)) return MOE_E_ALIGN;
+  const size_t groups = (size_t)R * (C / kBlock);
+  if (groups == 0) return MOE_OK;
+  const size_t blocks = (groups * 16 + 255) / 256;
+  if (blocks > 0x7fffffffull) return MOE_E_SHAPE;
+  act_quant_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>((const uint16_t *)x_bf16, groups, q, s);
+  return (int)hipGetLastError();
+}
+
+extern "C" int moe_weighted_reduce(void *stream, const void *y_bf16, const float *routing_weights,
+                                   const void *shared_y_bf16, int T, int K, int H, void *out_bf16) {
+  using namespace moe;
+  if (!y_bf16 || !routing_weights || !out_bf16) return MOE_E_NULL;
+  if (T < 0 || K < 1 || H < 1) return MOE_E_SHAPE;
+  if (H % 8) return MOE_E_ALIGN;
+  if (((uintptr_t)y_bf16 % 16) || ((uintptr_t)out_bf16 % 16) || (shared_y_bf16 && ((uintptr_t)shared_y_bf16 % 16)))
+    return MOE_E_ALIGN;
+  const size_t n = (size_t)T * (H / 8);
+  if (n == 0) return MOE_OK;
+  const size_t blocks = (n + 255) / 256;
+  if (blocks > 0x7fffffffull) return MOE_E_SHAPE;
+  weighted_reduce_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>(
+      (const uint16_t *)y_bf16, routing_weights, (const uint16_t *)shared_y_bf16, T, K, H, (uint16_t *)out_bf16);
+  return (int)hipGetLastError();
+}

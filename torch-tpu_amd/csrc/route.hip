@@ -1,0 +1,268 @@
+// Router selection kernels: one 64-lane wavefront owns one token's row of scores.
+//
+// A row of E <= 1024 scores lives in registers, element e in lane e % 64, register e / 64
+// (coalesced loads).  Every arg-max is a butterfly over the wave on (value, index) pairs with
+// "greater value, then lower index" as the order, so equal scores resolve to the lower index
+// on every lane identically and the K picks come out in descending order.
+#include "moe_common.h"
+#include "../../include/moe_hip.h"
+
+namespace moe {
+
+
+struct Best {
+  float v;
+  int i;   // element index, or INT_MAX when the lane has no candidate
+};
+
+__device__ __forceinline__ bool better(float av, int ai, float bv, int bi) {
+  // candidates with i == INT_MAX lose to everything
+  if (bi == 0x7fffffff) return true;
+  if (ai == 0x7fffffff) return false;
+  return (av > bv) || (av == bv && ai < bi);
+}
+
+__device__ __forceinline__ Best wave_argmax(Best b) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    float ov = __shfl_xor(b.v, off, 64);
+    int oi = __shfl_xor(b.i, off, 64);
+    if (!better(b.v, b.i, ov, oi)) { b.v = ov; b.i = oi; }
+  }
+  return b;
+}
+
+__device__ __forceinline__ float round_to_bf16(float f) { return bf16_to_f32(f32_to_bf16(f)); }
+
+// Select top_k of one row.  v[j] holds element lane + 64*j (only j < per_lane are used,
+// elements >= E must be pre-marked dead).  dead bit j set = element is not a candidate.
+// Group limiting (n_groups > 1): group score = top1 + top2 of the group (fp32 add, rounded to
+// bf16 when round_bf16), keep the topk_groups best groups, the rest get value -inf but stay
+// candidates, exactly as a masked_fill(-inf) followed by top-k would leave them.
+template <int PER_LANE>
+__device__ __forceinline__ void select_row(float (&v)[PER_LANE], int E, int lane, int n_groups, int topk_groups,
+                                           int top_k, bool round_bf16, float &my_value, int &my_index) {
+  uint32_t dead = 0;
+#pragma unroll
+  for (int j = 0; j < PER_LANE; j++)
+    if (lane + 64 * j >= E) dead |= 1u << j;
+
+  if (n_groups > 1) {
+    const int per = E / n_groups;
+    float gscore = 0.f;          // lane g keeps the score of group g (n_groups <= 64)
+    for (int g = 0; g < n_groups; g++) {
+      const int lo = g * per, hi = lo + per;
+      float sum = 0.f;
+      int first = -1;
+      for (int pass = 0; pass < 2; pass++) {
+        Best b{0.f, 0x7fffffff};
+#pragma unroll
+        for (int j = 0; j < PER_LANE; j++) {
+          int e = lane + 64 * j;
+          if (e >= lo && e < hi && e != first && !(dead >> j & 1))
+            if (better(v[j], e, b.v, b.i)) { b.v = v[j]; b.i = e; }
+        }
+        b = wave_argmax(b);
+        if (b.i != 0x7fffffff) sum = (pass == 0) ? b.v : sum + b.v;
+        first = b.i;
+      }
+      if (round_bf16) sum = round_to_bf16(sum);
+      if (lane == g) gscore = sum;
+    }
+    uint64_t keep = 0;
+    bool taken = false;
+    for (int s = 0; s < topk_groups; s++) {
+      Best b{gscore, (lane < n_groups && !taken) ? lane : 0x7fffffff};
+      b = wave_argmax(b);
+      if (b.i == 0x7fffffff) break;
+      keep |= 1ull << b.i;
+      if (lane == b.i) taken = true;
+    }
+#pragma unroll
+    for (int j = 0; j < PER_LANE; j++) {
+      int e = lane + 64 * j;
+      if (e < E && !(keep >> (e / per) & 1)) v[j] = -INFINITY;
+    }
+  }
+
+  my_value = 0.f;
+  my_index = -1;
+  for (int s = 0; s < top_k; s++) {
+    Best b{0.f, 0x7fffffff};
+#pragma unroll
+    for (int j = 0; j < PER_LANE; j++) {
+      int e = lane + 64 * j;
+      if (!(dead >> j & 1))
+        if (better(v[j], e, b.v, b.i)) { b.v = v[j]; b.i = e; }
+    }
+    b = wave_argmax(b);
+    if (b.i == 0x7fffffff) break;           // fewer than top_k elements: cannot happen (K <= E)
+#pragma unroll
+    for (int j = 0; j < PER_LANE; j++)
+      if (lane + 64 * j == b.i) dead |= 1u << j;
+    if (lane == s) { my_value = b.v; my_index = b.i; }
+  }
+}
+
+template <int PER_LANE, bool BF16>
+__global__ __launch_bounds__(256) void noaux_tc_topk_kernel(const void *__restrict__ scores, int T, int E, int n_groups,
+                                                             int topk_groups, int top_k, void *__restrict__ values_out,
+                                                             int32_t *__restrict__ indices_out) {
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (t >= T) return;
+  float v[PER_LANE];
+#pragma unroll
+  for (int j = 0; j < PER_LANE; j++) {
+    int e = lane + 64 * j;
+    float x = -INFINITY;
+    if (e < E) {
+      if (BF16) x = bf16_to_f32(((const uint16_t *)scores)[(size_t)t * E + e]);
+      else x = ((const float *)scores)[(size_t)t * E + e];
+    }
+    v[j] = x;
+  }
+  float val;
+  int idx;
+  select_row<PER_LANE>(v, E, lane, n_groups, topk_groups, top_k, BF16, val, idx);
+  if (lane < top_k) {
+    if (BF16) ((uint16_t *)values_out)[(size_t)t * top_k + lane] = f32_to_bf16(val);
+    else ((float *)values_out)[(size_t)t * top_k + lane] = val;
+    indices_out[(size_t)t * top_k + lane] = idx;
+  }
+}
+
+template <int PER_LANE>
+__global__ __launch_bounds__(256) void route_topk_kernel(const void *__restrict__ logits, int logits_bf16,
+                                                          const float *__restrict__ bias, int T, int E, int K, int mode,
+                                                          int n_groups, int topk_groups, int renorm, float scale,
+                                                          float *__restrict__ weights_out, int32_t *__restrict__ ids_out,
+                                                          float *__restrict__ scores_out) {
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (t >= T) return;
+  float raw[PER_LANE];   // score used for the weight (before the bias)
+  float v[PER_LANE];     // score used for the selection
+  float row_max = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < PER_LANE; j++) {
+    int e = lane + 64 * j;
+    float x = -INFINITY;
+    if (e < E) {
+      if (logits_bf16) x = bf16_to_f32(((const uint16_t *)logits)[(size_t)t * E + e]);
+      else x = ((const float *)logits)[(size_t)t * E + e];
+    }
+    if (mode == MOE_ROUTE_SIGMOID && e < E) x = 1.0f / (1.0f + expf(-x));
+    raw[j] = x;
+    row_max = fmaxf(row_max, x);
+    v[j] = (bias != nullptr && e < E) ? x + bias[e] : x;
+    if (scores_out != nullptr && e < E && mode != MOE_ROUTE_SOFTMAX) scores_out[(size_t)t * E + e] = x;
+  }
+  float denom_all = 0.f;
+  if (mode == MOE_ROUTE_SOFTMAX) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) row_max = fmaxf(row_max, __shfl_xor(row_max, off, 64));
+#pragma unroll
+    for (int j = 0; j < PER_LANE; j++) {
+      int e = lane + 64 * j;
+      float p = (e < E) ? expf(raw[j] - row_max) : 0.f;
+      raw[j] = p;     // un-normalised softmax numerator becomes the weight source
+      denom_all += p;
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) denom_all += __shfl_xor(denom_all, off, 64);
+    if (scores_out != nullptr) {
+#pragma unroll
+      for (int j = 0; j < PER_LANE; j++) {
+        int e = lane + 64 * j;
+        if (e < E) scores_out[(size_t)t * E + e] = raw[j] / denom_all;
+      }
+    }
+  }
+  float val;
+  int idx;
+  select_row<PER_LANE>(v, E, lane, n_groups, topk_groups, K, false, val, idx);
+  // weight of pick `lane`: fetch the un-biased score of element idx from its owner lane
+  float w = 0.f;
+#pragma unroll
+  for (int j = 0; j < PER_LANE; j++) {
+    // element idx lives in lane idx % 64, register idx / 64
+    float cand = __shfl(raw[j], idx >= 0 ? (idx & 63) : 0, 64);
+    if (idx >= 0 && (idx >> 6) == j) w = cand;
+  }
+  if (mode == MOE_ROUTE_SOFTMAX && !renorm) w = w / denom_all;
+  if (renorm) {
+    float s = (lane < K) ? w : 0.f;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) s += __shfl_xor(s, off, 64);
+    w = w / s;
+  }
+  if (lane < K) {
+    weights_out[(size_t)t * K + lane] = w * scale;
+    ids_out[(size_t)t * K + lane] = idx;
+  }
+}
+
+template <int PER_LANE>
+static int launch_noaux(hipStream_t st, const void *scores, int dtype, int T, int E, int n_groups, int topk_groups,
+                        int top_k, void *values, int32_t *indices) {
+  dim3 grid((T + 3) / 4), block(256);
+  if (dtype == MOE_DTYPE_BF16)
+    noaux_tc_topk_kernel<PER_LANE, true><<<grid, block, 0, st>>>(scores, T, E, n_groups, topk_groups, top_k, values, indices);
+  else
+    noaux_tc_topk_kernel<PER_LANE, false><<<grid, block, 0, st>>>(scores, T, E, n_groups, topk_groups, top_k, values, indices);
+  return (int)hipGetLastError();
+}
+
+static int check_route_shape(int T, int E, int K, int n_groups, int topk_groups) {
+  if (T < 0 || E < 1 || E > MOE_MAX_EXPERTS || K < 1 || K > E || K > MOE_MAX_TOPK) return MOE_E_SHAPE;
+  if (n_groups > 1) {
+    if (n_groups > 64 || E % n_groups != 0 || topk_groups < 1 || topk_groups > n_groups) return MOE_E_SHAPE;
+    if (E / n_groups < 2) return MOE_E_SHAPE;
+    if ((long)topk_groups * (E / n_groups) < K) return MOE_E_SHAPE;
+  }
+  return MOE_OK;
+}
+
+}  // namespace moe
+
+extern "C" int moe_noaux_tc_topk(void *stream, const void *scores, int scores_dtype, int T, int E, int n_groups,
+                                 int topk_groups, int top_k, void *values_out, int32_t *indices_out) {
+  using namespace moe;
+  if (!scores || !values_out || !indices_out) return MOE_E_NULL;
+  if (scores_dtype != MOE_DTYPE_F32 && scores_dtype != MOE_DTYPE_BF16) return MOE_E_MODE;
+  int rc = check_route_shape(T, E, top_k, n_groups, topk_groups);
+  if (rc) return rc;
+  if (T == 0) return MOE_OK;
+  hipStream_t st = (hipStream_t)stream;
+  if (E <= 64) return launch_noaux<1>(st, scores, scores_dtype, T, E, n_groups, topk_groups, top_k, values_out, indices_out);
+  if (E <= 128) return launch_noaux<2>(st, scores, scores_dtype, T, E, n_groups, topk_groups, top_k, values_out, indices_out);
+  if (E <= 256) return launch_noaux<4>(st, scores, scores_dtype, T, E, n_groups, topk_groups, top_k, values_out, indices_out);
+  if (E <= 512) return launch_noaux<8>(st, scores, scores_dtype, T, E, n_groups, topk_groups, top_k, values_out, indices_out);
+  return launch_noaux<16>(st, scores, scores_dtype, T, E, n_groups, topk_groups, top_k, values_out, indices_out);
+}
+
+extern "C" int moe_route_topk(void *stream, const void *logits, int logits_dtype, const float *bias, int T, int E,
+                              int K, int mode, int n_groups, int topk_groups, int renorm, float scale,
+                              float *weights_out, int32_t *ids_out, float *scores_out) {
+  using namespace moe;
+  if (!logits || !weights_out || !ids_out) return MOE_E_NULL;
+  if (logits_dtype != MOE_DTYPE_F32 && logits_dtype != MOE_DTYPE_BF16) return MOE_E_MODE;
+  if (mode != MOE_ROUTE_SOFTMAX && mode != MOE_ROUTE_SIGMOID && mode != MOE_ROUTE_SCORES) return MOE_E_MODE;
+  int rc = check_route_shape(T, E, K, n_groups, topk_groups);
+  if (rc) return rc;
+  if (T == 0) return MOE_OK;
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((T + 3) / 4), block(256);
+  const int bf = logits_dtype == MOE_DTYPE_BF16;
+#define MOE_LAUNCH_ROUTE(P)                                                                                          \
+  route_topk_kernel<P><<<grid, block, 0, st>>>(logits, bf, bias, T, E, K, mode, n_groups, topk_groups, renorm, scale, \
+                                               weights_out, ids_out, scores_out)
+  if (E <= 64) MOE_LAUNCH_ROUTE(1);
+  else if (E <= 128) MOE_LAUNCH_ROUTE(2);
+  else if (E <= 256) MOE_LAUNCH_ROUTE(4);
+  else if (E <= 512) MOE_LAUNCH_ROUTE(8);
+  else MOE_LAUNCH_ROUTE(16);
+#undef MOE_LAUNCH_ROUTE
+  return (int)hipGetLastError();
+}

@@ -1,0 +1,63 @@
+"""Weight packing and a module-shaped wrapper around the fused-MoE path.
+
+The reference passes three separate weight tensors per call: gate [E,I,H], up [E,I,H] and a
+PRE-TRANSPOSED down [E,I,H], with bf16 block scales of matching orientation
+(python/regression/test_llm/test_moe.py:285-288).  The kernels here want the reduction
+dimension contiguous for both GEMMs, so weights are packed once, at load time:
+W13 = gate rows followed by up rows [E,2I,H], W2 = down in its checkpoint orientation
+[E,H,I], scales widened to fp32.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import ops
+
+
+def pack_expert_weights(gate, up, down_t, gate_scale, up_scale, down_t_scale):
+    """Reference-layout fp8 weights -> (w13, w13_scale, w2, w2_scale) in kernel layout.
+    Pure data movement (concatenate / transpose / widen); values are untouched."""
+    w13 = torch.cat([gate, up], dim=1).contiguous()
+    w13_scale = torch.cat([gate_scale, up_scale], dim=1).to(torch.float32).contiguous()
+    w2 = down_t.transpose(1, 2).contiguous()
+    w2_scale = down_t_scale.transpose(1, 2).to(torch.float32).contiguous()
+    return w13, w13_scale, w2, w2_scale
+
+
+class FusedMoE:
+    """Router + routed experts (+ shared expert) of one MoE layer, inference only.
+
+    Mirrors how the reference's tests wrap the op in a module holding the weights
+    (python/regression/test_llm/test_moe.py:143-160), with the routing recipe of its callers
+    (python/regression/test_llm/test_torch_ops.py:441-456) in front.
+    """
+
+    def __init__(self, router_weight, w13, w13_scale, w2, w2_scale, top_k, mode="softmax", bias=None,
+                 n_groups=1, topk_groups=1, renorm=True, scale=1.0, shared=None):
+        self.router_weight = router_weight          # [E, H] bf16
+        self.w13, self.w13_scale, self.w2, self.w2_scale = w13, w13_scale, w2, w2_scale
+        self.top_k, self.mode, self.bias = top_k, mode, bias
+        self.n_groups, self.topk_groups, self.renorm, self.scale = n_groups, topk_groups, renorm, scale
+        self.shared = shared
+        self._ws = None
+
+    def _workspace(self, T):
+        E, I2, H = self.w13.shape
+        I_sh = self.shared[0].shape[1] // 2 if self.shared is not None else 0
+        need = ops.fused_experts_workspace_bytes(T, H, I2 // 2, E, self.top_k, I_sh)
+        if self._ws is None or self._ws.numel() < need:
+            self._ws = torch.empty(need, dtype=torch.uint8, device=self.w13.device)
+        return self._ws
+
+    def route(self, x):
+        logits = torch.matmul(x, self.router_weight.t()).float()
+        return ops.moe_route(logits, self.top_k, self.mode, self.bias, self.n_groups, self.topk_groups,
+                             self.renorm, self.scale)
+
+    def experts(self, x, weights, ids, out=None):
+        return ops.fused_experts_fp8(x, self.w13, self.w13_scale, self.w2, self.w2_scale, ids, weights, out=out,
+                                     shared=self.shared, workspace=self._workspace(x.shape[0]))
+
+    def __call__(self, x, out=None):
+        weights, ids = self.route(x)
+        return self.experts(x, weights, ids, out)

@@ -1,0 +1,99 @@
+"""Registers the reference's operator names in the `my_ops` namespace, so that callers written
+against torch-tpu (`torch.ops.my_ops.fused_moe_fused_experts(...)`, positional arguments, caller
+allocated outputs) run unchanged on a ROCm device.
+
+Schemas follow the reference's C++ declarations (torch_tpu/csrc/ops/my_ops/ops.hpp:610-676,
+716-722; registered at myOps.cpp:73-77).
+"""
+from __future__ import annotations
+
+import torch
+
+from . import ops
+from .layer import pack_expert_weights
+
+_lib = torch.library.Library("my_ops", "DEF")
+
+_EXPERTS_HEAD = ("Tensor(a!) output, Tensor input, Tensor? output_sample, Tensor? input_sample, "
+                 "Tensor gate_weights, Tensor up_weights, Tensor down_weights, "
+                 "Tensor? gate_scales, Tensor? up_scales, Tensor? down_scales, "
+                 "Tensor select_experts, Tensor routing_weights, Tensor? num_select_experts, "
+                 "Tensor? select_experts_middle, Tensor? routing_weights_middle, ")
+_EXPERTS_TAIL = ("int blocksize, int num_experts, int num_experts_per_tok, bool use_grouped_topk, "
+                 "int num_expert_group, int topk_group, Tensor? silu, Tensor? sigmoid, Tensor? m0, "
+                 "bool save_mid_res) -> Tensor(a!)")
+
+_lib.define("fused_moe_fused_experts(" + _EXPERTS_HEAD + _EXPERTS_TAIL)
+_lib.define("fused_moe_fused_experts_v2(" + _EXPERTS_HEAD + "Tensor? gather_buffer, Tensor? scatter_buffer, "
+            + _EXPERTS_TAIL)
+_lib.define("noaux_tc_topk(Tensor(a!) values, Tensor(b!) indices, Tensor scores, int n_groups, int topk_groups, "
+            "int top_k) -> Tensor(a!)")
+_lib.define("fused_moe_grouped_topk(Tensor topk_experts_res, Tensor topk_weights_res_bf16, Tensor left_bf16, "
+            "Tensor right_bf16, Tensor topk_weights_res, Tensor left, Tensor right, Tensor max, Tensor matmul_res, "
+            "Tensor softmax_res) -> Tensor")
+
+# packed copies of reference-layout weights, keyed by the identity of the six tensors
+_pack_cache: dict = {}
+
+
+def _packed(gate, up, down, gs, us, ds):
+    key = tuple((t.data_ptr(), t._version, tuple(t.shape)) for t in (gate, up, down, gs, us, ds))
+    hit = _pack_cache.get(key)
+    if hit is None:
+        if len(_pack_cache) > 8:
+            _pack_cache.clear()
+        hit = pack_expert_weights(gate, up, down, gs, us, ds)
+        _pack_cache[key] = hit
+    return hit
+
+
+def _fused_experts(output, input, output_sample, input_sample, gate_weights, up_weights, down_weights,
+                   gate_scales, up_scales, down_scales, select_experts, routing_weights, num_select_experts,
+                   select_experts_middle, routing_weights_middle, blocksize, num_experts, num_experts_per_tok,
+                   use_grouped_topk, num_expert_group, topk_group, silu, sigmoid, m0, save_mid_res):
+    if select_experts.dtype != torch.int32:
+        raise RuntimeError("select_experts must be int32 dtype")
+    if num_select_experts is not None and num_select_experts.dtype != torch.int64:
+        raise RuntimeError("num_select_experts must be int64 dtype")
+    for name, t in (("output_sample", output_sample), ("input_sample", input_sample),
+                    ("num_select_experts", num_select_experts), ("silu", silu), ("sigmoid", sigmoid), ("m0", m0)):
+        if t is not None:
+            raise RuntimeError(f"{name}: the reference never passes this argument and leaves its meaning "
+                               "undefined; it is not supported")
+    if save_mid_res:
+        raise RuntimeError("save_mid_res is not supported")
+    if gate_scales is None or up_scales is None or down_scales is None:
+        raise RuntimeError("bf16 (un-quantised) expert weights are not supported: pass fp8 weights with block scales")
+    if blocksize != 128:
+        raise RuntimeError("blocksize must be 128")
+    w13, w13s, w2, w2s = _packed(gate_weights, up_weights, down_weights, gate_scales, up_scales, down_scales)
+    if w13.shape[0] != num_experts or select_experts.shape[1] != num_experts_per_tok:
+        raise RuntimeError("num_experts / num_experts_per_tok do not match the tensors")
+    rw = None
+    if output.dim() == 2:
+        rw = routing_weights.to(torch.float32)
+    ops.fused_experts_fp8(input, w13, w13s, w2, w2s, select_experts, rw, out=output)
+    return output
+
+
+def _fused_experts_v2(output, input, output_sample, input_sample, gate_weights, up_weights, down_weights,
+                      gate_scales, up_scales, down_scales, select_experts, routing_weights, num_select_experts,
+                      select_experts_middle, routing_weights_middle, gather_buffer, scatter_buffer, blocksize,
+                      num_experts, num_experts_per_tok, use_grouped_topk, num_expert_group, topk_group, silu, sigmoid,
+                      m0, save_mid_res):
+    # the scratch tensors of the reference's second implementation are accepted and left untouched
+    return _fused_experts(output, input, output_sample, input_sample, gate_weights, up_weights, down_weights,
+                          gate_scales, up_scales, down_scales, select_experts, routing_weights, num_select_experts,
+                          select_experts_middle, routing_weights_middle, blocksize, num_experts, num_experts_per_tok,
+                          use_grouped_topk, num_expert_group, topk_group, silu, sigmoid, m0, save_mid_res)
+
+
+def _grouped_topk(*args):
+    raise RuntimeError("fused_moe_grouped_topk: the reference's fused router is closed-source, untested and "
+                       "undocumented; use noaux_tc_topk or torch_tpu_amd.moe_route instead")
+
+
+_lib.impl("fused_moe_fused_experts", _fused_experts, "CompositeExplicitAutograd")
+_lib.impl("fused_moe_fused_experts_v2", _fused_experts_v2, "CompositeExplicitAutograd")
+_lib.impl("noaux_tc_topk", ops.noaux_tc_topk, "CompositeExplicitAutograd")
+_lib.impl("fused_moe_grouped_topk", _grouped_topk, "CompositeExplicitAutograd")

@@ -1,0 +1,225 @@
+"""Host side of the FP8 fused-MoE path: thin torch wrappers over the C ABI.
+
+Tensors live on a ROCm device ("cuda" in PyTorch-ROCm); torch is used for memory and the
+current stream only.  Every wrapper validates what the C side cannot see (dtype, device,
+contiguity), passes raw pointers and the current HIP stream, and raises RuntimeError on a
+non-zero return, as the reference's ops raise through TORCH_CHECK
+(torch_tpu/csrc/ops/my_ops/fusedMoE.cpp:143,148,231).
+"""
+from __future__ import annotations
+
+import torch
+
+from ._lib import MoeHipError, check, lib
+
+ROUTE_SOFTMAX, ROUTE_SIGMOID, ROUTE_SCORES = 0, 1, 2
+_FP8 = torch.float8_e4m3fn
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need(cond: bool, msg: str):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _dev(t: torch.Tensor, name: str, dtype=None):
+    _need(isinstance(t, torch.Tensor), f"{name} must be a tensor")
+    _need(t.is_cuda, f"{name} must be on the GPU")
+    _need(t.is_contiguous(), f"{name} must be contiguous")
+    if dtype is not None:
+        _need(t.dtype in (dtype if isinstance(dtype, tuple) else (dtype,)), f"{name} must be {dtype}, got {t.dtype}")
+    return t.data_ptr()
+
+
+def _dtype_sel(t: torch.Tensor, name: str) -> int:
+    _need(t.dtype in (torch.float32, torch.bfloat16), f"{name} must be float32 or bfloat16")
+    return 0 if t.dtype == torch.float32 else 1
+
+
+def tile_rows(T: int, K: int, E: int) -> int:
+    return lib.moe_tile_rows(T, K, E)
+
+
+# --------------------------------------------------------------------------- routing
+def noaux_tc_topk(values, indices, scores, n_groups: int, topk_groups: int, top_k: int):
+    """Group-limited top-k into caller-allocated `values` / `indices`; returns `values`
+    (signature of the reference op, torch_tpu/csrc/ops/my_ops/NoauxTcTopk.cpp:9-67)."""
+    _need(scores.dim() == 2, "scores must be 2D tensor")
+    _need(values.dtype == scores.dtype, "values and scores must have the same dtype")
+    _need(indices.dtype == torch.int32, "indices must be int32")
+    T, E = scores.shape
+    _need(tuple(values.shape) == (T, top_k), "values shape must be [batch_size, top_k]")
+    _need(tuple(indices.shape) == (T, top_k), "indices shape must be [batch_size, top_k]")
+    _need(n_groups > 0 and E % n_groups == 0, "total_size must be divisible by n_groups")
+    _need(topk_groups <= n_groups, "topk_groups must be <= n_groups")
+    _need(top_k > 0, "top_k must be positive")
+    sel = _dtype_sel(scores, "scores")
+    rc = lib.moe_noaux_tc_topk(_stream(), _dev(scores, "scores"), sel, T, E, n_groups, topk_groups, top_k,
+                               _dev(values, "values"), _dev(indices, "indices"))
+    check(rc, "noaux_tc_topk")
+    return values
+
+
+def moe_route(logits, k: int, mode: str = "softmax", bias=None, n_groups: int = 1, topk_groups: int = 1,
+              renorm: bool = True, scale: float = 1.0, return_scores: bool = False):
+    """Top-k routing from router logits -> (fp32 weights [T,k], int32 ids [T,k][, fp32 scores [T,E]]).
+    mode: "softmax" | "sigmoid" | "scores" (the input already holds scores)."""
+    modes = {"softmax": ROUTE_SOFTMAX, "sigmoid": ROUTE_SIGMOID, "scores": ROUTE_SCORES}
+    _need(mode in modes, f"unknown routing mode {mode!r}")
+    _need(logits.dim() == 2, "logits must be [T, E]")
+    T, E = logits.shape
+    sel = _dtype_sel(logits, "logits")
+    weights = torch.empty(T, k, dtype=torch.float32, device=logits.device)
+    ids = torch.empty(T, k, dtype=torch.int32, device=logits.device)
+    scores = torch.empty(T, E, dtype=torch.float32, device=logits.device) if return_scores else None
+    bias_ptr = None
+    if bias is not None:
+        _need(bias.numel() == E, "bias must hold one value per expert")
+        bias_ptr = _dev(bias, "bias", torch.float32)
+    rc = lib.moe_route_topk(_stream(), _dev(logits, "logits"), sel, bias_ptr, T, E, k, modes[mode], n_groups,
+                            topk_groups, int(renorm), float(scale), weights.data_ptr(), ids.data_ptr(),
+                            scores.data_ptr() if scores is not None else None)
+    check(rc, "moe_route")
+    return (weights, ids, scores) if return_scores else (weights, ids)
+
+
+# --------------------------------------------------------------------------- permutation
+def moe_permute(ids, num_experts: int, return_workspace: bool = False):
+    """Stable counting sort of the flattened ids -> (sorted_slot [T*K], expert_offsets [E+1],
+    slot_to_row [T*K]), all int32."""
+    _need(ids.dim() == 2, "ids must be [T, K]")
+    T, K = ids.shape
+    dev = ids.device
+    sorted_slot = torch.empty(T * K, dtype=torch.int32, device=dev)
+    offsets = torch.empty(num_experts + 1, dtype=torch.int32, device=dev)
+    slot_to_row = torch.empty(T * K, dtype=torch.int32, device=dev)
+    nbytes = lib.moe_permute_workspace_bytes(T, K, num_experts)
+    _need(nbytes > 0, "bad permutation shape")
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    rc = lib.moe_permute(_stream(), _dev(ids, "ids", torch.int32), T, K, num_experts, sorted_slot.data_ptr(),
+                         offsets.data_ptr(), slot_to_row.data_ptr(), ws.data_ptr(), nbytes)
+    check(rc, "moe_permute")
+    if return_workspace:
+        return sorted_slot, offsets, slot_to_row, ws
+    return sorted_slot, offsets, slot_to_row
+
+
+# --------------------------------------------------------------------------- quantisation
+def act_quant(x):
+    """bf16 [R, C] -> (e4m3fn [R, C], fp32 scales [R, C/128])."""
+    _need(x.dim() == 2, "x must be [R, C]")
+    R, C = x.shape
+    q = torch.empty(R, C, dtype=_FP8, device=x.device)
+    s = torch.empty(R, C // 128, dtype=torch.float32, device=x.device)
+    rc = lib.moe_act_quant(_stream(), _dev(x, "x", torch.bfloat16), R, C, q.data_ptr(), s.data_ptr())
+    check(rc, "act_quant")
+    return q, s
+
+
+# --------------------------------------------------------------------------- experts
+def fused_experts_workspace_bytes(T, H, I, E, K, I_shared=0) -> int:
+    return lib.moe_fused_experts_workspace_bytes(T, H, I, E, K, I_shared)
+
+
+def fused_experts_fp8(x, w13, w13_scale, w2, w2_scale, ids, routing_weights=None, out=None, shared=None,
+                      workspace=None):
+    """The expert computation on packed weights.
+
+    x [T,H] bf16; w13 [E,2I,H] e4m3fn + fp32 scales [E,2I/128,H/128]; w2 [E,H,I] e4m3fn + fp32
+    scales [E,H/128,I/128]; ids [T,K] int32.
+    out [T,K,H] bf16: un-weighted per-slot results.  out [T,H] bf16: weighted sum over the
+    slots (routing_weights fp32 [T,K] required), plus the shared expert
+    shared=(w13 [1,2Is,H], w13_scale, w2 [1,H,Is], w2_scale) if given.
+    Default out is [T,H] when routing_weights is given, else [T,K,H]."""
+    _need(x.dim() == 2 and w13.dim() == 3 and w2.dim() == 3 and ids.dim() == 2, "bad ranks")
+    T, H = x.shape
+    E, I2, H2 = w13.shape
+    I = I2 // 2
+    K = ids.shape[1]
+    _need(H2 == H and tuple(w2.shape) == (E, H, I), "weight shapes do not match x")
+    _need(ids.shape[0] == T, "ids must be [T, K]")
+    _need(H % 128 == 0 and I % 128 == 0, "H and I must be multiples of 128")
+    _need(tuple(w13_scale.shape) == (E, I2 // 128, H // 128), "w13_scale must be [E, 2I/128, H/128]")
+    _need(tuple(w2_scale.shape) == (E, H // 128, I // 128), "w2_scale must be [E, H/128, I/128]")
+    if out is None:
+        shape = (T, H) if routing_weights is not None else (T, K, H)
+        out = torch.empty(shape, dtype=torch.bfloat16, device=x.device)
+    mode = 1 if out.dim() == 2 else 0
+    _need(tuple(out.shape) == ((T, H) if mode else (T, K, H)), "out must be [T,H] or [T,K,H]")
+    rw_ptr = None
+    if routing_weights is not None:
+        _need(tuple(routing_weights.shape) == (T, K), "routing_weights must be [T, K]")
+        rw_ptr = _dev(routing_weights, "routing_weights", torch.float32)
+    _need(mode == 0 or rw_ptr is not None, "routing_weights are required for a [T,H] output")
+    sh = [None, None, None, None]
+    I_sh = 0
+    if shared is not None:
+        s13, s13s, s2, s2s = shared
+        I_sh = s13.shape[1] // 2
+        _need(tuple(s13.shape) == (1, 2 * I_sh, H) and tuple(s2.shape) == (1, H, I_sh), "bad shared expert shapes")
+        _need(tuple(s13s.shape) == (1, 2 * I_sh // 128, H // 128) and tuple(s2s.shape) == (1, H // 128, I_sh // 128),
+              "bad shared expert scale shapes")
+        sh = [_dev(s13, "shared w13", _FP8), _dev(s13s, "shared w13 scale", torch.float32),
+              _dev(s2, "shared w2", _FP8), _dev(s2s, "shared w2 scale", torch.float32)]
+    need = fused_experts_workspace_bytes(T, H, I, E, K, I_sh)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+    _need(workspace.numel() * workspace.element_size() >= need, "workspace too small")
+    rc = lib.moe_fused_experts_fp8(
+        _stream(), _dev(x, "x", torch.bfloat16), T, H,
+        _dev(w13, "w13", _FP8), _dev(w13_scale, "w13_scale", torch.float32),
+        _dev(w2, "w2", _FP8), _dev(w2_scale, "w2_scale", torch.float32), I, E,
+        _dev(ids, "ids", torch.int32), rw_ptr, K,
+        sh[0], sh[1], sh[2], sh[3], I_sh,
+        _dev(out, "out", torch.bfloat16), mode,
+        _dev(workspace, "workspace"), workspace.numel() * workspace.element_size())
+    check(rc, "fused_experts_fp8")
+    return out
+
+
+def gemm1_swiglu(xq, xs, w13, w13_scale, ids_shape, sorted_slot, offsets, permute_ws):
+    """Stage: first grouped GEMM + SwiGLU + re-quantisation -> (hq [T*K, I] e4m3fn, hs [T*K, I/128])."""
+    T, K = ids_shape
+    E, I2, H = w13.shape
+    I = I2 // 2
+    hq = torch.empty(T * K, I, dtype=_FP8, device=xq.device)
+    hs = torch.empty(T * K, I // 128, dtype=torch.float32, device=xq.device)
+    rc = lib.moe_gemm1_swiglu(_stream(), _dev(xq, "xq", _FP8), _dev(xs, "xs", torch.float32), T, H,
+                              _dev(w13, "w13", _FP8), _dev(w13_scale, "w13_scale", torch.float32), I, E, K,
+                              _dev(sorted_slot, "sorted_slot", torch.int32), _dev(offsets, "offsets", torch.int32),
+                              _dev(permute_ws, "permute_ws"), hq.data_ptr(), hs.data_ptr())
+    check(rc, "gemm1_swiglu")
+    return hq, hs
+
+
+def gemm2(hq, hs, w2, w2_scale, ids_shape, sorted_slot, offsets, permute_ws, y=None):
+    """Stage: second grouped GEMM -> y [T, K, H] bf16 (slot order)."""
+    T, K = ids_shape
+    E, H, I = w2.shape
+    if y is None:
+        y = torch.empty(T, K, H, dtype=torch.bfloat16, device=hq.device)
+    rc = lib.moe_gemm2(_stream(), _dev(hq, "hq", _FP8), _dev(hs, "hs", torch.float32), T, H,
+                       _dev(w2, "w2", _FP8), _dev(w2_scale, "w2_scale", torch.float32), I, E, K,
+                       _dev(sorted_slot, "sorted_slot", torch.int32), _dev(offsets, "offsets", torch.int32),
+                       _dev(permute_ws, "permute_ws"), _dev(y, "y", torch.bfloat16))
+    check(rc, "gemm2")
+    return y
+
+
+def weighted_reduce(y, routing_weights, shared_y=None, out=None):
+    T, K, H = y.shape
+    if out is None:
+        out = torch.empty(T, H, dtype=torch.bfloat16, device=y.device)
+    rc = lib.moe_weighted_reduce(_stream(), _dev(y, "y", torch.bfloat16),
+                                 _dev(routing_weights, "routing_weights", torch.float32),
+                                 _dev(shared_y, "shared_y", torch.bfloat16) if shared_y is not None else None,
+                                 T, K, H, _dev(out, "out", torch.bfloat16))
+    check(rc, "weighted_reduce")
+    return out
+
+
+__all__ = ["MoeHipError", "noaux_tc_topk", "moe_route", "moe_permute", "act_quant", "fused_experts_fp8",
+           "fused_experts_workspace_bytes", "gemm1_swiglu", "gemm2", "weighted_reduce", "tile_rows"]
