@@ -311,11 +311,18 @@ def experts_ref_bf16(x, select_experts, w0, w1, w2, s0, s1, s2, block=BLOCK):
 # --------------------------------------------------------------------------- #
 # W8A8 pipeline in fp32 on the same quantised operands
 # --------------------------------------------------------------------------- #
-def experts_w8a8_fp32(x, select_experts, w13q, w13s, w2q, w2s, block=BLOCK, return_mid=False):
+def experts_w8a8_fp32(x, select_experts, w13q, w13s, w2q, w2s, block=BLOCK, return_mid=False, mid=None):
     """x [T,H] bf16; w13q [E,2I,H] e4m3 (gate rows then up rows), w13s [E,2I/128,H/128]
     fp32; w2q [E,H,I], w2s [E,H/128,I/128].  Every product is taken between
     dequantised fp32 operands; the SwiGLU output is re-quantised per row per 128
-    columns before the second GEMM.  -> fp32 [T, K, H] un-weighted."""
+    columns before the second GEMM.  -> fp32 [T, K, H] un-weighted.
+
+    mid = (hq uint8 [T,K,I], hs fp32 [T,K,I/128]): use these re-quantised SwiGLU
+    outputs instead of computing them (second GEMM only).  The re-quantisation
+    rounds values that sit on a rounding boundary either way depending on the
+    last bits of the fp32 sum, so two correct implementations of the first GEMM
+    can differ by one e4m3 step in isolated elements; this hook lets a test check
+    the second GEMM on exactly the operands another implementation produced."""
     T, K = select_experts.shape
     H = x.shape[1]
     I = w2q.shape[2]
@@ -327,10 +334,14 @@ def experts_w8a8_fp32(x, select_experts, w13q, w13s, w2q, w2s, block=BLOCK, retu
     flat = select_experts.reshape(-1).to(torch.int64)
     for e in torch.unique(flat).tolist():
         slots = torch.nonzero(flat == e).squeeze(-1)
-        rows = xd[slots // K]
-        gu = rows @ dequant_block(w13q[e], w13s[e], block).T
-        h = F.silu(gu[:, :I]) * gu[:, I:]
-        hq, hs = act_quant_group128(h, block)
+        if mid is None:
+            rows = xd[slots // K]
+            gu = rows @ dequant_block(w13q[e], w13s[e], block).T
+            h = F.silu(gu[:, :I]) * gu[:, I:]
+            hq, hs = act_quant_group128(h, block)
+        else:
+            hq = mid[0].reshape(T * K, I)[slots].view(torch.float8_e4m3fn)
+            hs = mid[1].reshape(T * K, -1)[slots]
         out[slots] = act_dequant_group128(hq, hs, block) @ dequant_block(w2q[e], w2s[e], block).T
         if return_mid:
             hq_all[slots] = hq.view(torch.uint8)
@@ -339,6 +350,15 @@ def experts_w8a8_fp32(x, select_experts, w13q, w13s, w2q, w2s, block=BLOCK, retu
     if return_mid:
         return out, (xq, xs, hq_all.reshape(T, K, I), hs_all.reshape(T, K, -1))
     return out
+
+
+def e4m3_step(code_u8: torch.Tensor) -> torch.Tensor:
+    """Grid spacing of e4m3fn around each code (distance to the next larger magnitude)."""
+    mag = (code_u8 & 0x7F).to(torch.int64)
+    tab = torch.from_numpy(e4m3_decode_table()[:0x7F].copy())
+    up = tab[(mag + 1).clamp(max=0x7E)] - tab[mag.clamp(max=0x7E)]
+    down = tab[mag.clamp(max=0x7E)] - tab[(mag - 1).clamp(min=0)]
+    return torch.maximum(up, down)
 
 
 def weighted_reduce(per_slot: torch.Tensor, routing_weights: torch.Tensor) -> torch.Tensor:
