@@ -1,0 +1,296 @@
+#!/usr/bin/env python3
+"""Benchmark of the FP8 fused-MoE layer on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3_prefill] [--no-cpu] [--no-decode]
+
+A step = one pass of the path over one batch of synthetic tokens that already sit in HBM:
+router GEMM -> top-k routing -> permutation -> activation quantisation -> grouped FP8 GEMM
+(W13) + SwiGLU + re-quantisation -> grouped FP8 GEMM (W2) -> shared expert -> weighted reduce.
+Prints ONE JSON line.  `value` = algorithmic FP8-GEMM TFLOP/s of the whole step,
+`roofline` = the dominant kernel (first grouped GEMM) against the roof that binds it,
+`decode` = the same layer at T in {1, 8, 32} as weight-streaming GB/s,
+`cpu_baseline` = the CPU oracle timed on this host on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+import __graft_entry__ as entry  # noqa: E402
+
+PEAK_FP8_TFLOPS = 5000.0      # MI355X dense FP8 MFMA, TFLOP/s
+PEAK_HBM_GBS = 8000.0         # MI355X HBM3E, GB/s
+
+WORKLOADS = {
+    # BASELINE.json configs[2]: DeepSeek-V3-shaped prefill layer
+    "c3_prefill": dict(H=7168, I=2048, E=256, K=8, I_sh=2048, T=4096, route="sigmoid", n_groups=8, topk_groups=4,
+                       scale=2.5, desc="DeepSeek-V3-shaped FP8 MoE layer, T=4096, E=256+1 shared, top-8"),
+    # configs[1]: Mixtral-8x7B-shaped layer at its largest T
+    "c2_prefill": dict(H=4096, I=14336, E=8, K=2, I_sh=0, T=4096, route="softmax", n_groups=1, topk_groups=1,
+                       scale=1.0, desc="Mixtral-8x7B-shaped FP8 MoE layer, T=4096, E=8, top-2"),
+    # configs[4]: Qwen3-30B-A3B-shaped layer, Zipf(1.2) expert popularity, ~10% empty experts
+    "c5_skewed": dict(H=2048, I=768, E=128, K=8, I_sh=0, T=16384, route="softmax", n_groups=1, topk_groups=1,
+                      scale=1.0, zipf=1.2, empty=13, desc="Qwen3-30B-A3B-shaped FP8 MoE layer, T=16384, Zipf load"),
+    # configs[0]: toy
+    "c1_toy": dict(H=256, I=512, E=8, K=2, I_sh=0, T=16, route="softmax", n_groups=1, topk_groups=1, scale=1.0,
+                   desc="toy FP8 MoE layer, T=16"),
+}
+
+
+def make_weights(pkg, E, N, Kd, dev, seed):
+    """[E, N, Kd] ~ N(0, 0.02) bf16 -> e4m3fn + fp32 block scales, generated on the GPU in slices."""
+    g = torch.Generator(device=dev).manual_seed(seed)
+    q = torch.empty(E, N, Kd, dtype=torch.float8_e4m3fn, device=dev)
+    s = torch.empty(E, N // 128, Kd // 128, dtype=torch.float32, device=dev)
+    step = max(1, (1 << 28) // (N * Kd))
+    for e0 in range(0, E, step):
+        e1 = min(E, e0 + step)
+        w = (torch.randn(e1 - e0, N, Kd, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+        q[e0:e1], s[e0:e1] = pkg.quant_weight_block128(w)
+    return q, s
+
+
+def build_layer(pkg, cfg, dev):
+    H, I, E, K = cfg["H"], cfg["I"], cfg["E"], cfg["K"]
+    w13, w13s = make_weights(pkg, E, 2 * I, H, dev, 1)
+    w2, w2s = make_weights(pkg, E, H, I, dev, 2)
+    shared = None
+    if cfg["I_sh"]:
+        s13, s13s = make_weights(pkg, 1, 2 * cfg["I_sh"], H, dev, 3)
+        s2, s2s = make_weights(pkg, 1, H, cfg["I_sh"], dev, 4)
+        shared = (s13, s13s, s2, s2s)
+    g = torch.Generator(device=dev).manual_seed(5)
+    wr = (torch.randn(E, H, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    bias = None
+    if cfg.get("zipf"):
+        # popularity ~ rank^-s through a logit offset; a few experts are switched off entirely
+        rank = torch.randperm(E, generator=g, device=dev).float() + 1
+        bias = -cfg["zipf"] * torch.log(rank) * 2.0
+        bias[torch.randperm(E, generator=g, device=dev)[:cfg["empty"]]] = -1e9
+    elif cfg["route"] == "sigmoid":
+        bias = torch.zeros(E, device=dev)           # uniform correction bias
+    moe = pkg.FusedMoE(wr, w13, w13s, w2, w2s, top_k=K, mode=cfg["route"], bias=bias, n_groups=cfg["n_groups"],
+                       topk_groups=cfg["topk_groups"], renorm=True, scale=cfg["scale"], shared=shared)
+    return moe
+
+
+def gemm_flops(cfg, T):
+    return 6.0 * cfg["H"] * cfg["I"] * T * cfg["K"] + 6.0 * cfg["H"] * cfg["I_sh"] * T
+
+
+def expert_bytes(H, I):
+    """fp8 weights + fp32 block scales of one expert (W13 and W2)."""
+    return 3 * H * I + 4 * 3 * (H // 128) * (I // 128)
+
+
+def time_steps(fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def event_time(fn, iters, warmup=2):
+    """Average duration of `fn`'s launches on the current stream, by HIP events."""
+    for _ in range(warmup):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) / iters * 1e-3
+
+
+def bench_prefill(pkg, moe, cfg, dev, steps, warmup):
+    T, H, I, E, K = cfg["T"], cfg["H"], cfg["I"], cfg["E"], cfg["K"]
+    g = torch.Generator(device=dev).manual_seed(11)
+    x = torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16)
+    out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+
+    def step():
+        moe(x, out=out)
+
+    sec = time_steps(step, steps, warmup)
+
+    # the dominant kernel on its own: first grouped GEMM (+SwiGLU+requant) over the routed experts
+    w, ids = moe.route(x)
+    xq, xs = pkg.act_quant(x)
+    ss, off, s2r, ws = pkg.moe_permute(ids, E, return_workspace=True)
+    hq = torch.empty(T * K, I, dtype=torch.float8_e4m3fn, device=dev)
+    hs = torch.empty(T * K, I // 128, dtype=torch.float32, device=dev)
+    from torch_tpu_amd._lib import check, lib
+    st = torch.cuda.current_stream().cuda_stream
+
+    def gemm1():
+        check(lib.moe_gemm1_swiglu(st, xq.data_ptr(), xs.data_ptr(), T, H, moe.w13.data_ptr(), moe.w13_scale.data_ptr(),
+                                   I, E, K, ss.data_ptr(), off.data_ptr(), ws.data_ptr(), hq.data_ptr(), hs.data_ptr()),
+              "gemm1")
+
+    y = torch.empty(T, K, H, dtype=torch.bfloat16, device=dev)
+
+    def gemm2():
+        check(lib.moe_gemm2(st, hq.data_ptr(), hs.data_ptr(), T, H, moe.w2.data_ptr(), moe.w2_scale.data_ptr(),
+                            I, E, K, ss.data_ptr(), off.data_ptr(), ws.data_ptr(), y.data_ptr()), "gemm2")
+
+    k1 = event_time(gemm1, max(3, steps))
+    k2 = event_time(gemm2, max(3, steps))
+    touched = int((off[1:] > off[:-1]).sum().item())
+    # algorithmic traffic of one launch of the first GEMM: each touched expert's W13 (+scales) once,
+    # quantised activations once, re-quantised SwiGLU output once
+    b1 = touched * (2 * I * H + 4 * (2 * I // 128) * (H // 128)) + T * H + 4 * T * (H // 128) \
+        + T * K * I + 4 * T * K * (I // 128) + 4 * T * K
+    f1 = 4.0 * H * I * T * K
+    b2 = touched * (I * H + 4 * (I // 128) * (H // 128)) + T * K * I + 4 * T * K * (I // 128) + 2 * T * K * H
+    f2 = 2.0 * H * I * T * K
+    intensity = f1 / b1
+    bound = "mfma" if intensity > PEAK_FP8_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9) else "hbm"
+    if bound == "hbm":
+        roof = dict(bound="hbm", achieved=b1 / k1 / 1e9, peak=PEAK_HBM_GBS, unit="GB/s")
+    else:
+        roof = dict(bound="mfma", achieved=f1 / k1 / 1e12, peak=PEAK_FP8_TFLOPS, unit="TFLOP/s")
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"] = None
+    roof.update(kernel="grouped_gemm_kernel<gated> (W13 GEMM + SwiGLU + requant)", launch_ms=k1 * 1e3,
+                algorithmic_bytes=b1, algorithmic_flops=f1, flop_per_byte=intensity,
+                mfma_tflops=f1 / k1 / 1e12, mfma_frac=f1 / k1 / 1e12 / PEAK_FP8_TFLOPS,
+                hbm_gbs=b1 / k1 / 1e9, hbm_frac=b1 / k1 / 1e9 / PEAK_HBM_GBS,
+                second_gemm=dict(launch_ms=k2 * 1e3, mfma_tflops=f2 / k2 / 1e12, hbm_gbs=b2 / k2 / 1e9,
+                                 hbm_frac=b2 / k2 / 1e9 / PEAK_HBM_GBS),
+                experts_touched=touched)
+    return sec, roof, x
+
+
+def bench_decode(pkg, moe, cfg, dev, steps, warmup):
+    """The same layer at T in {1, 8, 32}: HBM-bound weight streaming.  A pool of different token
+    batches is cycled so that consecutive steps touch different experts (no cache residency)."""
+    H, I, E, K = cfg["H"], cfg["I"], cfg["E"], cfg["K"]
+    res = []
+    for T in (1, 8, 32):
+        g = torch.Generator(device=dev).manual_seed(100 + T)
+        pool = [torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16) for _ in range(16)]
+        out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+        touched = []
+        for x in pool:
+            _, ids = moe.route(x)
+            touched.append(int(torch.unique(ids).numel()))
+        n_sh = 1 if cfg["I_sh"] else 0
+        avg_bytes = sum((t * expert_bytes(H, I) + n_sh * expert_bytes(H, cfg["I_sh"] or I)) for t in touched) \
+            / len(touched) + 2 * T * H * 2 + T * K * 8
+        state = {"i": 0}
+
+        def step():
+            moe(pool[state["i"] % len(pool)], out=out)
+            state["i"] += 1
+
+        sec = time_steps(step, max(steps, 32), max(warmup, 16))
+        res.append(dict(T=T, ms_per_step=sec * 1e3, tokens_per_s=T / sec, hbm_gbs=avg_bytes / sec / 1e9,
+                        hbm_frac=avg_bytes / sec / 1e9 / PEAK_HBM_GBS, experts_touched_avg=sum(touched) / len(touched),
+                        algorithmic_bytes=avg_bytes, launch_mode="eager"))
+    return res
+
+
+def cpu_baseline(pkg, moe, cfg, x, sample_tokens):
+    """The CPU oracle (routing, per-expert dequantise + fp32 matmul, weighted reduce) timed on the
+    first `sample_tokens` tokens of the batch; the same pass doubles as a parity check of the
+    device at full layer size."""
+    orc = entry.load_oracle()
+    cores = os.cpu_count() or 1
+    threads = min(cores, 16)
+    torch.set_num_threads(threads)
+    n = sample_tokens
+    # device side of the comparison: scores the device routed on, its picks and its output
+    logits_dev = torch.matmul(x[:n], moe.router_weight.t()).float()
+    if cfg["route"] == "sigmoid":
+        w_dev, ids_dev, scores_dev = pkg.moe_route(logits_dev, cfg["K"], "sigmoid", moe.bias, cfg["n_groups"],
+                                                   cfg["topk_groups"], True, cfg["scale"], return_scores=True)
+    else:
+        lg = logits_dev if moe.bias is None else logits_dev + moe.bias
+        w_dev, ids_dev = pkg.moe_route(lg, cfg["K"], "softmax")
+        scores_dev = lg
+    out_dev = moe.experts(x[:n].contiguous(), w_dev, ids_dev)
+    torch.cuda.synchronize()
+    xs = x[:n].cpu()
+    wr = moe.router_weight.float().cpu()
+    bias = None if moe.bias is None else moe.bias.cpu()
+    layer = tuple(t.cpu() for t in (moe.w13, moe.w13_scale, moe.w2, moe.w2_scale))
+    shared = None if moe.shared is None else tuple(t.cpu() for t in moe.shared)
+    scores_host = scores_dev.cpu()
+    t0 = time.perf_counter()
+    logits = xs.float() @ wr.T
+    if cfg["route"] == "sigmoid":
+        orc.route_sigmoid_grouped(logits, bias, cfg["K"], cfg["n_groups"], cfg["topk_groups"], cfg["scale"])
+        w_ref, ids_ref = orc.select_sigmoid_grouped(scores_host, bias, cfg["K"], cfg["n_groups"], cfg["topk_groups"],
+                                                    cfg["scale"])
+    else:
+        orc.route_softmax_topk(logits if bias is None else logits + bias, cfg["K"])
+        w_ref, ids_ref = orc.route_softmax_topk(scores_host, cfg["K"])
+    ref = orc.moe_w8a8_fp32(xs, ids_ref, w_ref, *layer, shared=shared)
+    sec = time.perf_counter() - t0
+    got = out_dev.float().cpu()
+    parity = {"routing_ids_equal_given_device_scores": bool(torch.equal(ids_dev.cpu(), ids_ref)),
+              "routing_weights_max_abs_diff": (w_dev.cpu() - w_ref).abs().max().item(),
+              "outputs_outside_rtol2e-2_atol1e-2": ((got - ref).abs() > 1e-2 + 2e-2 * ref.abs()).float().mean().item(),
+              "cos_diff": orc.cal_diff(ref, got)[0], "tokens_checked": n}
+    base = dict(value=gemm_flops(cfg, n) / sec / 1e12, unit="TFLOP/s", cores=threads, kind="port",
+                sample=f"first {n} tokens of the same batch through the CPU oracle (routing twice, per-expert "
+                       f"dequantise + fp32 matmul, weighted reduce): {sec:.1f} s, {n / sec:.2f} tokens/s",
+                tokens_per_s=n / sec, host_cpus=cores)
+    return base, parity
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c3_prefill", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--cpu-sample", type=int, default=32)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures ONE GPU: the path is single-device by design (expert-parallel sharding is "
+              "described in DESIGN.md, not built); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a ROCm GPU", file=sys.stderr)
+        sys.exit(2)
+    pkg = entry.load_package()
+    dev = "cuda:0"
+    cfg = WORKLOADS[args.workload]
+    moe = build_layer(pkg, cfg, dev)
+    sec, roof, x = bench_prefill(pkg, moe, cfg, dev, args.steps, args.warmup)
+    T = cfg["T"]
+    flops = gemm_flops(cfg, T)
+    result = {
+        "metric": "FP8 fused-MoE layer TFLOP/s (% MFMA peak) + decode HBM GB/s (% peak), 1 GPU",
+        "value": flops / sec / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3",
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {cfg['desc']}", "T": T, "hidden": cfg["H"],
+                   "intermediate": cfg["I"], "experts": cfg["E"], "top_k": cfg["K"], "shared_intermediate": cfg["I_sh"]},
+        "tokens_per_s": T / sec, "mfma_frac_of_peak": flops / sec / 1e12 / PEAK_FP8_TFLOPS,
+        "roofline": roof,
+    }
+    if not args.no_decode and args.workload == "c3_prefill":
+        result["decode"] = bench_decode(pkg, moe, cfg, dev, args.steps, args.warmup)
+    if not args.no_cpu:
+        base, parity = cpu_baseline(pkg, moe, cfg, x, min(args.cpu_sample, T))
+        result["cpu_baseline"] = base
+        result["parity_on_sample"] = parity
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

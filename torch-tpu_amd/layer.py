@@ -24,6 +24,20 @@ def pack_expert_weights(gate, up, down_t, gate_scale, up_scale, down_t_scale):
     return w13, w13_scale, w2, w2_scale
 
 
+def quant_weight_block128(w: torch.Tensor):
+    """bf16/fp32 weights [..., N, K] (N, K multiples of 128) -> (e4m3fn codes, fp32 scale per
+    128x128 block), scale = max(amax, 1e-10) / 448, codes = clamp(w / scale, +-448) rounded to
+    nearest even.  Runs wherever `w` lives; meant for converting a checkpoint once."""
+    N, K = w.shape[-2:]
+    if N % 128 or K % 128:
+        raise RuntimeError("weight dimensions must be multiples of 128")
+    lead = w.shape[:-2]
+    blk = w.to(torch.float32).reshape(*lead, N // 128, 128, K // 128, 128)
+    scale = blk.abs().amax(dim=(-3, -1)).clamp_min(1e-10) / 448.0
+    q = (blk / scale[..., :, None, :, None]).clamp(-448.0, 448.0).to(torch.float8_e4m3fn)
+    return q.reshape(*lead, N, K), scale
+
+
 class FusedMoE:
     """Router + routed experts (+ shared expert) of one MoE layer, inference only.
 
@@ -51,7 +65,10 @@ class FusedMoE:
 
     def route(self, x):
         logits = torch.matmul(x, self.router_weight.t()).float()
-        return ops.moe_route(logits, self.top_k, self.mode, self.bias, self.n_groups, self.topk_groups,
+        bias = self.bias
+        if self.mode == "softmax" and bias is not None:
+            logits, bias = logits + bias, None          # a softmax router's bias is part of the logits
+        return ops.moe_route(logits, self.top_k, self.mode, bias, self.n_groups, self.topk_groups,
                              self.renorm, self.scale)
 
     def experts(self, x, weights, ids, out=None):
