@@ -26,11 +26,19 @@
 //   butterflies -> LDS across the four wavefronts), scale = max(amax, 1e-10) / 448, h / scale -> e4m3fn.
 // GATED = false (second GEMM): the strip is 256 output columns, wavefront w owns 64 of them;
 //   the bf16 result row is written at its slot (t*K + k), which undoes the permutation.
+#include <stdlib.h>
 #include "moe_common.h"
 #include "moe_layout.h"
 #include "../../include/moe_hip.h"
 
 namespace moe {
+
+// development knob: MOE_HIP_GEMM_VARIANT picks among the compiled launch shapes
+static int gemm_variant() {
+  static int v = -1;
+  if (v < 0) { const char *s = getenv("MOE_HIP_GEMM_VARIANT"); v = s ? atoi(s) : 0; }
+  return v;
+}
 
 struct GemmArgs {
   const uint8_t *aq;            // activations fp8 [rows_a, Kd]
@@ -56,14 +64,23 @@ struct GemmArgs {
   int max_mtiles;               // entries allocated in tile_expert
 };
 
-template <int MT>
+constexpr int kMaxKB = 256;                 // reduction length limit: 256 * 128 = 32768
+
+template <int MT, int NW, int STAGES, int WSTAGES>
 struct GemmSmem {
   static constexpr int BM = 16 * MT;
-  alignas(16) uint8_t tok[2][BM * 128];   // token tile, two stages, swizzled 16-byte chunks
-  float sa[2][BM];              // activation scales of the step
-  int arow[BM];                 // source row in aq / as for each tile row
-  float amax[4][BM];            // GATED epilogue: per-wavefront partial amax
+  static constexpr int SA = BM < 64 ? 64 : BM;   // the scale DMA always writes 64 lanes
+  alignas(1024) uint8_t wt[WSTAGES][16 * 2048];   // weight tiles: [tile][half][lane][16 bytes], read by their owner
+  alignas(1024) uint8_t tok[STAGES][BM * 128];   // token tiles, XOR-swizzled 16-byte chunks
+  alignas(256) float sa[STAGES][SA];             // activation scales of each staged step
+  int arow[BM];                                  // source row in aq / as for each tile row
+  float amax[NW][BM];                            // GATED epilogue: per-wavefront partial amax
+  float sb[2][kMaxKB];                           // weight-block scales of the strip for every 128-step
 };
+
+typedef __attribute__((address_space(3))) uint8_t lds_byte;
+// byte offset of a __shared__ object inside the workgroup's LDS allocation (what M0 wants)
+__device__ __forceinline__ uint32_t lds_offset(const void *p) { return (uint32_t)(uintptr_t)(lds_byte *)p; }
 
 __device__ __forceinline__ v8i load_w_frag(const uint8_t *p) {
   v4i lo = *(const v4i *)p;
@@ -81,12 +98,16 @@ __device__ __forceinline__ v8i concat8(v4i lo, v4i hi) {
   return r;
 }
 
-template <int MT, bool GATED>
-__global__ __launch_bounds__(256) void grouped_gemm_kernel(const GemmArgs a) {
+// MT     token m-tiles (of 16 rows) per workgroup
+// NW     wavefronts per workgroup (4 or 8); each owns WT = 16 / NW of the strip's 16 weight tiles
+// DEPTH  128-steps of weights kept in flight per wavefront (register ring)
+template <int MT, int NW, int DEPTH, bool GATED, bool WREG>
+__global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a) {
   constexpr int BM = 16 * MT;
-  constexpr int NCHUNK = BM * 8;                      // 16-byte chunks of one token-tile stage
-  constexpr int NLOAD = (NCHUNK + 255) / 256;         // chunks per thread
-  __shared__ GemmSmem<MT> sm;
+  constexpr int NT = 64 * NW;                         // threads
+  constexpr int WT = 16 / NW;                         // weight tiles per wavefront
+  constexpr int STAGES = DEPTH + 1;                   // token tiles staged in LDS
+  __shared__ GemmSmem<MT, NW, STAGES, WREG ? 1 : STAGES> sm;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -94,10 +115,16 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(const GemmArgs a) {
   const int li = lane & 15, lg = lane >> 4;
 
   // ---- which tile -------------------------------------------------------------------------
-  // Workgroup ids are dealt round-robin to the 8 XCDs; remap so that each XCD (own L2) gets a
-  // contiguous range of logical tiles: neighbours share the token tile.
-  const int per_xcd = a.total_blocks >> 3;
+  // Workgroup ids are dealt round-robin to the 8 XCDs (id % 8).  Remap so that each XCD, which
+  // has its own L2, works on a contiguous range of the real tiles (their number is only known
+  // on the device): neighbours in that range share the token tile and, for experts with more
+  // than one row tile, the weight strip.
+  const int n_mtiles = a.fixed_expert >= 0 ? (a.rows_a + BM - 1) / BM : min(a.tile_prefix[a.E], a.max_mtiles);
+  const int n_work = n_mtiles * a.n_strips;
+  const int per_xcd = (n_work + 7) >> 3;
+  if ((int)(blockIdx.x >> 3) >= per_xcd) return;
   const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (logical >= n_work) return;
   const int mtile = logical / a.n_strips;
   const int strip = logical - mtile * a.n_strips;
   int e, row0, rows;                                  // expert, first permuted row, rows in tile
@@ -106,15 +133,15 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(const GemmArgs a) {
     row0 = mtile * BM;
     rows = min(BM, a.rows_a - row0);
   } else {
-    if (mtile >= min(a.tile_prefix[a.E], a.max_mtiles)) return;
     e = a.tile_expert[mtile];
     if (e < 0 || e >= a.E) return;
     row0 = a.expert_offsets[e] + (mtile - a.tile_prefix[e]) * BM;
     rows = min(BM, a.expert_offsets[e + 1] - row0);
   }
   if (rows <= 0) return;
+  const int mt_live = (rows + 15) >> 4;               // m-tiles that hold at least one row
 
-  for (int i = tid; i < BM; i += 256) {
+  for (int i = tid; i < BM; i += NT) {
     const int p = row0 + min(i, rows - 1);
     int src = p;
     if (GATED && a.fixed_expert < 0) src = a.sorted_slot[p] / a.topk;
@@ -126,109 +153,243 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(const GemmArgs a) {
   const int n_wblk = a.n_rows_w >> 7;                 // weight-scale rows per expert
 
   // ---- per-lane source addresses ------------------------------------------------------------
-  const uint8_t *wptr[4];
+  // GATED: tiles 0..WT/2-1 are gate columns, WT/2..WT-1 the matching up columns.
+  const uint8_t *wptr[WT];
 #pragma unroll
-  for (int j = 0; j < 4; j++) {
+  for (int j = 0; j < WT; j++) {
     int wrow;
-    if (GATED) wrow = (j < 2 ? 0 : a.N) + strip * 128 + wave * 32 + (j & 1) * 16 + li;
-    else wrow = strip * 256 + wave * 64 + j * 16 + li;
+    if (GATED) wrow = (j < WT / 2 ? 0 : a.N) + strip * 128 + wave * (8 * WT) + (j % (WT / 2)) * 16 + li;
+    else wrow = strip * 256 + wave * (16 * WT) + j * 16 + li;
     wrow = min(wrow, a.n_rows_w - 1);
     wptr[j] = a.w + ((size_t)e * a.n_rows_w + wrow) * a.Kd + lg * 32;
   }
-  const float *sb0_ptr, *sb1_ptr;
-  if (GATED) {
-    sb0_ptr = a.ws + ((size_t)e * n_wblk + strip) * NKB;
-    sb1_ptr = a.ws + ((size_t)e * n_wblk + (a.N >> 7) + strip) * NKB;
-  } else {
-    const int nblk = min(strip * 2 + (wave >> 1), n_wblk - 1);
-    sb0_ptr = a.ws + ((size_t)e * n_wblk + nblk) * NKB;
-    sb1_ptr = sb0_ptr;
+  // The strip's weight-block scales for all steps go to LDS once (two rows: gate/up blocks for
+  // the gated GEMM, the strip's two 128-column blocks otherwise): uniform values re-read per
+  // step from LDS instead of through the vector-memory queue.
+  {
+    const int blk0 = GATED ? strip : min(strip * 2, n_wblk - 1);
+    const int blk1 = GATED ? (a.N >> 7) + strip : min(strip * 2 + 1, n_wblk - 1);
+    for (int i = tid; i < 2 * NKB; i += NT) {
+      const int r = i >= NKB, kb = i - r * NKB;
+      sm.sb[r][kb] = a.ws[((size_t)e * n_wblk + (r ? blk1 : blk0)) * NKB + kb];
+    }
   }
-  size_t tok_src[NLOAD];
-  int tok_dst[NLOAD];
+  const int sb_row0 = GATED ? 0 : (wave * WT) / 8;      // which of the two rows this wavefront's tiles use
+  const int sb_row1 = GATED ? 1 : sb_row0;
+  // Token tile -> LDS by direct loads: one instruction moves 64 x 16 bytes = 8 rows x 128 bytes to
+  // LDS bytes [M0 + 16*lane); the XOR swizzle is applied on the source side (lane l fetches the
+  // chunk that belongs at position l).  NTOK instructions per wavefront and step; wavefronts past
+  // the tile's end repeat its last eight rows (same bytes to the same place).
+  constexpr int NROW8 = BM / 8;                        // 1 KB row-groups in the tile
+  constexpr int NTOK = (NROW8 + NW - 1) / NW;
+  size_t tok_src[NTOK];
+  uint32_t tok_m0[NTOK];
 #pragma unroll
-  for (int u = 0; u < NLOAD; u++) {
-    const int q = min(tid + 256 * u, NCHUNK - 1);
-    const int row = q >> 3, c = q & 7;
+  for (int u = 0; u < NTOK; u++) {
+    const int t = min(wave * NTOK + u, NROW8 - 1);
+    const int row = 8 * t + (lane >> 3);
+    const int c = (lane & 7) ^ (lane >> 3);
     tok_src[u] = (size_t)sm.arow[row] * a.Kd + c * 16;
-    tok_dst[u] = row * 128 + ((c ^ (row & 7)) << 4);
+    tok_m0[u] = t * 1024;
   }
-  const size_t sa_src = (size_t)sm.arow[min(tid, BM - 1)] * NKB;
+  constexpr int NSA = (BM + 63) / 64;                  // 64-row groups of scales
+  const int sa_grp = wave % NSA;
+  const size_t sa_src = (size_t)sm.arow[min(sa_grp * 64 + lane, BM - 1)] * NKB;
+  const uint32_t wt_base = __builtin_amdgcn_readfirstlane(lds_offset(&sm.wt[0][0])) + wave * (WT * 2048);
+  constexpr uint32_t kWtStage = 16 * 2048;
+  const uint32_t tok_base = __builtin_amdgcn_readfirstlane(lds_offset(&sm.tok[0][0]));
+  const uint32_t sa_base = __builtin_amdgcn_readfirstlane(lds_offset(&sm.sa[0][0])) + sa_grp * 256;
+  constexpr uint32_t kTokStage = BM * 128, kSaStage = sizeof(float) * GemmSmem<MT, NW, STAGES, 1>::SA;
 
-  v4f acc[MT][4];
+  v4f acc[MT][WT];
 #pragma unroll
   for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-    for (int j = 0; j < 4; j++) acc[mt][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < WT; j++) acc[mt][j] = (v4f){0.f, 0.f, 0.f, 0.f};
 
-  v8i w0[4], w1[4];
-  v4i treg[NLOAD];
-  float sareg = 0.f, sbA0, sbA1, sbB0 = 0.f, sbB1 = 0.f;
+  // ---- operand pipelines ----------------------------------------------------------------------
+  // Both operands travel HBM/L2 -> LDS by direct loads (no registers held while in flight), DEPTH
+  // steps ahead, through STAGES = DEPTH + 1 LDS stages.  The loads are inline assembly waited for
+  // by hand: the memory counter retires loads in issue order and every wavefront issues the same
+  // sequence each step (token tile pieces, token scales, its own weight fragments), so "how many
+  // younger loads may still be in flight" is a compile-time constant.
+  //   weights: the wavefront's WT tiles, each as two 1 KB halves laid out [lane][16 bytes] - the
+  //            owner reads them back with two linear 128-bit LDS reads per tile;
+  //   tokens:  1 KB pieces = 8 rows x 128 bytes, swizzled on the source side.
+  constexpr int L_STEP = NTOK + 1 + 2 * WT;            // loads per wavefront and step
+  v4i wlo[WREG ? DEPTH : 1][WT], whi[WREG ? DEPTH : 1][WT];   // WREG: weight fragments ride in a register ring
+  auto request_weights_reg = [&](int kb, v4i(&lo)[WT], v4i(&hi)[WT]) {
+#pragma unroll
+    for (int j = 0; j < WT; j++) {
+      const uint8_t *ptr = wptr[j] + (size_t)kb * 128;
+      asm volatile("global_load_dwordx4 %0, %2, off\n\tglobal_load_dwordx4 %1, %2, off offset:16"
+                   : "=&v"(lo[j]), "=&v"(hi[j]) : "v"(ptr) : "memory");
+    }
+  };
+  auto arrived_weights = [&](v4i(&lo)[WT], v4i(&hi)[WT]) {
+#pragma unroll
+    for (int j = 0; j < WT; j++) asm volatile("" : "+v"(lo[j]), "+v"(hi[j]));
+  };
+  auto request = [&](int kb, int stage) {
+#pragma unroll
+    for (int u = 0; u < NTOK; u++) {
+      const uint8_t *ptr = a.aq + tok_src[u] + (size_t)kb * 128;
+      const uint32_t m0 = tok_base + stage * kTokStage + tok_m0[u];
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0), "v"(ptr) : "memory", "m0");
+    }
+    {
+      const float *ptr = a.as + sa_src + kb;
+      const uint32_t m0 = sa_base + stage * kSaStage;
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(m0), "v"(ptr) : "memory", "m0");
+    }
+    if (!WREG)
+#pragma unroll
+    for (int j = 0; j < WT; j++) {
+      const uint8_t *ptr = wptr[j] + (size_t)kb * 128;
+      const uint32_t m0 = wt_base + stage * kWtStage + j * 2048;
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\t"
+                   // the instruction offset moves the LDS address as well as the global one: 0x400 - 16
+                   "s_add_u32 m0, m0, 0x3f0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off offset:16"
+                   ::"s"(m0), "v"(ptr) : "memory", "m0", "scc");
+    }
+  };
 
-  auto issue_loads = [&](int kb, v8i(&wn)[4], float &s0, float &s1) {
+  // m-tiles are processed in groups of up to four; a group is skipped when it holds no row.  A
+  // group first issues all of its LDS reads (one exposed LDS latency per group, not per tile),
+  // then its matrix instructions back to back, each tile's scale multiply-adds trailing the
+  // matrix instruction that feeds them.
+  constexpr int MG = MT < 4 ? MT : 4;
+  auto compute = [&](int stage, int kb, const v4i(&lo)[WT], const v4i(&hi)[WT]) {
+    v8i wc[WT];
+    const uint8_t *wbase = sm.wt[WREG ? 0 : stage] + wave * (WT * 2048) + lane * 16;
 #pragma unroll
-    for (int j = 0; j < 4; j++) wn[j] = load_w_frag(wptr[j] + (size_t)kb * 128);
+    for (int j = 0; j < WT; j++) {
+      if (WREG) wc[j] = concat8(lo[j], hi[j]);
+      else wc[j] = concat8(*(const v4i *)(wbase + j * 2048), *(const v4i *)(wbase + j * 2048 + 1024));
+    }
+    const float s0 = sm.sb[sb_row0][kb], s1 = sm.sb[sb_row1][kb];
+    const uint8_t *tbase = sm.tok[stage] + li * 128;
+    const int o0 = ((2 * lg) ^ (li & 7)) << 4, o1 = ((2 * lg + 1) ^ (li & 7)) << 4;
+    const float *sap = sm.sa[stage] + li;
 #pragma unroll
-    for (int u = 0; u < NLOAD; u++) treg[u] = *(const v4i *)(a.aq + tok_src[u] + (size_t)kb * 128);
-    if (tid < BM) sareg = a.as[sa_src + kb];
-    s0 = sb0_ptr[kb];
-    s1 = sb1_ptr[kb];
-  };
-  auto stage_store = [&](int stage) {
+    for (int mg = 0; mg < MT / MG; mg++) {
+      if (mg == 0 || mg * MG < mt_live) {
+        v8i x[MG];
+        float sa_[MG];
 #pragma unroll
-    for (int u = 0; u < NLOAD; u++)
-      if (tid + 256 * u < NCHUNK) *(v4i *)(sm.tok[stage] + tok_dst[u]) = treg[u];
-    if (tid < BM) sm.sa[stage][tid] = sareg;
-  };
-  auto compute = [&](const v8i(&wc)[4], int stage, float s0, float s1) {
-    const int sw = li & 7;
+        for (int mi = 0; mi < MG; mi++) {
+          const int mt = mg * MG + mi;
+          x[mi] = concat8(*(const v4i *)(tbase + mt * 2048 + o0), *(const v4i *)(tbase + mt * 2048 + o1));
+          sa_[mi] = sap[mt * 16];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        v4f p[MG][WT];
 #pragma unroll
-    for (int mt = 0; mt < MT; mt++) {
-      const uint8_t *base = sm.tok[stage] + (mt * 16 + li) * 128;
-      const v4i x0 = *(const v4i *)(base + (((2 * lg) ^ sw) << 4));
-      const v4i x1 = *(const v4i *)(base + (((2 * lg + 1) ^ sw) << 4));
-      const v8i x = concat8(x0, x1);
-      const float s_a = sm.sa[stage][mt * 16 + li];
-      const float f0 = s_a * s0, f1 = s_a * s1;
+        for (int mi = 0; mi < MG; mi++) {
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const v4f zero = {0.f, 0.f, 0.f, 0.f};
-        const v4f p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wc[j], x, zero, 0, 0, 0, 0, 0, 0);
-        const float f = (GATED && j >= 2) ? f1 : f0;
+          for (int j = 0; j < WT; j++) {
+            const v4f zero = {0.f, 0.f, 0.f, 0.f};
+            p[mi][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wc[j], x[mi], zero, 0, 0, 0, 0, 0, 0);
+          }
+        }
 #pragma unroll
-        for (int r = 0; r < 4; r++) acc[mt][j][r] = fmaf(p[r], f, acc[mt][j][r]);
+        for (int mi = 0; mi < MG; mi++) {
+          const int mt = mg * MG + mi;
+          const float f0 = sa_[mi] * s0, f1 = sa_[mi] * s1;
+#pragma unroll
+          for (int j = 0; j < WT; j++) {
+            const float f = (GATED && j >= WT / 2) ? f1 : f0;
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[mt][j][r] = fmaf(p[mi][j][r], f, acc[mt][j][r]);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
   };
 
-  // ---- main loop: two 128-steps per trip so the weight registers ping-pong without copies -----
-  issue_loads(0, w0, sbA0, sbA1);
-  stage_store(0);
-  __syncthreads();
-  for (int kb = 0; kb < NKB; kb += 2) {
-    const bool more1 = kb + 1 < NKB;
-    if (more1) issue_loads(kb + 1, w1, sbB0, sbB1);
-    compute(w0, 0, sbA0, sbA1);
-    if (more1) stage_store(1);
-    __syncthreads();
-    if (!more1) break;
-    const bool more2 = kb + 2 < NKB;
-    if (more2) issue_loads(kb + 2, w0, sbA0, sbA1);
-    compute(w1, 1, sbB0, sbB1);
-    if (more2) stage_store(0);
-    __syncthreads();
+  // ---- main loop -----------------------------------------------------------------------------
+  // Step kb: wait until this wavefront's requests for step kb have landed | barrier: everybody's
+  // share of the token tile is there and everybody is done reading the stage that is reused next |
+  // request step kb+DEPTH into that stage | matrix work on stage kb % STAGES.
+  // DEPTH-1 whole steps stay in flight across the wait, DEPTH during the matrix work.
+  if (!WREG) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) request(min(d, NKB - 1), d);
+    int kb = 0, stage = 0, stage_req = DEPTH;
+    for (; kb + DEPTH < NKB; kb++) {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 1) * L_STEP) : "memory");
+      __syncthreads();
+      request(kb + DEPTH, stage_req);
+      compute(stage, kb, wlo[0], whi[0]);
+      stage = stage + 1 == STAGES ? 0 : stage + 1;
+      stage_req = stage_req + 1 == STAGES ? 0 : stage_req + 1;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    for (; kb < NKB; kb++) {
+      __syncthreads();
+      compute(stage, kb, wlo[0], whi[0]);
+      stage = stage + 1 == STAGES ? 0 : stage + 1;
+    }
+  } else {
+    // weights in a register ring (slot kb % DEPTH; loop unrolled by DEPTH so slots are compile-time):
+    // the token request of step kb+DEPTH goes out before the matrix work of step kb, the weight
+    // request after it, into the slot that work has just read
+    constexpr int L_TOKS = NTOK + 1;
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) {
+      request(min(d, NKB - 1), d);
+      request_weights_reg(min(d, NKB - 1), wlo[d], whi[d]);
+    }
+    int kb0 = 0;
+    for (; kb0 + 2 * DEPTH <= NKB; kb0 += DEPTH) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; d++) {
+        const int kb = kb0 + d;
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 1) * (L_TOKS + 2 * WT)) : "memory");
+        arrived_weights(wlo[d], whi[d]);
+        __syncthreads();
+        request(kb + DEPTH, (kb + DEPTH) % STAGES);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(kb % STAGES, kb, wlo[d], whi[d]);
+        __builtin_amdgcn_sched_barrier(0);
+        request_weights_reg(kb + DEPTH, wlo[d], whi[d]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) arrived_weights(wlo[d], whi[d]);
+    for (; kb0 < NKB; kb0 += DEPTH) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; d++) {
+        const int kb = kb0 + d;
+        if (kb < NKB) {
+          __syncthreads();
+          compute(kb % STAGES, kb, wlo[d], whi[d]);
+          if (kb + DEPTH < NKB) {
+            request(kb + DEPTH, (kb + DEPTH) % STAGES);
+            request_weights_reg(kb + DEPTH, wlo[d], whi[d]);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            arrived_weights(wlo[d], whi[d]);
+          }
+        }
+      }
+    }
   }
+  __syncthreads();
 
   // ---- epilogue -------------------------------------------------------------------------------
   if (GATED) {
+    constexpr int G = WT / 2;                          // gate tiles per wavefront
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
       float m = 0.f;
 #pragma unroll
-      for (int j = 0; j < 2; j++)
+      for (int j = 0; j < G; j++)
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-          const float g = acc[mt][j][r], u = acc[mt][j + 2][r];
+          const float g = acc[mt][j][r], u = acc[mt][j + G][r];
           const float h = (g / (1.0f + expf(-g))) * u;
           acc[mt][j][r] = h;
           m = fmaxf(m, fabsf(h));
@@ -242,13 +403,15 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(const GemmArgs a) {
     for (int mt = 0; mt < MT; mt++) {
       const int i = mt * 16 + li;
       const bool valid = i < rows;
-      const float am = fmaxf(fmaxf(sm.amax[0][i], sm.amax[1][i]), fmaxf(sm.amax[2][i], sm.amax[3][i]));
+      float am = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; w++) am = fmaxf(am, sm.amax[w][i]);
       const float sc = group_scale(am);
       const size_t orow = (size_t)(row0 + i);
 #pragma unroll
-      for (int j = 0; j < 2; j++) {
+      for (int j = 0; j < G; j++) {
         const uint32_t packed = pack4_fp8(acc[mt][j][0] / sc, acc[mt][j][1] / sc, acc[mt][j][2] / sc, acc[mt][j][3] / sc);
-        if (valid) *(uint32_t *)(a.hq + orow * a.N + strip * 128 + wave * 32 + j * 16 + lg * 4) = packed;
+        if (valid) *(uint32_t *)(a.hq + orow * a.N + strip * 128 + wave * (16 * G) + j * 16 + lg * 4) = packed;
       }
       if (valid && wave == 0 && lg == 0) a.hs[orow * n_grp + strip] = sc;
     }
@@ -260,8 +423,8 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(const GemmArgs a) {
       int slot = row0 + min(i, rows - 1);
       if (a.fixed_expert < 0) slot = a.sorted_slot[slot];
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const int col = strip * 256 + wave * 64 + j * 16 + lg * 4;
+      for (int j = 0; j < WT; j++) {
+        const int col = strip * 256 + wave * (16 * WT) + j * 16 + lg * 4;
         if (valid && col < a.N) {
           v2i o;
           o[0] = (int)((uint32_t)f32_to_bf16(acc[mt][j][0]) | ((uint32_t)f32_to_bf16(acc[mt][j][1]) << 16));
@@ -273,6 +436,8 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(const GemmArgs a) {
   }
 }
 
+// Launch shape per tile height.  Eight wavefronts (two per SIMD, two weight tiles each) keep
+// more loads in flight for the bandwidth-bound shapes.
 template <bool GATED>
 static int launch_gemm(hipStream_t st, GemmArgs &a, int tile_m, int max_mtiles) {
   a.n_strips = GATED ? a.N / 128 : (a.N + 255) / 256;
@@ -281,14 +446,21 @@ static int launch_gemm(hipStream_t st, GemmArgs &a, int tile_m, int max_mtiles) 
   total = (total + 7) / 8 * 8;
   if (total <= 0 || total > 0x7fffffffl) return MOE_E_SHAPE;
   a.total_blocks = (int)total;
-  dim3 grid((unsigned)total), block(256);
+  dim3 grid((unsigned)total);
+  const int cfg = gemm_variant();
+#define MOE_GEMM(MT, NW, D, WREG) grouped_gemm_kernel<MT, NW, D, GATED, WREG><<<grid, dim3(64 * NW), 0, st>>>(a)
   switch (tile_m) {
-    case 16: grouped_gemm_kernel<1, GATED><<<grid, block, 0, st>>>(a); break;
-    case 32: grouped_gemm_kernel<2, GATED><<<grid, block, 0, st>>>(a); break;
-    case 64: grouped_gemm_kernel<4, GATED><<<grid, block, 0, st>>>(a); break;
-    case 128: grouped_gemm_kernel<8, GATED><<<grid, block, 0, st>>>(a); break;
+    case 16: MOE_GEMM(1, 8, 3, false); break;
+    case 32: MOE_GEMM(2, 8, 3, false); break;
+    case 64: MOE_GEMM(4, 8, 2, false); break;
+    case 128:
+      if (cfg == 1) MOE_GEMM(8, 4, 2, true);
+      else if (cfg == 2) MOE_GEMM(8, 8, 2, false);
+      else MOE_GEMM(8, 8, 2, true);
+      break;
     default: return MOE_E_SHAPE;
   }
+#undef MOE_GEMM
   return (int)hipGetLastError();
 }
 
@@ -296,6 +468,7 @@ static int check_dims(int T, int H, int I, int E, int K) {
   if (T < 0 || H < 1 || I < 1 || E < 1 || E > MOE_MAX_EXPERTS || K < 1 || K > MOE_MAX_TOPK) return MOE_E_SHAPE;
   if ((long)T * K > (1l << 30)) return MOE_E_SHAPE;
   if (H % kBlock || I % kBlock) return MOE_E_ALIGN;
+  if (H > kMaxKB * kBlock || I > kMaxKB * kBlock) return MOE_E_SHAPE;
   return MOE_OK;
 }
 

@@ -2,6 +2,7 @@
 #pragma once
 #include <stddef.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 namespace moe {
 
@@ -15,9 +16,12 @@ static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; 
 // more than T rows: small T gets small tiles.
 static inline int choose_tile_m(int T, int K, int E) {
   (void)K; (void)E;
+  static int forced = -1;
+  if (forced < 0) { const char *s = getenv("MOE_HIP_TILE_M"); forced = s ? atoi(s) : 0; }
   if (T <= 16) return 16;
   if (T <= 32) return 32;
   if (T <= 64) return 64;
+  if (forced == 192) return 192;
   return 128;
 }
 
