@@ -189,7 +189,9 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     const int t = min(wave * NTOK + u, NROW8 - 1);
     const int row = 8 * t + (lane >> 3);
     const int c = (lane & 7) ^ (lane >> 3);
-    tok_src[u] = (size_t)sm.arow[row] * a.Kd + c * 16;
+    // row-groups past the tile's last row are never read by a matrix instruction that matters:
+    // every lane fetches the same 16 bytes there, which costs one cache line instead of eight
+    tok_src[u] = 8 * t < rows ? (size_t)sm.arow[row] * a.Kd + c * 16 : (size_t)sm.arow[0] * a.Kd;
     tok_m0[u] = t * 1024;
   }
   constexpr int NSA = (BM + 63) / 64;                  // 64-row groups of scales
@@ -258,7 +260,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   // group first issues all of its LDS reads (one exposed LDS latency per group, not per tile),
   // then its matrix instructions back to back, each tile's scale multiply-adds trailing the
   // matrix instruction that feeds them.
-  constexpr int MG = MT < 4 ? MT : 4;
+  constexpr int MG = MT < 4 ? MT : (MT % 4 == 0 && MT <= 8 ? 4 : (MT % 3 == 0 ? 3 : 2));
   auto compute = [&](int stage, int kb, const v4i(&lo)[WT], const v4i(&hi)[WT]) {
     v8i wc[WT];
     const uint8_t *wbase = sm.wt[WREG ? 0 : stage] + wave * (WT * 2048) + lane * 16;
@@ -458,6 +460,7 @@ static int launch_gemm(hipStream_t st, GemmArgs &a, int tile_m, int max_mtiles) 
       else if (cfg == 2) MOE_GEMM(8, 8, 2, false);
       else MOE_GEMM(8, 8, 2, true);
       break;
+    case 192: MOE_GEMM(12, 8, 2, true); break;
     default: return MOE_E_SHAPE;
   }
 #undef MOE_GEMM

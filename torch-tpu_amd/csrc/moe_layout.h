@@ -15,14 +15,14 @@ static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; 
 // without passing it around.  A token's K experts are distinct, so no expert ever holds
 // more than T rows: small T gets small tiles.
 static inline int choose_tile_m(int T, int K, int E) {
-  (void)K; (void)E;
-  static int forced = -1;
-  if (forced < 0) { const char *s = getenv("MOE_HIP_TILE_M"); forced = s ? atoi(s) : 0; }
   if (T <= 16) return 16;
   if (T <= 32) return 32;
   if (T <= 64) return 64;
-  if (forced == 192) return 192;
-  return 128;
+  // Balanced routing puts T*K/E rows on an expert, give or take a few standard deviations.  A
+  // second, nearly empty tile costs as much weight traffic as a full one, so prefer the tile
+  // that holds a typical expert whole.
+  const double mean = (double)T * K / E;
+  return mean > 96.0 ? 192 : 128;
 }
 
 struct PermuteWs {
