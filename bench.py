@@ -270,6 +270,12 @@ def main():
     dev = "cuda:0"
     cfg = WORKLOADS[args.workload]
     moe = build_layer(pkg, cfg, dev)
+    # a plain device copy of known size (1 GiB read + 1 GiB written): the yardstick that the
+    # FETCH_SIZE / WRITE_SIZE counters of a profiled run are scaled by
+    ref_src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    ref_dst = torch.empty_like(ref_src)
+    ref_dst.copy_(ref_src)
+    del ref_src, ref_dst
     sec, roof, x = bench_prefill(pkg, moe, cfg, dev, args.steps, args.warmup)
     T = cfg["T"]
     flops = gemm_flops(cfg, T)

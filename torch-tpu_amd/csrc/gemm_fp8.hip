@@ -11,7 +11,9 @@
 // 16x16 result) and the TOKEN tile is the "B" operand (its 16 rows become the columns).  A
 // lane then holds 4 consecutive output columns of ONE token, which makes the activation scale
 // a single value per lane and instruction, and lets the epilogue pack 4 outputs per store.
-//   lane l of an operand: row (l % 16), reduction bytes 32*(l / 16) .. +31 of the 128-step
+//   lane l of an operand: row (l % 16), reduction bytes 16g..16g+15 and 64+16g..64+16g+15 of the
+//                         128-step, g = l / 16 (the instruction only needs both operands to agree;
+//                         this split makes the 128-bit LDS reads of the token tile conflict-free)
 //   lane l of the result: c[r] = (weight row 4*(l / 16) + r, token l % 16)
 //
 // Data movement per step: weights stream HBM -> registers directly in operand layout (each
@@ -154,15 +156,18 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
 
   // ---- per-lane source addresses ------------------------------------------------------------
   // GATED: tiles 0..WT/2-1 are gate columns, WT/2..WT-1 the matching up columns.
-  const uint8_t *wptr[WT];
+  // Every global address of the loop is "uniform 64-bit base in SGPRs + 32-bit per-lane offset":
+  // one VGPR per address instead of two and no vector address arithmetic per step.
+  const uint8_t *wtile[WT];                            // uniform: first row of the wavefront's tile j
 #pragma unroll
   for (int j = 0; j < WT; j++) {
     int wrow;
-    if (GATED) wrow = (j < WT / 2 ? 0 : a.N) + strip * 128 + wave * (8 * WT) + (j % (WT / 2)) * 16 + li;
-    else wrow = strip * 256 + wave * (16 * WT) + j * 16 + li;
-    wrow = min(wrow, a.n_rows_w - 1);
-    wptr[j] = a.w + ((size_t)e * a.n_rows_w + wrow) * a.Kd + lg * 32;
+    if (GATED) wrow = (j < WT / 2 ? 0 : a.N) + strip * 128 + wave * (8 * WT) + (j % (WT / 2)) * 16;
+    else wrow = strip * 256 + wave * (16 * WT) + j * 16;
+    wrow = min(wrow, a.n_rows_w - 16);                 // tiles past the matrix re-read its last rows
+    wtile[j] = a.w + ((size_t)e * a.n_rows_w + wrow) * a.Kd;
   }
+  const uint32_t woff = (uint32_t)li * (uint32_t)a.Kd + lg * 16;   // lane's row and first 16-byte chunk in a tile
   // The strip's weight-block scales for all steps go to LDS once (two rows: gate/up blocks for
   // the gated GEMM, the strip's two 128-column blocks otherwise): uniform values re-read per
   // step from LDS instead of through the vector-memory queue.
@@ -182,7 +187,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   // the tile's end repeat its last eight rows (same bytes to the same place).
   constexpr int NROW8 = BM / 8;                        // 1 KB row-groups in the tile
   constexpr int NTOK = (NROW8 + NW - 1) / NW;
-  size_t tok_src[NTOK];
+  uint32_t tok_src[NTOK];
   uint32_t tok_m0[NTOK];
 #pragma unroll
   for (int u = 0; u < NTOK; u++) {
@@ -191,12 +196,12 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     const int c = (lane & 7) ^ (lane >> 3);
     // row-groups past the tile's last row are never read by a matrix instruction that matters:
     // every lane fetches the same 16 bytes there, which costs one cache line instead of eight
-    tok_src[u] = 8 * t < rows ? (size_t)sm.arow[row] * a.Kd + c * 16 : (size_t)sm.arow[0] * a.Kd;
+    tok_src[u] = 8 * t < rows ? (uint32_t)sm.arow[row] * (uint32_t)a.Kd + c * 16 : (uint32_t)sm.arow[0] * (uint32_t)a.Kd;
     tok_m0[u] = t * 1024;
   }
   constexpr int NSA = (BM + 63) / 64;                  // 64-row groups of scales
   const int sa_grp = wave % NSA;
-  const size_t sa_src = (size_t)sm.arow[min(sa_grp * 64 + lane, BM - 1)] * NKB;
+  const uint32_t sa_src = (uint32_t)sm.arow[min(sa_grp * 64 + lane, BM - 1)] * (uint32_t)NKB * 4u;   // bytes
   const uint32_t wt_base = __builtin_amdgcn_readfirstlane(lds_offset(&sm.wt[0][0])) + wave * (WT * 2048);
   constexpr uint32_t kWtStage = 16 * 2048;
   const uint32_t tok_base = __builtin_amdgcn_readfirstlane(lds_offset(&sm.tok[0][0]));
@@ -223,9 +228,9 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   auto request_weights_reg = [&](int kb, v4i(&lo)[WT], v4i(&hi)[WT]) {
 #pragma unroll
     for (int j = 0; j < WT; j++) {
-      const uint8_t *ptr = wptr[j] + (size_t)kb * 128;
-      asm volatile("global_load_dwordx4 %0, %2, off\n\tglobal_load_dwordx4 %1, %2, off offset:16"
-                   : "=&v"(lo[j]), "=&v"(hi[j]) : "v"(ptr) : "memory");
+      const uint8_t *base = wtile[j] + (size_t)kb * 128;
+      asm volatile("global_load_dwordx4 %0, %2, %3\n\tglobal_load_dwordx4 %1, %2, %3 offset:64"
+                   : "=&v"(lo[j]), "=&v"(hi[j]) : "v"(woff), "s"(base) : "memory");
     }
   };
   auto arrived_weights = [&](v4i(&lo)[WT], v4i(&hi)[WT]) {
@@ -235,24 +240,24 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   auto request = [&](int kb, int stage) {
 #pragma unroll
     for (int u = 0; u < NTOK; u++) {
-      const uint8_t *ptr = a.aq + tok_src[u] + (size_t)kb * 128;
+      const uint8_t *base = a.aq + (size_t)kb * 128;
       const uint32_t m0 = tok_base + stage * kTokStage + tok_m0[u];
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0), "v"(ptr) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(tok_src[u]), "s"(base) : "memory", "m0");
     }
     {
-      const float *ptr = a.as + sa_src + kb;
+      const float *base = a.as + kb;
       const uint32_t m0 = sa_base + stage * kSaStage;
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(m0), "v"(ptr) : "memory", "m0");
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(m0), "v"(sa_src), "s"(base) : "memory", "m0");
     }
     if (!WREG)
 #pragma unroll
     for (int j = 0; j < WT; j++) {
-      const uint8_t *ptr = wptr[j] + (size_t)kb * 128;
+      const uint8_t *base = wtile[j] + (size_t)kb * 128;
       const uint32_t m0 = wt_base + stage * kWtStage + j * 2048;
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\t"
-                   // the instruction offset moves the LDS address as well as the global one: 0x400 - 16
-                   "s_add_u32 m0, m0, 0x3f0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off offset:16"
-                   ::"s"(m0), "v"(ptr) : "memory", "m0", "scc");
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t"
+                   // the instruction offset moves the LDS address as well as the global one: 0x400 - 64
+                   "s_add_u32 m0, m0, 0x3c0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:64"
+                   ::"s"(m0), "v"(woff), "s"(base) : "memory", "m0", "scc");
     }
   };
 
@@ -260,7 +265,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   // group first issues all of its LDS reads (one exposed LDS latency per group, not per tile),
   // then its matrix instructions back to back, each tile's scale multiply-adds trailing the
   // matrix instruction that feeds them.
-  constexpr int MG = MT < 4 ? MT : (MT % 4 == 0 && MT <= 8 ? 4 : (MT % 3 == 0 ? 3 : 2));
+  constexpr int MG = MT < 4 ? MT : (MT % 4 == 0 && MT <= 8 ? 4 : (DEPTH >= 3 ? 2 : 3));
   auto compute = [&](int stage, int kb, const v4i(&lo)[WT], const v4i(&hi)[WT]) {
     v8i wc[WT];
     const uint8_t *wbase = sm.wt[WREG ? 0 : stage] + wave * (WT * 2048) + lane * 16;
@@ -271,7 +276,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     }
     const float s0 = sm.sb[sb_row0][kb], s1 = sm.sb[sb_row1][kb];
     const uint8_t *tbase = sm.tok[stage] + li * 128;
-    const int o0 = ((2 * lg) ^ (li & 7)) << 4, o1 = ((2 * lg + 1) ^ (li & 7)) << 4;
+    const int o0 = (lg ^ (li & 7)) << 4, o1 = ((lg + 4) ^ (li & 7)) << 4;
     const float *sap = sm.sa[stage] + li;
 #pragma unroll
     for (int mg = 0; mg < MT / MG; mg++) {
@@ -460,7 +465,10 @@ static int launch_gemm(hipStream_t st, GemmArgs &a, int tile_m, int max_mtiles) 
       else if (cfg == 2) MOE_GEMM(8, 8, 2, false);
       else MOE_GEMM(8, 8, 2, true);
       break;
-    case 192: MOE_GEMM(12, 8, 2, true); break;
+    case 192:
+      if (cfg == 3) MOE_GEMM(12, 8, 3, true);
+      else MOE_GEMM(12, 8, 2, true);
+      break;
     default: return MOE_E_SHAPE;
   }
 #undef MOE_GEMM
@@ -472,6 +480,8 @@ static int check_dims(int T, int H, int I, int E, int K) {
   if ((long)T * K > (1l << 30)) return MOE_E_SHAPE;
   if (H % kBlock || I % kBlock) return MOE_E_ALIGN;
   if (H > kMaxKB * kBlock || I > kMaxKB * kBlock) return MOE_E_SHAPE;
+  // per-lane offsets into the activation tensors are 32-bit
+  if ((double)T * H >= 2147483648.0 || (double)T * K * I >= 2147483648.0) return MOE_E_SHAPE;
   return MOE_OK;
 }
 
