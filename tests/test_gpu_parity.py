@@ -283,11 +283,13 @@ def test_fused_experts(pkg, oracle, dev, T, H, I, E, K):
     check_experts(pkg, oracle, dev, x, layer, ids, w)
 
 
-def test_fused_experts_with_shared_expert_and_empty_experts(pkg, oracle, dev):
-    say("shared expert")
-    T, H, I, E, K = 70, 512, 256, 16, 4
+@pytest.mark.parametrize("T,I_sh", [(70, 384), (70, 256), (5, 256), (200, 256)])
+def test_fused_experts_with_shared_expert_and_empty_experts(pkg, oracle, dev, T, I_sh):
+    """A shared expert of the routed width rides in the routed launches; another width gets its own."""
+    say("shared expert", T, I_sh)
+    H, I, E, K = 512, 256, 16, 4
     layer = oracle.make_layer(E, H, I, seed=6)
-    shared = oracle.make_layer(1, H, 384, seed=7)
+    shared = oracle.make_layer(1, H, I_sh, seed=7)
     g = torch.Generator().manual_seed(8)
     x = torch.randn(T, H, generator=g).to(torch.bfloat16)
     ids, w = distinct_ids(T, 8, K, seed=9)               # experts 8..15 never chosen

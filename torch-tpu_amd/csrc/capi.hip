@@ -9,10 +9,12 @@ int permute_launch(hipStream_t st, const int32_t *ids, int T, int K, int E, int 
                    int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &ws);
 int gemm1_launch(hipStream_t st, const uint8_t *xq, const float *xs, int T, int H, const uint8_t *w13,
                  const float *w13s, int I, int E, int K, const int32_t *sorted_slot, const int32_t *expert_offsets,
-                 const PermuteWs *pw, int fixed_expert, uint8_t *hq, float *hs);
+                 const PermuteWs *pw, int fixed_expert, uint8_t *hq, float *hs, const uint8_t *sh_w13,
+                 const float *sh_w13s, uint8_t *sh_hq, float *sh_hs);
 int gemm2_launch(hipStream_t st, const uint8_t *hq, const float *hs, int rows_a, int T, int H, const uint8_t *w2,
                  const float *w2s, int I, int E, int K, const int32_t *sorted_slot, const int32_t *expert_offsets,
-                 const PermuteWs *pw, int fixed_expert, uint16_t *y);
+                 const PermuteWs *pw, int fixed_expert, uint16_t *y, const uint8_t *sh_hq, const float *sh_hs,
+                 int sh_rows, const uint8_t *sh_w2, const float *sh_w2s, uint16_t *sh_y);
 
 // Carves the caller's workspace.  Every piece starts on a 256-byte boundary.
 struct FusedWs {
@@ -112,18 +114,23 @@ extern "C" int moe_fused_experts_fp8(void *stream, const void *x_bf16, int T, in
   if (rc) return rc;
   rc = moe_act_quant(stream, x_bf16, T, H, w.xq, w.xs);
   if (rc) return rc;
-  rc = gemm1_launch(st, w.xq, w.xs, T, H, w13, w13_scale, I, E, K, w.sorted_slot, w.expert_offsets, &pw, -1, w.hq, w.hs);
+  // a shared expert of the routed experts' width rides in the routed launches (its tiles fill the
+  // machine together with theirs); any other width gets launches of its own
+  const bool fuse_shared = has_shared && I_sh == I;
+  rc = gemm1_launch(st, w.xq, w.xs, T, H, w13, w13_scale, I, E, K, w.sorted_slot, w.expert_offsets, &pw, -1, w.hq, w.hs,
+                    fuse_shared ? shared_w13 : nullptr, shared_w13_scale, w.sh_hq, w.sh_hs);
   if (rc) return rc;
   uint16_t *y = out_mode == 0 ? (uint16_t *)out_bf16 : w.y;
-  rc = gemm2_launch(st, w.hq, w.hs, T * K, T, H, w2, w2_scale, I, E, K, w.sorted_slot, w.expert_offsets, &pw, -1, y);
+  rc = gemm2_launch(st, w.hq, w.hs, T * K, T, H, w2, w2_scale, I, E, K, w.sorted_slot, w.expert_offsets, &pw, -1, y,
+                    w.sh_hq, w.sh_hs, T, fuse_shared ? shared_w2 : nullptr, shared_w2_scale, w.sh_y);
   if (rc) return rc;
   if (out_mode == 0) return MOE_OK;
-  if (has_shared) {
+  if (has_shared && !fuse_shared) {
     rc = gemm1_launch(st, w.xq, w.xs, T, H, shared_w13, shared_w13_scale, I_sh, 1, 1, nullptr, nullptr, nullptr, 0,
-                      w.sh_hq, w.sh_hs);
+                      w.sh_hq, w.sh_hs, nullptr, nullptr, nullptr, nullptr);
     if (rc) return rc;
     rc = gemm2_launch(st, w.sh_hq, w.sh_hs, T, T, H, shared_w2, shared_w2_scale, I_sh, 1, 1, nullptr, nullptr, nullptr,
-                      0, w.sh_y);
+                      0, w.sh_y, nullptr, nullptr, 0, nullptr, nullptr, nullptr);
     if (rc) return rc;
   }
   return moe_weighted_reduce(stream, y, routing_weights, has_shared ? w.sh_y : nullptr, T, K, H, out_bf16);

@@ -64,6 +64,16 @@ struct GemmArgs {
   int E;                        // experts (tile_prefix[E] = number of row tiles)
   int fixed_expert;             // >= 0: dense mode, every row belongs to this expert and A row p = p
   int max_mtiles;               // entries allocated in tile_expert
+  // optional shared expert riding in the same launch (same N / Kd as the routed experts): its
+  // row tiles follow the routed ones; rows are the tokens in order
+  const uint8_t *sh_aq;         // its activations ([sh_rows, Kd]; the token tensor for the first GEMM)
+  const float *sh_as;
+  const uint8_t *sh_w;
+  const float *sh_ws;
+  uint8_t *sh_hq;
+  float *sh_hs;
+  uint16_t *sh_y;
+  int sh_rows;                  // 0 = no shared expert in this launch
 };
 
 constexpr int kMaxKB = 256;                 // reduction length limit: 256 * 128 = 32768
@@ -121,7 +131,8 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   // has its own L2, works on a contiguous range of the real tiles (their number is only known
   // on the device): neighbours in that range share the token tile and, for experts with more
   // than one row tile, the weight strip.
-  const int n_mtiles = a.fixed_expert >= 0 ? (a.rows_a + BM - 1) / BM : min(a.tile_prefix[a.E], a.max_mtiles);
+  const int n_routed = a.fixed_expert >= 0 ? (a.rows_a + BM - 1) / BM : min(a.tile_prefix[a.E], a.max_mtiles);
+  const int n_mtiles = n_routed + (a.sh_rows + BM - 1) / BM;
   const int n_work = n_mtiles * a.n_strips;
   const int per_xcd = (n_work + 7) >> 3;
   if ((int)(blockIdx.x >> 3) >= per_xcd) return;
@@ -130,7 +141,13 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   const int mtile = logical / a.n_strips;
   const int strip = logical - mtile * a.n_strips;
   int e, row0, rows;                                  // expert, first permuted row, rows in tile
-  if (a.fixed_expert >= 0) {
+  const bool shared = mtile >= n_routed;              // a tile of the shared expert
+  const bool direct = shared || a.fixed_expert >= 0;  // rows are taken in order, no permutation
+  if (shared) {
+    e = 0;
+    row0 = (mtile - n_routed) * BM;
+    rows = min(BM, a.sh_rows - row0);
+  } else if (a.fixed_expert >= 0) {
     e = a.fixed_expert;
     row0 = mtile * BM;
     rows = min(BM, a.rows_a - row0);
@@ -140,14 +157,19 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     row0 = a.expert_offsets[e] + (mtile - a.tile_prefix[e]) * BM;
     rows = min(BM, a.expert_offsets[e + 1] - row0);
   }
+  const uint8_t *const aq = shared ? a.sh_aq : a.aq;
+  const float *const as = shared ? a.sh_as : a.as;
+  const uint8_t *const wq = shared ? a.sh_w : a.w;
+  const float *const ws = shared ? a.sh_ws : a.ws;
+  const int rows_a = shared ? a.sh_rows : a.rows_a;
   if (rows <= 0) return;
   const int mt_live = (rows + 15) >> 4;               // m-tiles that hold at least one row
 
   for (int i = tid; i < BM; i += NT) {
     const int p = row0 + min(i, rows - 1);
     int src = p;
-    if (GATED && a.fixed_expert < 0) src = a.sorted_slot[p] / a.topk;
-    sm.arow[i] = min(max(src, 0), a.rows_a - 1);
+    if (GATED && !direct) src = a.sorted_slot[p] / a.topk;
+    sm.arow[i] = min(max(src, 0), rows_a - 1);
   }
   __syncthreads();
 
@@ -165,7 +187,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     if (GATED) wrow = (j < WT / 2 ? 0 : a.N) + strip * 128 + wave * (8 * WT) + (j % (WT / 2)) * 16;
     else wrow = strip * 256 + wave * (16 * WT) + j * 16;
     wrow = min(wrow, a.n_rows_w - 16);                 // tiles past the matrix re-read its last rows
-    wtile[j] = a.w + ((size_t)e * a.n_rows_w + wrow) * a.Kd;
+    wtile[j] = wq + ((size_t)e * a.n_rows_w + wrow) * a.Kd;
   }
   const uint32_t woff = (uint32_t)li * (uint32_t)a.Kd + lg * 16;   // lane's row and first 16-byte chunk in a tile
   // The strip's weight-block scales for all steps go to LDS once (two rows: gate/up blocks for
@@ -176,7 +198,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     const int blk1 = GATED ? (a.N >> 7) + strip : min(strip * 2 + 1, n_wblk - 1);
     for (int i = tid; i < 2 * NKB; i += NT) {
       const int r = i >= NKB, kb = i - r * NKB;
-      sm.sb[r][kb] = a.ws[((size_t)e * n_wblk + (r ? blk1 : blk0)) * NKB + kb];
+      sm.sb[r][kb] = ws[((size_t)e * n_wblk + (r ? blk1 : blk0)) * NKB + kb];
     }
   }
   const int sb_row0 = GATED ? 0 : (wave * WT) / 8;      // which of the two rows this wavefront's tiles use
@@ -240,12 +262,12 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   auto request = [&](int kb, int stage) {
 #pragma unroll
     for (int u = 0; u < NTOK; u++) {
-      const uint8_t *base = a.aq + (size_t)kb * 128;
+      const uint8_t *base = aq + (size_t)kb * 128;
       const uint32_t m0 = tok_base + stage * kTokStage + tok_m0[u];
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(tok_src[u]), "s"(base) : "memory", "m0");
     }
     {
-      const float *base = a.as + kb;
+      const float *base = as + kb;
       const uint32_t m0 = sa_base + stage * kSaStage;
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(m0), "v"(sa_src), "s"(base) : "memory", "m0");
     }
@@ -418,9 +440,9 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
 #pragma unroll
       for (int j = 0; j < G; j++) {
         const uint32_t packed = pack4_fp8(acc[mt][j][0] / sc, acc[mt][j][1] / sc, acc[mt][j][2] / sc, acc[mt][j][3] / sc);
-        if (valid) *(uint32_t *)(a.hq + orow * a.N + strip * 128 + wave * (16 * G) + j * 16 + lg * 4) = packed;
+        if (valid) *(uint32_t *)((shared ? a.sh_hq : a.hq) + orow * a.N + strip * 128 + wave * (16 * G) + j * 16 + lg * 4) = packed;
       }
-      if (valid && wave == 0 && lg == 0) a.hs[orow * n_grp + strip] = sc;
+      if (valid && wave == 0 && lg == 0) (shared ? a.sh_hs : a.hs)[orow * n_grp + strip] = sc;
     }
   } else {
 #pragma unroll
@@ -428,7 +450,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
       const int i = mt * 16 + li;
       const bool valid = i < rows;
       int slot = row0 + min(i, rows - 1);
-      if (a.fixed_expert < 0) slot = a.sorted_slot[slot];
+      if (!direct) slot = a.sorted_slot[slot];
 #pragma unroll
       for (int j = 0; j < WT; j++) {
         const int col = strip * 256 + wave * (16 * WT) + j * 16 + lg * 4;
@@ -436,7 +458,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
           v2i o;
           o[0] = (int)((uint32_t)f32_to_bf16(acc[mt][j][0]) | ((uint32_t)f32_to_bf16(acc[mt][j][1]) << 16));
           o[1] = (int)((uint32_t)f32_to_bf16(acc[mt][j][2]) | ((uint32_t)f32_to_bf16(acc[mt][j][3]) << 16));
-          *(v2i *)(a.y + (size_t)slot * a.N + col) = o;
+          *(v2i *)((shared ? a.sh_y : a.y) + (size_t)slot * a.N + col) = o;
         }
       }
     }
@@ -448,7 +470,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
 template <bool GATED>
 static int launch_gemm(hipStream_t st, GemmArgs &a, int tile_m, int max_mtiles) {
   a.n_strips = GATED ? a.N / 128 : (a.N + 255) / 256;
-  a.max_mtiles = max_mtiles;
+  a.max_mtiles = max_mtiles - (a.sh_rows + tile_m - 1) / tile_m;
   long total = (long)max_mtiles * a.n_strips;
   total = (total + 7) / 8 * 8;
   if (total <= 0 || total > 0x7fffffffl) return MOE_E_SHAPE;
@@ -487,8 +509,10 @@ static int check_dims(int T, int H, int I, int E, int K) {
 
 int gemm1_launch(hipStream_t st, const uint8_t *xq, const float *xs, int T, int H, const uint8_t *w13,
                  const float *w13s, int I, int E, int K, const int32_t *sorted_slot, const int32_t *expert_offsets,
-                 const PermuteWs *pw, int fixed_expert, uint8_t *hq, float *hs) {
+                 const PermuteWs *pw, int fixed_expert, uint8_t *hq, float *hs, const uint8_t *sh_w13,
+                 const float *sh_w13s, uint8_t *sh_hq, float *sh_hs) {
   GemmArgs a{};
+  if (sh_w13) { a.sh_aq = xq; a.sh_as = xs; a.sh_w = sh_w13; a.sh_ws = sh_w13s; a.sh_hq = sh_hq; a.sh_hs = sh_hs; a.sh_rows = T; }
   a.aq = xq; a.as = xs; a.w = w13; a.ws = w13s;
   a.sorted_slot = sorted_slot; a.expert_offsets = expert_offsets;
   a.tile_prefix = pw ? pw->tile_prefix : nullptr; a.tile_expert = pw ? pw->tile_expert : nullptr;
@@ -496,13 +520,15 @@ int gemm1_launch(hipStream_t st, const uint8_t *xq, const float *xs, int T, int 
   a.Kd = H; a.N = I; a.n_rows_w = 2 * I; a.rows_a = T; a.topk = K; a.E = E; a.fixed_expert = fixed_expert;
   const int tile_m = choose_tile_m(T, K, E);
   const int max_mtiles = fixed_expert >= 0 ? (T + tile_m - 1) / tile_m : pw->max_tiles;
-  return launch_gemm<true>(st, a, tile_m, max_mtiles);
+  return launch_gemm<true>(st, a, tile_m, max_mtiles + (a.sh_rows + tile_m - 1) / tile_m);
 }
 
 int gemm2_launch(hipStream_t st, const uint8_t *hq, const float *hs, int rows_a, int T, int H, const uint8_t *w2,
                  const float *w2s, int I, int E, int K, const int32_t *sorted_slot, const int32_t *expert_offsets,
-                 const PermuteWs *pw, int fixed_expert, uint16_t *y) {
+                 const PermuteWs *pw, int fixed_expert, uint16_t *y, const uint8_t *sh_hq, const float *sh_hs,
+                 int sh_rows, const uint8_t *sh_w2, const float *sh_w2s, uint16_t *sh_y) {
   GemmArgs a{};
+  if (sh_w2) { a.sh_aq = sh_hq; a.sh_as = sh_hs; a.sh_w = sh_w2; a.sh_ws = sh_w2s; a.sh_y = sh_y; a.sh_rows = sh_rows; }
   a.aq = hq; a.as = hs; a.w = w2; a.ws = w2s;
   a.sorted_slot = sorted_slot; a.expert_offsets = expert_offsets;
   a.tile_prefix = pw ? pw->tile_prefix : nullptr; a.tile_expert = pw ? pw->tile_expert : nullptr;
@@ -510,7 +536,7 @@ int gemm2_launch(hipStream_t st, const uint8_t *hq, const float *hs, int rows_a,
   a.Kd = I; a.N = H; a.n_rows_w = H; a.rows_a = rows_a; a.topk = K; a.E = E; a.fixed_expert = fixed_expert;
   const int tile_m = choose_tile_m(T, K, E);
   const int max_mtiles = fixed_expert >= 0 ? (rows_a + tile_m - 1) / tile_m : pw->max_tiles;
-  return launch_gemm<false>(st, a, tile_m, max_mtiles);
+  return launch_gemm<false>(st, a, tile_m, max_mtiles + (a.sh_rows + tile_m - 1) / tile_m);
 }
 
 }  // namespace moe
@@ -527,7 +553,7 @@ extern "C" int moe_gemm1_swiglu(void *stream, const uint8_t *xq, const float *xs
   if (T == 0) return MOE_OK;
   PermuteWs pw = permute_ws_layout(const_cast<void *>(permute_workspace), T, K, E);
   return gemm1_launch((hipStream_t)stream, xq, xs, T, H, w13, w13_scale, I, E, K, sorted_slot, expert_offsets, &pw, -1,
-                      hq, hs);
+                      hq, hs, nullptr, nullptr, nullptr, nullptr);
 }
 
 extern "C" int moe_gemm2(void *stream, const uint8_t *hq, const float *hs, int T, int H, const uint8_t *w2,
@@ -542,5 +568,5 @@ extern "C" int moe_gemm2(void *stream, const uint8_t *hq, const float *hs, int T
   if (T == 0) return MOE_OK;
   PermuteWs pw = permute_ws_layout(const_cast<void *>(permute_workspace), T, K, E);
   return gemm2_launch((hipStream_t)stream, hq, hs, T * K, T, H, w2, w2_scale, I, E, K, sorted_slot, expert_offsets, &pw,
-                      -1, (uint16_t *)y_bf16);
+                      -1, (uint16_t *)y_bf16, nullptr, nullptr, 0, nullptr, nullptr, nullptr);
 }

@@ -9,7 +9,7 @@
 //   scatter  one wavefront per chunk again: ranks its slots in slot order with a ballot
 //            "match-any" loop, so equal experts keep their original order (stable), and writes
 //            sorted_slot / slot_to_row.
-// A problem of at most kChunk slots is done by one wavefront in a single launch.
+// A problem of at most kChunk slots is done by one workgroup in a single launch.
 #include "moe_common.h"
 #include "moe_layout.h"
 #include "../../include/moe_hip.h"
@@ -137,64 +137,64 @@ __global__ __launch_bounds__(64) void permute_scatter_kernel(const int32_t *__re
   }
 }
 
-// whole permutation of at most kChunk slots by one wavefront
-__global__ __launch_bounds__(64) void permute_small_kernel(const int32_t *__restrict__ ids, int TK, int E, int tile_m,
-                                                           int max_tiles, int32_t *__restrict__ sorted_slot,
-                                                           int32_t *__restrict__ expert_offsets,
-                                                           int32_t *__restrict__ slot_to_row,
-                                                           int32_t *__restrict__ tile_prefix,
-                                                           int32_t *__restrict__ tile_expert) {
+// Whole permutation of at most kChunk slots by one workgroup, one slot per thread: the rank of a
+// slot inside its expert is the number of earlier slots with the same id (every thread walks
+// the id list in LDS in step, so each read is a broadcast), the expert offsets are a block scan of
+// the histogram.
+__global__ __launch_bounds__(kChunk) void permute_small_kernel(const int32_t *__restrict__ ids, int TK, int E, int tile_m,
+                                                              int max_tiles, int32_t *__restrict__ sorted_slot,
+                                                              int32_t *__restrict__ expert_offsets,
+                                                              int32_t *__restrict__ slot_to_row,
+                                                              int32_t *__restrict__ tile_prefix,
+                                                              int32_t *__restrict__ tile_expert) {
   __shared__ int hist[MOE_MAX_EXPERTS];
-  __shared__ int base[MOE_MAX_EXPERTS];
-  const int lane = threadIdx.x;
-  for (int e = lane; e < E; e += 64) hist[e] = 0;
+  __shared__ int offs[MOE_MAX_EXPERTS];
+  __shared__ int sid[kChunk];
+  __shared__ int wave_sums[2][kChunk / 64];
+  const int s = threadIdx.x;
+  for (int e = s; e < E; e += kChunk) hist[e] = 0;
+  int v = (s < TK) ? ids[s] : -1;
+  const bool valid = v >= 0 && v < E;
+  sid[s] = valid ? v : -1;
   __syncthreads();
-  for (int s = lane; s < TK; s += 64) {
-    int v = ids[s];
-    if (v >= 0 && v < E) atomicAdd(&hist[v], 1);
-  }
+  if (valid) atomicAdd(&hist[v], 1);
+  int rank = 0;
+  for (int j = 0; j < s; j++) rank += (sid[j] == v);
   __syncthreads();
-  // lane owns experts [lane*per, lane*per+per)
-  const int per = (E + 63) / 64;
-  int sum = 0, tsum = 0;
-  for (int j = 0; j < per; j++) {
-    int e = lane * per + j;
-    if (e < E) { sum += hist[e]; tsum += (hist[e] + tile_m - 1) / tile_m; }
-  }
-  int inc = sum, tinc = tsum;
+  // exclusive scans of the counts and of the tile counts over the experts, kChunk experts per pass
+  int carry = 0, tcarry = 0;
+  for (int e0 = 0; e0 < E; e0 += kChunk) {
+    const int e = e0 + s;
+    const int c = e < E ? hist[e] : 0;
+    const int t = (c + tile_m - 1) / tile_m;
+    int inc = c, tinc = t;
+    const int lane = s & 63, wave = s >> 6;
 #pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    int y = __shfl_up(inc, off, 64), ty = __shfl_up(tinc, off, 64);
-    if (lane >= off) { inc += y; tinc += ty; }
-  }
-  int run = inc - sum, trun = tinc - tsum;
-  for (int j = 0; j < per; j++) {
-    int e = lane * per + j;
-    if (e < E) {
-      int cnt = hist[e];
-      expert_offsets[e] = run;
-      base[e] = run;
-      tile_prefix[e] = trun;
-      write_tiles(e, cnt, trun, tile_m, tile_expert, max_tiles);
-      run += cnt;
-      trun += (cnt + tile_m - 1) / tile_m;
+    for (int off = 1; off < 64; off <<= 1) {
+      const int y = __shfl_up(inc, off, 64), ty = __shfl_up(tinc, off, 64);
+      if (lane >= off) { inc += y; tinc += ty; }
     }
+    if (lane == 63) { wave_sums[0][wave] = inc; wave_sums[1][wave] = tinc; }
+    __syncthreads();
+    int base = carry, tbase = tcarry, tot = 0, ttot = 0;
+    for (int w = 0; w < kChunk / 64; w++) {
+      if (w < wave) { base += wave_sums[0][w]; tbase += wave_sums[1][w]; }
+      tot += wave_sums[0][w]; ttot += wave_sums[1][w];
+    }
+    if (e < E) {
+      offs[e] = base + inc - c;
+      expert_offsets[e] = base + inc - c;
+      tile_prefix[e] = tbase + tinc - t;
+      write_tiles(e, c, tbase + tinc - t, tile_m, tile_expert, max_tiles);
+    }
+    carry += tot; tcarry += ttot;
+    __syncthreads();
   }
-  if (lane == 63) { expert_offsets[E] = inc; tile_prefix[E] = tinc; }
-  __syncthreads();
-  for (int s0 = 0; s0 < TK; s0 += 64) {
-    const int s = s0 + lane;
-    int v = (s < TK) ? ids[s] : -1;
-    const bool valid = (s < TK) && v >= 0 && v < E;
-    int rank, cnt;
-    bool is_last;
-    match_rank(v, valid, lane, rank, cnt, is_last);
-    int row = valid ? base[v] + rank : -1;
-    __syncthreads();
-    if (valid && is_last) base[v] += cnt;
-    __syncthreads();
+  if (s == 0) { expert_offsets[E] = carry; tile_prefix[E] = tcarry; }
+  if (s < TK) {
+    const int row = valid ? offs[v] + rank : -1;
     if (valid && row < TK) sorted_slot[row] = s;
-    if (s < TK) slot_to_row[s] = row;
+    slot_to_row[s] = row;
   }
 }
 
@@ -202,7 +202,7 @@ int permute_launch(hipStream_t st, const int32_t *ids, int T, int K, int E, int 
                    int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &ws) {
   const int TK = T * K;
   if (TK <= kChunk) {
-    permute_small_kernel<<<1, 64, 0, st>>>(ids, TK, E, tile_m, ws.max_tiles, sorted_slot, expert_offsets, slot_to_row,
+    permute_small_kernel<<<1, kChunk, 0, st>>>(ids, TK, E, tile_m, ws.max_tiles, sorted_slot, expert_offsets, slot_to_row,
                                            ws.tile_prefix, ws.tile_expert);
     return (int)hipGetLastError();
   }

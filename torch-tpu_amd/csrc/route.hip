@@ -22,14 +22,28 @@ __device__ __forceinline__ bool better(float av, int ai, float bv, int bi) {
   return (av > bv) || (av == bv && ai < bi);
 }
 
+// Arg-max over the wavefront with data-parallel-primitive moves (no LDS round trips): an inclusive
+// scan inside each row of 16 lanes (row_shr 1, 2, 4, 8), then row 0 -> 1 and 2 -> 3 (row_bcast:15),
+// then rows 0-1 -> 2-3 (row_bcast:31); lane 63 ends up with the winner, which is broadcast.
+// Lanes that have no source in a move see a candidate that loses to everything.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ void argmax_step(Best &b) {
+  const float ov = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, b.v), CTRL, ROW_MASK, 0xf, false));
+  const int oi = __builtin_amdgcn_update_dpp(0x7fffffff, b.i, CTRL, ROW_MASK, 0xf, false);
+  if (!better(b.v, b.i, ov, oi)) { b.v = ov; b.i = oi; }
+}
+
 __device__ __forceinline__ Best wave_argmax(Best b) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) {
-    float ov = __shfl_xor(b.v, off, 64);
-    int oi = __shfl_xor(b.i, off, 64);
-    if (!better(b.v, b.i, ov, oi)) { b.v = ov; b.i = oi; }
-  }
-  return b;
+  argmax_step<0x111, 0xf>(b);   // row_shr:1
+  argmax_step<0x112, 0xf>(b);   // row_shr:2
+  argmax_step<0x114, 0xf>(b);   // row_shr:4
+  argmax_step<0x118, 0xf>(b);   // row_shr:8
+  argmax_step<0x142, 0xa>(b);   // row_bcast:15 into rows 1 and 3
+  argmax_step<0x143, 0xc>(b);   // row_bcast:31 into rows 2 and 3
+  Best r;
+  r.v = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, b.v), 63));
+  r.i = __builtin_amdgcn_readlane(b.i, 63);
+  return r;
 }
 
 __device__ __forceinline__ float round_to_bf16(float f) { return bf16_to_f32(f32_to_bf16(f)); }
