@@ -94,7 +94,7 @@ int moe_route_topk(void *stream, const void *logits, int logits_dtype, const flo
  * workspace: moe_permute_workspace_bytes(T, K, E) bytes.
  */
 size_t moe_permute_workspace_bytes(int T, int K, int E);
-/* Rows of one expert that a grouped-GEMM workgroup owns for this problem shape (16..128); the
+/* Rows of one expert that a grouped-GEMM workgroup owns for this problem shape (16..192); the
  * permutation leaves the matching tile list in its workspace.  The reference's launcher picks
  * its token slice per core the same way, on the host (fusedMoE.cpp:60-78). */
 int moe_tile_rows(int T, int K, int E);

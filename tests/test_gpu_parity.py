@@ -350,3 +350,92 @@ def test_layer_module_end_to_end_toy_config(pkg, oracle, dev):
     assert torch.equal(ids.cpu(), ids_ref)
     ref = oracle.moe_w8a8_fp32(x, ids_ref, w_ref, *layer)
     assert outside_fraction(out.float().cpu(), ref) <= MAX_OUTSIDE
+
+
+# ----------------------------------------------------------------------------- full size, graphs
+def test_full_size_properties_deepseek_shape(pkg, oracle, dev):
+    """DeepSeek-V3 layer shape at T=4096 (too large for the oracle as a whole): routing and permutation
+    are checked exactly, the expert output through properties that do not depend on size, and a
+    sample of tokens against the oracle."""
+    say("full size C3")
+    T, H, I, E, K = 4096, 7168, 2048, 256, 8
+    g = torch.Generator(device=dev).manual_seed(3)
+    x = torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16)
+    wr = (torch.randn(E, H, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+
+    def weights(n, k, seed):
+        gg = torch.Generator(device=dev).manual_seed(seed)
+        q = torch.empty(E, n, k, dtype=torch.float8_e4m3fn, device=dev)
+        s = torch.empty(E, n // 128, k // 128, dtype=torch.float32, device=dev)
+        for e0 in range(0, E, 16):
+            w = (torch.randn(16, n, k, generator=gg, device=dev) * 0.02).to(torch.bfloat16)
+            q[e0:e0 + 16], s[e0:e0 + 16] = pkg.quant_weight_block128(w)
+        return q, s
+
+    w13, w13s = weights(2 * I, H, 1)
+    w2, w2s = weights(H, I, 2)
+    logits = torch.matmul(x, wr.t()).float()
+    w, ids, scores = pkg.moe_route(logits, K, "sigmoid", None, 8, 4, True, 2.5, return_scores=True)
+    w_ref, ids_ref = oracle.select_sigmoid_grouped(scores.cpu(), None, K, 8, 4, 2.5)
+    assert torch.equal(ids.cpu(), ids_ref) and torch.allclose(w.cpu(), w_ref, rtol=1e-5)
+    ss, off, s2r = pkg.moe_permute(ids, E)
+    ss_ref, off_ref, s2r_ref = oracle.permute_counting_sort(ids_ref, E)
+    assert torch.equal(ss.cpu(), ss_ref) and torch.equal(off.cpu(), off_ref) and torch.equal(s2r.cpu(), s2r_ref)
+
+    y = pkg.fused_experts_fp8(x, w13, w13s, w2, w2s, ids)                  # [T,K,H]
+    out = pkg.fused_experts_fp8(x, w13, w13s, w2, w2s, ids, w)             # [T,H]
+    torch.cuda.synchronize()
+    assert torch.isfinite(y.float()).all()
+    # (a) the weighted form is the fp32 weighted sum of the per-slot form
+    red = torch.einsum("tk,tkh->th", w, y.float())
+    torch.testing.assert_close(out.float(), red, rtol=1e-2, atol=1e-2)
+    # (b) a token's result does not depend on what else is in the batch, nor on slot order
+    sub = torch.arange(0, T, 37, device=dev)
+    y_sub = pkg.fused_experts_fp8(x[sub].contiguous(), w13, w13s, w2, w2s, ids[sub].contiguous())
+    assert torch.equal(y_sub.view(torch.int16), y[sub].view(torch.int16))
+    ids_rev = ids[sub].flip(1).contiguous()
+    y_rev = pkg.fused_experts_fp8(x[sub].contiguous(), w13, w13s, w2, w2s, ids_rev)
+    assert torch.equal(y_rev.flip(1).view(torch.int16), y[sub].view(torch.int16))
+    # (c) sixteen tokens against the oracle
+    pick = torch.arange(5, T, 256)
+    xs = x[pick.to(dev)].cpu()
+    layer = tuple(t.cpu() for t in (w13, w13s, w2, w2s))
+    ref = oracle.experts_w8a8_fp32(xs, ids_ref[pick], *layer)
+    got = y[pick.to(dev)].float().cpu()
+    assert outside_fraction(got, ref) <= MAX_OUTSIDE
+    assert oracle.cal_diff(ref, got)[0] < 1e-5
+
+
+def test_hip_graph_replay_matches_eager(pkg, oracle, dev):
+    """The whole step under HIP graph capture: replayed several times, with eager work and
+    synchronisation in between, every replay must reproduce the eager bits."""
+    say("hip graph")
+    T, H, I, E, K = 8, 512, 256, 16, 4
+    layer = tuple(t.to(dev) for t in oracle.make_layer(E, H, I, seed=21))
+    shared = tuple(t.to(dev) for t in oracle.make_layer(1, H, I, seed=22))
+    g = torch.Generator().manual_seed(23)
+    wr = (torch.randn(E, H, generator=g) * 0.02).to(torch.bfloat16).to(dev)
+    moe = pkg.FusedMoE(wr, *layer, top_k=K, mode="sigmoid", n_groups=4, topk_groups=2, scale=2.5, shared=shared)
+    xs = [torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev) for _ in range(3)]
+    x_static = xs[0].clone()
+    out_static = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    eager = [moe(x).clone() for x in xs]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        moe(x_static, out=out_static)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        moe(x_static, out=out_static)
+    for rep in range(2):
+        for x, want in zip(xs, eager):
+            x_static.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out_static, want), f"replay {rep} differs from eager"
+            scratch = moe(xs[(rep + 1) % 3])            # eager work between replays
+            torch.cuda.synchronize()
+            del scratch

@@ -1,8 +1,8 @@
 // Grouped block-scaled FP8 GEMMs of the expert MLP on gfx950 matrix cores.
 //
-// One workgroup (4 wavefronts) owns a tile of one expert: BM = 16*MT permuted rows (tokens)
-// by a strip of that expert's weight rows (output columns).  The reduction runs in steps of
-// 128 = one quantisation block = one v_mfma_f32_16x16x128_f8f6f4, so every matrix
+// One workgroup of NW = 8 wavefronts owns a tile of one expert: BM = 16*MT permuted rows
+// (tokens) by a strip of that expert's weight rows (output columns).  The reduction runs in
+// steps of 128 = one quantisation block = one v_mfma_f32_16x16x128_f8f6f4, so every matrix
 // instruction yields the un-scaled partial sum of exactly one (activation group, weight block)
 // pair and the two fp32 scales are applied in registers right after it:
 //     acc += partial * (act_scale[row, kb] * weight_scale[n_block, kb]).
@@ -16,31 +16,24 @@
 //                         this split makes the 128-bit LDS reads of the token tile conflict-free)
 //   lane l of the result: c[r] = (weight row 4*(l / 16) + r, token l % 16)
 //
-// Data movement per step: weights stream HBM -> registers directly in operand layout (each
-// weight byte is used by one wavefront only, so LDS would add nothing); the token tile is
-// shared by the four wavefronts and goes HBM/L2 -> registers -> LDS (XOR-swizzled 16-byte
-// chunks, conflict-free 128-bit reads), double buffered, one barrier per step.  Loads for
-// step kb+1 are issued before the matrix work of step kb.
+// Data movement per step: the token tile is shared by all wavefronts and goes HBM/L2 -> LDS
+// with direct-to-LDS loads (no registers held while in flight, XOR swizzle applied on the source
+// side) through DEPTH + 1 stages; each wavefront's WT = 16 / NW weight tiles are used by nobody
+// else and go HBM -> registers in operand layout through a DEPTH-deep register ring (WREG) or,
+// for small row tiles, -> LDS the same way as the tokens.  Requests run DEPTH steps ahead of
+// the matrix work and are waited for with hand-placed s_waitcnt; one barrier per step.
 //
 // GATED = true  (first GEMM): the strip is 128 gate columns plus the 128 matching up columns of
-//   W13; wavefront w owns gate columns 32w..32w+31 and the same up columns.  Epilogue:
+//   W13; wavefront w owns gate columns 16w..16w+15 and the same up columns.  Epilogue:
 //   h = silu(gate) * up, per-token amax over the strip's 128 columns (registers -> lane
-//   butterflies -> LDS across the four wavefronts), scale = max(amax, 1e-10) / 448, h / scale -> e4m3fn.
-// GATED = false (second GEMM): the strip is 256 output columns, wavefront w owns 64 of them;
+//   butterflies -> LDS across the wavefronts), scale = max(amax, 1e-10) / 448, h / scale -> e4m3fn.
+// GATED = false (second GEMM): the strip is 256 output columns, wavefront w owns 32 of them;
 //   the bf16 result row is written at its slot (t*K + k), which undoes the permutation.
-#include <stdlib.h>
 #include "moe_common.h"
 #include "moe_layout.h"
 #include "../../include/moe_hip.h"
 
 namespace moe {
-
-// development knob: MOE_HIP_GEMM_VARIANT picks among the compiled launch shapes
-static int gemm_variant() {
-  static int v = -1;
-  if (v < 0) { const char *s = getenv("MOE_HIP_GEMM_VARIANT"); v = s ? atoi(s) : 0; }
-  return v;
-}
 
 struct GemmArgs {
   const uint8_t *aq;            // activations fp8 [rows_a, Kd]
@@ -476,21 +469,15 @@ static int launch_gemm(hipStream_t st, GemmArgs &a, int tile_m, int max_mtiles) 
   if (total <= 0 || total > 0x7fffffffl) return MOE_E_SHAPE;
   a.total_blocks = (int)total;
   dim3 grid((unsigned)total);
-  const int cfg = gemm_variant();
 #define MOE_GEMM(MT, NW, D, WREG) grouped_gemm_kernel<MT, NW, D, GATED, WREG><<<grid, dim3(64 * NW), 0, st>>>(a)
+  // small tiles: both operands through LDS (few registers, deeper pipeline); large tiles: weights in
+  // a register ring so that LDS holds three stages of the bigger token tile
   switch (tile_m) {
     case 16: MOE_GEMM(1, 8, 3, false); break;
     case 32: MOE_GEMM(2, 8, 3, false); break;
     case 64: MOE_GEMM(4, 8, 2, false); break;
-    case 128:
-      if (cfg == 1) MOE_GEMM(8, 4, 2, true);
-      else if (cfg == 2) MOE_GEMM(8, 8, 2, false);
-      else MOE_GEMM(8, 8, 2, true);
-      break;
-    case 192:
-      if (cfg == 3) MOE_GEMM(12, 8, 3, true);
-      else MOE_GEMM(12, 8, 2, true);
-      break;
+    case 128: MOE_GEMM(8, 8, 2, true); break;
+    case 192: MOE_GEMM(12, 8, 2, true); break;
     default: return MOE_E_SHAPE;
   }
 #undef MOE_GEMM

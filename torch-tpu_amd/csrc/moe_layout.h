@@ -2,7 +2,6 @@
 #pragma once
 #include <stddef.h>
 #include <stdint.h>
-#include <stdlib.h>
 
 namespace moe {
 
