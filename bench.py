@@ -131,7 +131,7 @@ def bench_prefill(pkg, moe, cfg, dev, steps, warmup):
     xq, xs = pkg.act_quant(x)
     ss, off, s2r, ws = pkg.moe_permute(ids, E, return_workspace=True)
     hq = torch.empty(T * K, I, dtype=torch.float8_e4m3fn, device=dev)
-    hs = torch.empty(T * K, I // 128, dtype=torch.float32, device=dev)
+    hs = torch.empty(T * K, pkg.scale_pitch(I // 128), dtype=torch.float32, device=dev)
     from torch_tpu_amd._lib import check, lib
     st = torch.cuda.current_stream().cuda_stream
 

@@ -103,9 +103,17 @@ int moe_permute(void *stream, const int32_t *ids, int T, int K, int E,
                 void *workspace, size_t workspace_bytes);
 
 /*
+ * Activation-scale tensors (the s of moe_act_quant, xs / hs of the stage entry points) hold one
+ * fp32 per row and 128-column group, rows padded to moe_scale_pitch(groups) floats - whole
+ * 64-byte pieces, which the grouped GEMMs fetch with single aligned reads.  The padding is never
+ * interpreted.  Base addresses must be 64-byte aligned.
+ */
+int moe_scale_pitch(int n_groups);
+
+/*
  * Per-token, per-128-column dynamic quantisation of bf16 activations.
- * x [R, C] bf16 -> q [R, C] fp8, s [R, C/128] fp32.  No counterpart in the open part of the
- * reference (its W8A8 sibling is closed: torch_tpu/csrc/ops/my_ops/MlpW8A8Quant.cpp:34-46).
+ * x [R, C] bf16 -> q [R, C] fp8, s [R, moe_scale_pitch(C/128)] fp32.  No counterpart in the open
+ * part of the reference (its W8A8 sibling is closed: torch_tpu/csrc/ops/my_ops/MlpW8A8Quant.cpp:34-46).
  */
 int moe_act_quant(void *stream, const void *x_bf16, int R, int C, uint8_t *q, float *s);
 
@@ -137,7 +145,7 @@ int moe_fused_experts_fp8(void *stream,
  * Stages of the above, exposed for tests and for timing one kernel at a time.  All take
  * the permutation produced by moe_permute() and the tile list it leaves in its workspace.
  *
- * moe_gemm1_swiglu:  hq [T*K, I] fp8 / hs [T*K, I/128] fp32 (rows in permuted order)
+ * moe_gemm1_swiglu:  hq [T*K, I] fp8 / hs [T*K, moe_scale_pitch(I/128)] fp32 (rows in permuted order)
  *                    = requant(silu(x W_gate^T) * (x W_up^T)) with xq/xs from moe_act_quant.
  * moe_gemm2:         y [T*K, H] bf16, row of slot s at y[s] (slot order, i.e. [T, K, H]).
  * moe_weighted_reduce: out [T, H] bf16 = sum_k w[t,k] * y[t,k,:] (+ shared_y[t,:] if given).

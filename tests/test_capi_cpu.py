@@ -17,7 +17,7 @@ def declared_symbols():
 
 def test_header_declares_the_expected_entry_points():
     syms = declared_symbols()
-    for s in ["moe_fused_experts_fp8", "moe_noaux_tc_topk", "moe_route_topk", "moe_permute", "moe_act_quant",
+    for s in ["moe_fused_experts_fp8", "moe_noaux_tc_topk", "moe_route_topk", "moe_permute", "moe_scale_pitch", "moe_act_quant",
               "moe_gemm1_swiglu", "moe_gemm2", "moe_weighted_reduce", "moe_hip_version"]:
         assert s in syms
 

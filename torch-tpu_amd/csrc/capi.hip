@@ -45,13 +45,13 @@ static FusedWs fused_layout(void *base, int T, int H, int I, int E, int K, int I
   w.expert_offsets = (int32_t *)take((size_t)(E + 1) * 4);
   w.slot_to_row = (int32_t *)take(TK * 4);
   w.xq = (uint8_t *)take((size_t)T * H);
-  w.xs = (float *)take((size_t)T * (H / kBlock) * 4);
+  w.xs = (float *)take((size_t)T * scale_pitch(H / kBlock) * 4);
   w.hq = (uint8_t *)take(TK * I);
-  w.hs = (float *)take(TK * (I / kBlock) * 4);
+  w.hs = (float *)take(TK * scale_pitch(I / kBlock) * 4);
   w.y = (uint16_t *)take(TK * H * 2);
   if (I_sh > 0) {
     w.sh_hq = (uint8_t *)take((size_t)T * I_sh);
-    w.sh_hs = (float *)take((size_t)T * (I_sh / kBlock) * 4);
+    w.sh_hs = (float *)take((size_t)T * scale_pitch(I_sh / kBlock) * 4);
     w.sh_y = (uint16_t *)take((size_t)T * H * 2);
   }
   w.bytes = off;

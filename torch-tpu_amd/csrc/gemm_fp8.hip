@@ -37,7 +37,7 @@ namespace moe {
 
 struct GemmArgs {
   const uint8_t *aq;            // activations fp8 [rows_a, Kd]
-  const float *as;              // activation scales [rows_a, Kd/128]
+  const float *as;              // activation scales [rows_a, as_pitch] (Kd/128 used columns)
   const uint8_t *w;             // weights fp8 [E, n_rows_w, Kd]
   const float *ws;              // weight scales [E, n_rows_w/128, Kd/128]
   const int32_t *sorted_slot;   // [TK]
@@ -47,6 +47,8 @@ struct GemmArgs {
   uint8_t *hq;                  // GATED: [TK, N] fp8
   float *hs;                    // GATED: [TK, N/128]
   uint16_t *y;                  // !GATED: [TK, N] bf16 in slot order
+  int as_pitch;                 // floats per row of as / sh_as: scale_pitch(Kd/128)
+  int hs_pitch;                 // GATED: floats per row of hs / sh_hs: scale_pitch(N/128)
   int Kd;                       // reduction length (multiple of 128)
   int N;                        // GATED: I (gate columns); !GATED: H
   int n_rows_w;                 // GATED: 2*I; !GATED: H
@@ -71,18 +73,20 @@ struct GemmArgs {
 
 constexpr int kMaxKB = 256;                 // reduction length limit: 256 * 128 = 32768
 
-template <int MT, int NW, int STAGES, int WSTAGES>
+template <int MT, int NW, int STAGES, int WSTAGES, int WTILE = 2048>
 struct GemmSmem {
   static constexpr int BM = 16 * MT;
-  static constexpr int SA = BM < 64 ? 64 : BM;   // the scale DMA always writes 64 lanes
-  alignas(1024) uint8_t wt[WSTAGES][16 * 2048];   // weight tiles: [tile][half][lane][16 bytes], read by their owner
+  alignas(1024) uint8_t wt[WSTAGES][16 * WTILE];   // weight tiles: [tile][half][lane][16 bytes], read by their owner
   alignas(1024) uint8_t tok[STAGES][BM * 128];   // token tiles, XOR-swizzled 16-byte chunks
-  alignas(256) float sa[STAGES][SA];             // activation scales of each staged step
+  alignas(1024) float sac[2][MT * 256];          // activation scales, 16 steps at a time: [m-tile][4-step part][row][4]
   int arow[BM];                                  // source row in aq / as for each tile row
   float amax[NW][BM];                            // GATED epilogue: per-wavefront partial amax
   float sb[2][kMaxKB];                           // weight-block scales of the strip for every 128-step
 };
 
+#ifndef MOE_W_MOD
+#define MOE_W_MOD ""
+#endif
 typedef __attribute__((address_space(3))) uint8_t lds_byte;
 // byte offset of a __shared__ object inside the workgroup's LDS allocation (what M0 wants)
 __device__ __forceinline__ uint32_t lds_offset(const void *p) { return (uint32_t)(uintptr_t)(lds_byte *)p; }
@@ -112,7 +116,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   constexpr int NT = 64 * NW;                         // threads
   constexpr int WT = 16 / NW;                         // weight tiles per wavefront
   constexpr int STAGES = DEPTH + 1;                   // token tiles staged in LDS
-  __shared__ GemmSmem<MT, NW, STAGES, WREG ? 1 : STAGES> sm;
+  __shared__ GemmSmem<MT, NW, STAGES, WREG ? 1 : STAGES, WREG ? 64 : 2048> sm;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -162,6 +166,9 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     const int p = row0 + min(i, rows - 1);
     int src = p;
     if (GATED && !direct) src = a.sorted_slot[p] / a.topk;
+#ifdef MOE_DBG_SAMETOK
+    src = i;
+#endif
     sm.arow[i] = min(max(src, 0), rows_a - 1);
   }
   __syncthreads();
@@ -214,14 +221,25 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     tok_src[u] = 8 * t < rows ? (uint32_t)sm.arow[row] * (uint32_t)a.Kd + c * 16 : (uint32_t)sm.arow[0] * (uint32_t)a.Kd;
     tok_m0[u] = t * 1024;
   }
-  constexpr int NSA = (BM + 63) / 64;                  // 64-row groups of scales
-  const int sa_grp = wave % NSA;
-  const uint32_t sa_src = (uint32_t)sm.arow[min(sa_grp * 64 + lane, BM - 1)] * (uint32_t)NKB * 4u;   // bytes
+  // Activation scales travel 16 steps (64 bytes of a row) at a time: one instruction moves the 16
+  // rows of an m-tile, lane (part, row) fetching 16 bytes = 4 steps, into [part][row][4] order, which
+  // the 16 lanes that later read one step of 16 rows hit in 16 different banks.  Two buffers; the
+  // chunk after the current one is requested when the current one starts.
+  constexpr int NSC = (MT + NW - 1) / NW;              // scale instructions per wavefront and chunk
+  uint32_t sac_src[NSC];
+  uint32_t sac_m0[NSC];
+#pragma unroll
+  for (int u = 0; u < NSC; u++) {
+    const int mt = min(wave + u * NW, MT - 1);
+    sac_src[u] = (uint32_t)sm.arow[mt * 16 + li] * (uint32_t)a.as_pitch * 4u + lg * 16;   // bytes
+    sac_m0[u] = mt * 1024;
+  }
   const uint32_t wt_base = __builtin_amdgcn_readfirstlane(lds_offset(&sm.wt[0][0])) + wave * (WT * 2048);
   constexpr uint32_t kWtStage = 16 * 2048;
   const uint32_t tok_base = __builtin_amdgcn_readfirstlane(lds_offset(&sm.tok[0][0]));
-  const uint32_t sa_base = __builtin_amdgcn_readfirstlane(lds_offset(&sm.sa[0][0])) + sa_grp * 256;
-  constexpr uint32_t kTokStage = BM * 128, kSaStage = sizeof(float) * GemmSmem<MT, NW, STAGES, 1>::SA;
+  const uint32_t sac_base = __builtin_amdgcn_readfirstlane(lds_offset(&sm.sac[0][0]));
+  constexpr uint32_t kTokStage = BM * 128, kSacBuf = MT * 1024;
+  const int n_chunks = (NKB + 15) >> 4;
 
   v4f acc[MT][WT];
 #pragma unroll
@@ -238,19 +256,27 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   //   weights: the wavefront's WT tiles, each as two 1 KB halves laid out [lane][16 bytes] - the
   //            owner reads them back with two linear 128-bit LDS reads per tile;
   //   tokens:  1 KB pieces = 8 rows x 128 bytes, swizzled on the source side.
-  constexpr int L_STEP = NTOK + 1 + 2 * WT;            // loads per wavefront and step
+  constexpr int L_STEP = NTOK + 2 * WT;                // loads per wavefront and step (scale chunks come on top)
   v4i wlo[WREG ? DEPTH : 1][WT], whi[WREG ? DEPTH : 1][WT];   // WREG: weight fragments ride in a register ring
   auto request_weights_reg = [&](int kb, v4i(&lo)[WT], v4i(&hi)[WT]) {
 #pragma unroll
     for (int j = 0; j < WT; j++) {
       const uint8_t *base = wtile[j] + (size_t)kb * 128;
-      asm volatile("global_load_dwordx4 %0, %2, %3\n\tglobal_load_dwordx4 %1, %2, %3 offset:64"
+      asm volatile("global_load_dwordx4 %0, %2, %3" MOE_W_MOD "\n\tglobal_load_dwordx4 %1, %2, %3 offset:64" MOE_W_MOD
                    : "=&v"(lo[j]), "=&v"(hi[j]) : "v"(woff), "s"(base) : "memory");
     }
   };
   auto arrived_weights = [&](v4i(&lo)[WT], v4i(&hi)[WT]) {
 #pragma unroll
     for (int j = 0; j < WT; j++) asm volatile("" : "+v"(lo[j]), "+v"(hi[j]));
+  };
+  auto request_scales = [&](int chunk) {
+#pragma unroll
+    for (int u = 0; u < NSC; u++) {
+      const float *base = as + chunk * 16;
+      const uint32_t m0 = sac_base + (chunk & 1) * kSacBuf + sac_m0[u];
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(sac_src[u]), "s"(base) : "memory", "m0");
+    }
   };
   auto request = [&](int kb, int stage) {
 #pragma unroll
@@ -259,19 +285,14 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
       const uint32_t m0 = tok_base + stage * kTokStage + tok_m0[u];
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(tok_src[u]), "s"(base) : "memory", "m0");
     }
-    {
-      const float *base = as + kb;
-      const uint32_t m0 = sa_base + stage * kSaStage;
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(m0), "v"(sa_src), "s"(base) : "memory", "m0");
-    }
     if (!WREG)
 #pragma unroll
     for (int j = 0; j < WT; j++) {
       const uint8_t *base = wtile[j] + (size_t)kb * 128;
       const uint32_t m0 = wt_base + stage * kWtStage + j * 2048;
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t"
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" MOE_W_MOD "\n\t"
                    // the instruction offset moves the LDS address as well as the global one: 0x400 - 64
-                   "s_add_u32 m0, m0, 0x3c0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:64"
+                   "s_add_u32 m0, m0, 0x3c0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:64" MOE_W_MOD
                    ::"s"(m0), "v"(woff), "s"(base) : "memory", "m0", "scc");
     }
   };
@@ -292,7 +313,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     const float s0 = sm.sb[sb_row0][kb], s1 = sm.sb[sb_row1][kb];
     const uint8_t *tbase = sm.tok[stage] + li * 128;
     const int o0 = (lg ^ (li & 7)) << 4, o1 = ((lg + 4) ^ (li & 7)) << 4;
-    const float *sap = sm.sa[stage] + li;
+    const float *sap = sm.sac[(kb >> 4) & 1] + ((kb & 12) << 4) + li * 4 + (kb & 3);
 #pragma unroll
     for (int mg = 0; mg < MT / MG; mg++) {
       if (mg == 0 || mg * MG < mt_live) {
@@ -302,7 +323,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
         for (int mi = 0; mi < MG; mi++) {
           const int mt = mg * MG + mi;
           x[mi] = concat8(*(const v4i *)(tbase + mt * 2048 + o0), *(const v4i *)(tbase + mt * 2048 + o1));
-          sa_[mi] = sap[mt * 16];
+          sa_[mi] = sap[mt * 256];
         }
         __builtin_amdgcn_sched_barrier(0);
         v4f p[MG][WT];
@@ -335,6 +356,10 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   // share of the token tile is there and everybody is done reading the stage that is reused next |
   // request step kb+DEPTH into that stage | matrix work on stage kb % STAGES.
   // DEPTH-1 whole steps stay in flight across the wait, DEPTH during the matrix work.
+  // Scale chunk c+1 is requested right after the barrier of step 16c: every wavefront has then left
+  // step 16c-1, the last reader of the buffer it goes to, and any later step's wait covers it (a wait
+  // leaves only the (DEPTH-1) youngest steps' loads outstanding, so extra loads make it stricter).
+  request_scales(0);
   if (!WREG) {
 #pragma unroll
     for (int d = 0; d < DEPTH; d++) request(min(d, NKB - 1), d);
@@ -342,6 +367,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     for (; kb + DEPTH < NKB; kb++) {
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 1) * L_STEP) : "memory");
       __syncthreads();
+      if ((kb & 15) == 0 && (kb >> 4) + 1 < n_chunks) request_scales((kb >> 4) + 1);
       request(kb + DEPTH, stage_req);
       compute(stage, kb, wlo[0], whi[0]);
       stage = stage + 1 == STAGES ? 0 : stage + 1;
@@ -357,7 +383,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     // weights in a register ring (slot kb % DEPTH; loop unrolled by DEPTH so slots are compile-time):
     // the token request of step kb+DEPTH goes out before the matrix work of step kb, the weight
     // request after it, into the slot that work has just read
-    constexpr int L_TOKS = NTOK + 1;
+    constexpr int L_TOKS = NTOK;
 #pragma unroll
     for (int d = 0; d < DEPTH; d++) {
       request(min(d, NKB - 1), d);
@@ -370,12 +396,21 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
         const int kb = kb0 + d;
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 1) * (L_TOKS + 2 * WT)) : "memory");
         arrived_weights(wlo[d], whi[d]);
+#ifndef MOE_DBG_NOBARRIER
         __syncthreads();
+#endif
+        if ((kb & 15) == 0 && (kb >> 4) + 1 < n_chunks) request_scales((kb >> 4) + 1);
+#if !defined(MOE_DBG_NOLOAD) && !defined(MOE_DBG_NOTOK)
         request(kb + DEPTH, (kb + DEPTH) % STAGES);
+#endif
         __builtin_amdgcn_sched_barrier(0);
+#ifndef MOE_DBG_NOCOMPUTE
         compute(kb % STAGES, kb, wlo[d], whi[d]);
+#endif
         __builtin_amdgcn_sched_barrier(0);
+#if !defined(MOE_DBG_NOLOAD) && !defined(MOE_DBG_NOW)
         request_weights_reg(kb + DEPTH, wlo[d], whi[d]);
+#endif
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -420,7 +455,6 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
       if (lg == 0) sm.amax[wave][mt * 16 + li] = m;
     }
     __syncthreads();
-    const int n_grp = a.N >> 7;
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
       const int i = mt * 16 + li;
@@ -435,7 +469,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
         const uint32_t packed = pack4_fp8(acc[mt][j][0] / sc, acc[mt][j][1] / sc, acc[mt][j][2] / sc, acc[mt][j][3] / sc);
         if (valid) *(uint32_t *)((shared ? a.sh_hq : a.hq) + orow * a.N + strip * 128 + wave * (16 * G) + j * 16 + lg * 4) = packed;
       }
-      if (valid && wave == 0 && lg == 0) (shared ? a.sh_hs : a.hs)[orow * n_grp + strip] = sc;
+      if (valid && wave == 0 && lg == 0) (shared ? a.sh_hs : a.hs)[orow * a.hs_pitch + strip] = sc;
     }
   } else {
 #pragma unroll
@@ -477,7 +511,10 @@ static int launch_gemm(hipStream_t st, GemmArgs &a, int tile_m, int max_mtiles) 
     case 32: MOE_GEMM(2, 8, 3, false); break;
     case 64: MOE_GEMM(4, 8, 2, false); break;
     case 128: MOE_GEMM(8, 8, 2, true); break;
-    case 192: MOE_GEMM(12, 8, 2, true); break;
+    #ifndef MOE_D192
+#define MOE_D192 2
+#endif
+    case 192: MOE_GEMM(12, 8, MOE_D192, true); break;
     default: return MOE_E_SHAPE;
   }
 #undef MOE_GEMM
@@ -504,6 +541,7 @@ int gemm1_launch(hipStream_t st, const uint8_t *xq, const float *xs, int T, int 
   a.sorted_slot = sorted_slot; a.expert_offsets = expert_offsets;
   a.tile_prefix = pw ? pw->tile_prefix : nullptr; a.tile_expert = pw ? pw->tile_expert : nullptr;
   a.hq = hq; a.hs = hs; a.y = nullptr;
+  a.as_pitch = scale_pitch(H / kBlock); a.hs_pitch = scale_pitch(I / kBlock);
   a.Kd = H; a.N = I; a.n_rows_w = 2 * I; a.rows_a = T; a.topk = K; a.E = E; a.fixed_expert = fixed_expert;
   const int tile_m = choose_tile_m(T, K, E);
   const int max_mtiles = fixed_expert >= 0 ? (T + tile_m - 1) / tile_m : pw->max_tiles;
@@ -520,6 +558,7 @@ int gemm2_launch(hipStream_t st, const uint8_t *hq, const float *hs, int rows_a,
   a.sorted_slot = sorted_slot; a.expert_offsets = expert_offsets;
   a.tile_prefix = pw ? pw->tile_prefix : nullptr; a.tile_expert = pw ? pw->tile_expert : nullptr;
   a.hq = nullptr; a.hs = nullptr; a.y = y;
+  a.as_pitch = scale_pitch(I / kBlock); a.hs_pitch = 0;
   a.Kd = I; a.N = H; a.n_rows_w = H; a.rows_a = rows_a; a.topk = K; a.E = E; a.fixed_expert = fixed_expert;
   const int tile_m = choose_tile_m(T, K, E);
   const int max_mtiles = fixed_expert >= 0 ? (rows_a + tile_m - 1) / tile_m : pw->max_tiles;
@@ -536,7 +575,8 @@ extern "C" int moe_gemm1_swiglu(void *stream, const uint8_t *xq, const float *xs
     return MOE_E_NULL;
   int rc = check_dims(T, H, I, E, K);
   if (rc) return rc;
-  if (((uintptr_t)xq % 16) || ((uintptr_t)w13 % 16) || ((uintptr_t)hq % 4)) return MOE_E_ALIGN;
+  if (((uintptr_t)xq % 16) || ((uintptr_t)w13 % 16) || ((uintptr_t)hq % 4) || ((uintptr_t)xs % 64) || ((uintptr_t)hs % 64))
+    return MOE_E_ALIGN;
   if (T == 0) return MOE_OK;
   PermuteWs pw = permute_ws_layout(const_cast<void *>(permute_workspace), T, K, E);
   return gemm1_launch((hipStream_t)stream, xq, xs, T, H, w13, w13_scale, I, E, K, sorted_slot, expert_offsets, &pw, -1,
@@ -551,7 +591,7 @@ extern "C" int moe_gemm2(void *stream, const uint8_t *hq, const float *hs, int T
     return MOE_E_NULL;
   int rc = check_dims(T, H, I, E, K);
   if (rc) return rc;
-  if (((uintptr_t)hq % 16) || ((uintptr_t)w2 % 16) || ((uintptr_t)y_bf16 % 8)) return MOE_E_ALIGN;
+  if (((uintptr_t)hq % 16) || ((uintptr_t)w2 % 16) || ((uintptr_t)y_bf16 % 8) || ((uintptr_t)hs % 64)) return MOE_E_ALIGN;
   if (T == 0) return MOE_OK;
   PermuteWs pw = permute_ws_layout(const_cast<void *>(permute_workspace), T, K, E);
   return gemm2_launch((hipStream_t)stream, hq, hs, T * K, T, H, w2, w2_scale, I, E, K, sorted_slot, expert_offsets, &pw,

@@ -9,6 +9,10 @@ constexpr int kChunk = 256;   // slots ranked by one wavefront in the permutatio
 
 static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
+// Rows of an activation-scale tensor are padded to whole 64-byte pieces: the grouped GEMMs fetch
+// the scales of 16 reduction steps of a row with one aligned 64-byte read.
+static inline int scale_pitch(int n_groups) { return (n_groups + 15) & ~15; }
+
 // Rows of one expert that a grouped-GEMM workgroup owns.  A pure function of the problem
 // shape so that the permutation (which builds the tile list) and the GEMM launchers agree
 // without passing it around.  A token's K experts are distinct, so no expert ever holds

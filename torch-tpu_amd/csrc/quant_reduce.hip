@@ -3,13 +3,15 @@
 //   weighted_reduce  bf16 [T, K, H] per-slot results -> bf16 [T, H], fp32 weighted sum
 // Both move 16 bytes per lane per access; rows are contiguous so every access is coalesced.
 #include "moe_common.h"
+#include "moe_layout.h"
 #include "../../include/moe_hip.h"
 
 namespace moe {
 
 // 16 lanes share one 128-column group: 8 bf16 per lane.
 __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t *__restrict__ x, size_t n_groups,
-                                                        uint8_t *__restrict__ q, float *__restrict__ s) {
+                                                        int groups_per_row, int pitch, uint8_t *__restrict__ q,
+                                                        float *__restrict__ s) {
   const size_t g = ((size_t)blockIdx.x * 256 + threadIdx.x) >> 4;
   const int sub = threadIdx.x & 15;
   const bool live = g < n_groups;
@@ -33,7 +35,7 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t *__restri
   out[0] = (int)pack4_fp8(f[0] / sc, f[1] / sc, f[2] / sc, f[3] / sc);
   out[1] = (int)pack4_fp8(f[4] / sc, f[5] / sc, f[6] / sc, f[7] / sc);
   *(v2i *)(q + g * kBlock + sub * 8) = out;
-  if (sub == 0) s[g] = sc;
+  if (sub == 0) s[(g / groups_per_row) * pitch + g % groups_per_row] = sc;
 }
 
 // One lane produces 8 consecutive columns of one token.
@@ -76,17 +78,20 @@ __global__ __launch_bounds__(256) void weighted_reduce_kernel(const uint16_t *__
 
 }  // namespace moe
 
+extern "C" int moe_scale_pitch(int n_groups) { return n_groups < 0 ? 0 : moe::scale_pitch(n_groups); }
+
 extern "C" int moe_act_quant(void *stream, const void *x_bf16, int R, int C, uint8_t *q, float *s) {
   using namespace moe;
   if (!x_bf16 || !q || !s) return MOE_E_NULL;
   if (R < 0 || C < 1) return MOE_E_SHAPE;
   if (C % kBlock) return MOE_E_ALIGN;
-  if (((uintptr_t)x_bf16 % 16) || ((uintptr_t)q % 8) || ((uintptr_t)s % 4)) return MOE_E_ALIGN;
+  if (((uintptr_t)x_bf16 % 16) || ((uintptr_t)q % 8) || ((uintptr_t)s % 64)) return MOE_E_ALIGN;
   const size_t groups = (size_t)R * (C / kBlock);
   if (groups == 0) return MOE_OK;
   const size_t blocks = (groups * 16 + 255) / 256;
   if (blocks > 0x7fffffffull) return MOE_E_SHAPE;
-  act_quant_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>((const uint16_t *)x_bf16, groups, q, s);
+  act_quant_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>((const uint16_t *)x_bf16, groups, C / kBlock,
+                                                                      scale_pitch(C / kBlock), q, s);
   return (int)hipGetLastError();
 }
 

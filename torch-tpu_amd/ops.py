@@ -108,12 +108,37 @@ def moe_permute(ids, num_experts: int, return_workspace: bool = False):
 
 
 # --------------------------------------------------------------------------- quantisation
+def scale_pitch(n_groups: int) -> int:
+    """Floats per row of an activation-scale tensor holding n_groups scales per row."""
+    return lib.moe_scale_pitch(n_groups)
+
+
+def _new_scales(rows: int, n_groups: int, device):
+    """[rows, n_groups] fp32 view of a freshly allocated row-padded scale tensor."""
+    return torch.empty(rows, scale_pitch(n_groups), dtype=torch.float32, device=device)[:, :n_groups]
+
+
+def _scales(t: torch.Tensor, name: str):
+    """Device address of a scale tensor in the row-padded layout the kernels read; a tensor in any
+    other layout is copied into a padded one first (returned so that it stays alive)."""
+    _need(isinstance(t, torch.Tensor) and t.is_cuda and t.dim() == 2, f"{name} must be a 2-d GPU tensor")
+    _need(t.dtype == torch.float32, f"{name} must be float32")
+    rows, n = t.shape
+    pitch = scale_pitch(n)
+    room = t.untyped_storage().nbytes() - t.storage_offset() * 4 >= rows * pitch * 4
+    if not (t.stride(1) == 1 and (rows <= 1 or t.stride(0) == pitch) and t.data_ptr() % 64 == 0 and room):
+        padded = _new_scales(rows, n, t.device)
+        padded.copy_(t)
+        t = padded
+    return t.data_ptr(), t
+
+
 def act_quant(x):
-    """bf16 [R, C] -> (e4m3fn [R, C], fp32 scales [R, C/128])."""
+    """bf16 [R, C] -> (e4m3fn [R, C], fp32 scales [R, C/128]: a view of a row-padded tensor)."""
     _need(x.dim() == 2, "x must be [R, C]")
     R, C = x.shape
     q = torch.empty(R, C, dtype=_FP8, device=x.device)
-    s = torch.empty(R, C // 128, dtype=torch.float32, device=x.device)
+    s = _new_scales(R, C // 128, x.device)
     rc = lib.moe_act_quant(_stream(), _dev(x, "x", torch.bfloat16), R, C, q.data_ptr(), s.data_ptr())
     check(rc, "act_quant")
     return q, s
@@ -186,8 +211,9 @@ def gemm1_swiglu(xq, xs, w13, w13_scale, ids_shape, sorted_slot, offsets, permut
     E, I2, H = w13.shape
     I = I2 // 2
     hq = torch.empty(T * K, I, dtype=_FP8, device=xq.device)
-    hs = torch.empty(T * K, I // 128, dtype=torch.float32, device=xq.device)
-    rc = lib.moe_gemm1_swiglu(_stream(), _dev(xq, "xq", _FP8), _dev(xs, "xs", torch.float32), T, H,
+    hs = _new_scales(T * K, I // 128, xq.device)
+    xs_ptr, xs = _scales(xs, "xs")
+    rc = lib.moe_gemm1_swiglu(_stream(), _dev(xq, "xq", _FP8), xs_ptr, T, H,
                               _dev(w13, "w13", _FP8), _dev(w13_scale, "w13_scale", torch.float32), I, E, K,
                               _dev(sorted_slot, "sorted_slot", torch.int32), _dev(offsets, "offsets", torch.int32),
                               _dev(permute_ws, "permute_ws"), hq.data_ptr(), hs.data_ptr())
@@ -201,7 +227,8 @@ def gemm2(hq, hs, w2, w2_scale, ids_shape, sorted_slot, offsets, permute_ws, y=N
     E, H, I = w2.shape
     if y is None:
         y = torch.empty(T, K, H, dtype=torch.bfloat16, device=hq.device)
-    rc = lib.moe_gemm2(_stream(), _dev(hq, "hq", _FP8), _dev(hs, "hs", torch.float32), T, H,
+    hs_ptr, hs = _scales(hs, "hs")
+    rc = lib.moe_gemm2(_stream(), _dev(hq, "hq", _FP8), hs_ptr, T, H,
                        _dev(w2, "w2", _FP8), _dev(w2_scale, "w2_scale", torch.float32), I, E, K,
                        _dev(sorted_slot, "sorted_slot", torch.int32), _dev(offsets, "offsets", torch.int32),
                        _dev(permute_ws, "permute_ws"), _dev(y, "y", torch.bfloat16))
