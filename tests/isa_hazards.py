@@ -53,6 +53,10 @@ def hazards(body, max_states=24):
         if l.startswith("."):
             continue
         blocks[cur].append(l.split(";")[0].strip())
+        if l.startswith(("s_cbranch", "s_branch", "s_endpgm")):     # unlabelled fall-through block
+            cur = f"{cur}+"
+            blocks[cur] = []
+            order.append(cur)
     succ = {}
     for n, b in enumerate(order):
         out, fall = [], True

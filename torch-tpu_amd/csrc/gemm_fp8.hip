@@ -29,6 +29,7 @@
 //   butterflies -> LDS across the wavefronts), scale = max(amax, 1e-10) / 448, h / scale -> e4m3fn.
 // GATED = false (second GEMM): the strip is 256 output columns, wavefront w owns 32 of them;
 //   the bf16 result row is written at its slot (t*K + k), which undoes the permutation.
+#include <type_traits>
 #include "moe_common.h"
 #include "moe_layout.h"
 #include "../../include/moe_hip.h"
@@ -81,7 +82,7 @@ struct GemmSmem {
   alignas(1024) float sac[2][MT * 256];          // activation scales, 16 steps at a time: [m-tile][4-step part][row][4]
   int arow[BM];                                  // source row in aq / as for each tile row
   float amax[NW][BM];                            // GATED epilogue: per-wavefront partial amax
-  float sb[2][kMaxKB];                           // weight-block scales of the strip for every 128-step
+  float sb[2][kMaxKB + 4];                       // weight-block scales of the strip for every 128-step, then zeros
 };
 
 #ifndef MOE_W_MOD
@@ -115,7 +116,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   constexpr int BM = 16 * MT;
   constexpr int NT = 64 * NW;                         // threads
   constexpr int WT = 16 / NW;                         // weight tiles per wavefront
-  constexpr int STAGES = DEPTH + 1;                   // token tiles staged in LDS
+  constexpr int STAGES = WREG ? 4 : DEPTH + 1;        // token tiles staged in LDS
   __shared__ GemmSmem<MT, NW, STAGES, WREG ? 1 : STAGES, WREG ? 64 : 2048> sm;
 
   const int tid = threadIdx.x;
@@ -200,6 +201,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
       const int r = i >= NKB, kb = i - r * NKB;
       sm.sb[r][kb] = ws[((size_t)e * n_wblk + (r ? blk1 : blk0)) * NKB + kb];
     }
+    if (tid < 8) sm.sb[tid >> 2][NKB + (tid & 3)] = 0.f;
   }
   const int sb_row0 = GATED ? 0 : (wave * WT) / 8;      // which of the two rows this wavefront's tiles use
   const int sb_row1 = GATED ? 1 : sb_row0;
@@ -360,7 +362,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   // step 16c-1, the last reader of the buffer it goes to, and any later step's wait covers it (a wait
   // leaves only the (DEPTH-1) youngest steps' loads outstanding, so extra loads make it stricter).
   request_scales(0);
-  if (!WREG) {
+  if constexpr (!WREG) {
 #pragma unroll
     for (int d = 0; d < DEPTH; d++) request(min(d, NKB - 1), d);
     int kb = 0, stage = 0, stage_req = DEPTH;
@@ -380,59 +382,138 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
       stage = stage + 1 == STAGES ? 0 : stage + 1;
     }
   } else {
-    // weights in a register ring (slot kb % DEPTH; loop unrolled by DEPTH so slots are compile-time):
-    // the token request of step kb+DEPTH goes out before the matrix work of step kb, the weight
-    // request after it, into the slot that work has just read
-    constexpr int L_TOKS = NTOK;
+    // Large tiles: weights in a register ring of two steps, token tiles three steps ahead through
+    // four LDS stages, and ONE software pipeline over all m-tiles of all steps: the LDS reads of
+    // m-tile g+2 and the scale multiply-adds of m-tile g-1 are issued around the matrix
+    // instructions of m-tile g, across step boundaries.  For that the token tile of step s+1 is
+    // made visible (wait + barrier) one step early, at the top of step s.  Per step and wavefront
+    // the loads go out in a fixed order - token tile of step s+3 at the top, weights of step s+2
+    // at the end - so the wait at the top of step s+1 leaves exactly those two requests in flight.
+    // Requests past the last step re-read it (cheap cache hits) instead of branching; a step past
+    // an odd count multiplies by the zero weight scale stored behind the table.  The loop body is
+    // instantiated per number of live m-tiles, so there is no branch between matrix instructions.
+    static_assert(DEPTH == 2 || DEPTH == 3, "the register ring holds two or three steps");
+    constexpr int R = DEPTH;                             // ring slots = steps per pass of the unrolled loop
+    constexpr int XB = R == 2 ? 4 : 3;                   // token operand buffers; R * LIVE is a multiple of it
+    constexpr int L_WAIT = NTOK + 2 * WT * (R - 1);      // loads younger than the ones a step boundary needs
+    const int last = NKB - 1;
+    const int o0 = (lg ^ (li & 7)) << 4, o1 = ((lg + 4) ^ (li & 7)) << 4;
+    auto run = [&](auto live_c) {
+      constexpr int LIVE = decltype(live_c)::value;
+      static_assert(LIVE % 2 == 0 && LIVE >= 2 && LIVE <= MT, "live m-tiles come in pairs");
+      constexpr int PD = 2;                              // m-tiles between an LDS read and its use
+      // the first requests go out inside the instantiation: no branch may sit between a register
+      // load's request and its wait (the compiler would copy the registers while the load is in flight)
+      request(0, 0);
+      request(min(1, last), 1);
+      request_weights_reg(0, wlo[0], whi[0]);
+      request(min(2, last), 2);
 #pragma unroll
-    for (int d = 0; d < DEPTH; d++) {
-      request(min(d, NKB - 1), d);
-      request_weights_reg(min(d, NKB - 1), wlo[d], whi[d]);
-    }
-    int kb0 = 0;
-    for (; kb0 + 2 * DEPTH <= NKB; kb0 += DEPTH) {
+      for (int d = 1; d < R; d++) request_weights_reg(min(d, last), wlo[d], whi[d]);
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(L_WAIT) : "memory");
+      arrived_weights(wlo[0], whi[0]);
+      __syncthreads();
+      if (n_chunks > 1) request_scales(1);
+      request(min(3, last), 3);
+      auto read_x = [&](int kb, int mt) {
+        const uint8_t *t = sm.tok[kb & 3] + li * 128 + mt * 2048;
+        return concat8(*(const v4i *)(t + o0), *(const v4i *)(t + o1));
+      };
+      auto read_sa = [&](int kb, int mt) {
+        kb = min(kb, last);                              // a step past the end: any finite scale (times zero)
+        return sm.sac[(kb >> 4) & 1][mt * 256 + ((kb & 12) << 4) + li * 4 + (kb & 3)];
+      };
+      v8i x[XB];
+      float sa_[XB], sc[R][2], f_[2][2];
+      v4f p[2][WT];
 #pragma unroll
-      for (int d = 0; d < DEPTH; d++) {
-        const int kb = kb0 + d;
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 1) * (L_TOKS + 2 * WT)) : "memory");
-        arrived_weights(wlo[d], whi[d]);
-#ifndef MOE_DBG_NOBARRIER
-        __syncthreads();
-#endif
-        if ((kb & 15) == 0 && (kb >> 4) + 1 < n_chunks) request_scales((kb >> 4) + 1);
-#if !defined(MOE_DBG_NOLOAD) && !defined(MOE_DBG_NOTOK)
-        request(kb + DEPTH, (kb + DEPTH) % STAGES);
-#endif
-        __builtin_amdgcn_sched_barrier(0);
-#ifndef MOE_DBG_NOCOMPUTE
-        compute(kb % STAGES, kb, wlo[d], whi[d]);
-#endif
-        __builtin_amdgcn_sched_barrier(0);
-#if !defined(MOE_DBG_NOLOAD) && !defined(MOE_DBG_NOW)
-        request_weights_reg(kb + DEPTH, wlo[d], whi[d]);
-#endif
-        __builtin_amdgcn_sched_barrier(0);
+      for (int q = 0; q < PD; q++) {
+        const int qq = q < LIVE ? q : q - LIVE, kk = q < LIVE ? 0 : 1;
+        x[q] = read_x(kk, LIVE - 1 - qq); sa_[q] = read_sa(kk, LIVE - 1 - qq);
       }
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      sc[0][0] = sm.sb[sb_row0][0]; sc[0][1] = sm.sb[sb_row1][0];
+      // the multiply-add slot of the very first m-tile adds zero
 #pragma unroll
-    for (int d = 0; d < DEPTH; d++) arrived_weights(wlo[d], whi[d]);
-    for (; kb0 < NKB; kb0 += DEPTH) {
+      for (int j = 0; j < WT; j++) p[1][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+      f_[1][0] = f_[1][1] = 0.f;
+      for (int s0 = 0; s0 < NKB; s0 += R) {
 #pragma unroll
-      for (int d = 0; d < DEPTH; d++) {
-        const int kb = kb0 + d;
-        if (kb < NKB) {
+        for (int h = 0; h < R; h++) {
+          const int kb = s0 + h;
+          sc[(h + 1) % R][0] = sm.sb[sb_row0][kb + 1]; sc[(h + 1) % R][1] = sm.sb[sb_row1][kb + 1];
+          v8i wc[WT];
+#pragma unroll
+          for (int j = 0; j < WT; j++) wc[j] = concat8(wlo[h][j], whi[h][j]);
+          // one m-tile: LDS reads two m-tiles ahead, its matrix instructions, then the multiply-adds
+          // of the m-tile before it (tp), whose products are complete by now
+          // m-tiles are walked from the last live one down to 0 so that the m-tile whose products are
+          // still pending at a step boundary is m-tile 0 whatever the number of live m-tiles
+          auto tile = [&](int q, int tp) {
+            const int g = h * LIVE + q;                  // position in the R-step pattern
+            {
+              const int qq = q + PD < LIVE ? q + PD : q + PD - LIVE;
+              const int kk = q + PD < LIVE ? kb : kb + 1;
+              x[(g + PD) % XB] = read_x(kk, LIVE - 1 - qq);
+              sa_[(g + PD) % XB] = read_sa(kk, LIVE - 1 - qq);
+            }
+#pragma unroll
+            for (int j = 0; j < WT; j++) {
+              const v4f zero = {0.f, 0.f, 0.f, 0.f};
+              p[g & 1][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wc[j], x[g % XB], zero, 0, 0, 0, 0, 0, 0);
+            }
+            f_[g & 1][0] = sa_[g % XB] * sc[h][0];
+            f_[g & 1][1] = sa_[g % XB] * sc[h][1];
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < WT; j++) {
+              const float f = (GATED && j >= WT / 2) ? f_[(g + 1) & 1][1] : f_[(g + 1) & 1][0];
+#pragma unroll
+              for (int r = 0; r < 4; r++) acc[tp][j][r] = fmaf(p[(g + 1) & 1][j][r], f, acc[tp][j][r]);
+              // pins the multiply-adds here: without it they are sunk below the whole step's matrix
+              // instructions, whose results then all stay live
+              asm volatile("" : "+v"(acc[tp][j]));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          };
+#ifndef MOE_DBG_NOCOMPUTE
+          tile(0, 0);
+#pragma unroll
+          for (int q = 1; q < LIVE; q++) tile(q, LIVE - q);
+#endif
+          // top of step kb + 1
+#if !defined(MOE_DBG_NOLOAD) && !defined(MOE_DBG_NOW)
+          request_weights_reg(min(kb + R, last), wlo[h], whi[h]);
+#endif
+          asm volatile("s_waitcnt vmcnt(%0)" ::"n"(L_WAIT) : "memory");
+          arrived_weights(wlo[(h + 1) % R], whi[(h + 1) % R]);
           __syncthreads();
-          compute(kb % STAGES, kb, wlo[d], whi[d]);
-          if (kb + DEPTH < NKB) {
-            request(kb + DEPTH, (kb + DEPTH) % STAGES);
-            request_weights_reg(kb + DEPTH, wlo[d], whi[d]);
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            arrived_weights(wlo[d], whi[d]);
-          }
+          if (((kb + 1) & 15) == 0 && ((kb + 1) >> 4) + 1 < n_chunks) request_scales(((kb + 1) >> 4) + 1);
+#if !defined(MOE_DBG_NOLOAD) && !defined(MOE_DBG_NOTOK)
+          request(min(kb + 4, last), kb & 3);
+#endif
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
-    }
+      // the requests past the last step are still in flight: they land before anything else happens
+      // (their registers and LDS stages must not be reused under them)
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int d = 0; d < R; d++) arrived_weights(wlo[d], whi[d]);
+      // m-tile 0 of the last step is still pending
+#pragma unroll
+      for (int j = 0; j < WT; j++) {
+        const float f = (GATED && j >= WT / 2) ? f_[1][1] : f_[1][0];
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[0][j][r] = fmaf(p[1][j][r], f, acc[0][j][r]);
+      }
+    };
+    auto pick = [&](auto self, auto live_c) -> void {
+      constexpr int LIVE = decltype(live_c)::value;
+      if constexpr (LIVE >= MT) run(std::integral_constant<int, MT>{});
+      else if (mt_live <= LIVE) run(live_c);
+      else self(self, std::integral_constant<int, LIVE + 2>{});
+    };
+    pick(pick, std::integral_constant<int, 2>{});
   }
   __syncthreads();
 
