@@ -136,23 +136,46 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   if ((int)(blockIdx.x >> 3) >= per_xcd) return;
   const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (logical >= n_work) return;
-  const int mtile = logical / a.n_strips;
-  const int strip = logical - mtile * a.n_strips;
-  int e, row0, rows;                                  // expert, first permuted row, rows in tile
-  const bool shared = mtile >= n_routed;              // a tile of the shared expert
+  // Inside one expert the (row tile, strip) pairs are walked in blocks of up to kBlockM row tiles x
+  // kBlockS strips, so that the ~32 workgroups an XCD runs at a time share a few token tiles and a few
+  // weight strips through its L2 instead of streaming 32 different strips.
+  constexpr int kBlockM = 6, kBlockS = 5;
+  const int g0 = logical / a.n_strips;                // some row tile of the expert this work item is in
+  int e, first_mtile, n_mt;                           // expert, its first row tile, its row tiles
+  const bool shared = g0 >= n_routed;                 // a tile of the shared expert
   const bool direct = shared || a.fixed_expert >= 0;  // rows are taken in order, no permutation
   if (shared) {
-    e = 0;
+    e = 0; first_mtile = n_routed; n_mt = n_mtiles - n_routed;
+  } else if (a.fixed_expert >= 0) {
+    e = a.fixed_expert; first_mtile = 0; n_mt = n_routed;
+  } else {
+    e = a.tile_expert[g0];
+    if (e < 0 || e >= a.E) return;
+    first_mtile = a.tile_prefix[e];
+    n_mt = min(a.tile_prefix[e + 1], a.max_mtiles) - first_mtile;
+  }
+  int mtile, strip;
+  {
+    const int local = logical - first_mtile * a.n_strips;
+    const int mb = local / (kBlockM * a.n_strips);
+    const int r1 = local - mb * kBlockM * a.n_strips;
+    const int hm = min(kBlockM, n_mt - kBlockM * mb);
+    if (hm <= 0) return;
+    const int sb = r1 / (hm * kBlockS);
+    const int r2 = r1 - sb * hm * kBlockS;
+    const int w = min(kBlockS, a.n_strips - kBlockS * sb);
+    mtile = first_mtile + kBlockM * mb + r2 / w;
+    strip = kBlockS * sb + r2 % w;
+  }
+  int row0, rows;                                     // first permuted row, rows in tile
+  if (shared) {
     row0 = (mtile - n_routed) * BM;
     rows = min(BM, a.sh_rows - row0);
   } else if (a.fixed_expert >= 0) {
-    e = a.fixed_expert;
     row0 = mtile * BM;
     rows = min(BM, a.rows_a - row0);
   } else {
-    e = a.tile_expert[mtile];
-    if (e < 0 || e >= a.E) return;
-    row0 = a.expert_offsets[e] + (mtile - a.tile_prefix[e]) * BM;
+    row0 = a.expert_offsets[e] + (mtile - first_mtile) * BM;
     rows = min(BM, a.expert_offsets[e + 1] - row0);
   }
   const uint8_t *const aq = shared ? a.sh_aq : a.aq;
