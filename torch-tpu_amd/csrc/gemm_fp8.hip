@@ -81,6 +81,7 @@ struct GemmSmem {
   alignas(1024) uint8_t tok[STAGES][BM * 128];   // token tiles, XOR-swizzled 16-byte chunks
   alignas(1024) float sac[2][MT * 256];          // activation scales, 16 steps at a time: [m-tile][4-step part][row][4]
   int arow[BM];                                  // source row in aq / as for each tile row
+  int oslot[BM];                                 // second GEMM: output row of each tile row
   float amax[NW][BM];                            // GATED epilogue: per-wavefront partial amax
   float sb[2][kMaxKB + 4];                       // weight-block scales of the strip for every 128-step, then zeros
 };
@@ -194,6 +195,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     src = i;
 #endif
     sm.arow[i] = min(max(src, 0), rows_a - 1);
+    if (!GATED) sm.oslot[i] = direct ? p : a.sorted_slot[p];      // output row (slot) of each tile row
   }
   __syncthreads();
 
@@ -580,12 +582,15 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     for (int mt = 0; mt < MT; mt++) {
       const int i = mt * 16 + li;
       const bool valid = i < rows;
-      int slot = row0 + min(i, rows - 1);
-      if (!direct) slot = a.sorted_slot[slot];
+      const int slot = sm.oslot[i];
 #pragma unroll
       for (int j = 0; j < WT; j++) {
         const int col = strip * 256 + wave * (16 * WT) + j * 16 + lg * 4;
+#ifdef MOE_DBG_NOSTORE
+        if (valid && col < 0) {
+#else
         if (valid && col < a.N) {
+#endif
           v2i o;
           o[0] = (int)((uint32_t)f32_to_bf16(acc[mt][j][0]) | ((uint32_t)f32_to_bf16(acc[mt][j][1]) << 16));
           o[1] = (int)((uint32_t)f32_to_bf16(acc[mt][j][2]) | ((uint32_t)f32_to_bf16(acc[mt][j][3]) << 16));

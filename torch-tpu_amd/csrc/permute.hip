@@ -6,9 +6,9 @@
 //   scan     one workgroup: per expert, running sum over the chunks (turns the histogram into
 //            the chunk's starting rank inside its expert), then an exclusive scan over the
 //            experts -> expert_offsets, and the list of row tiles the GEMMs walk.
-//   scatter  one wavefront per chunk again: ranks its slots in slot order with a ballot
-//            "match-any" loop, so equal experts keep their original order (stable), and writes
-//            sorted_slot / slot_to_row.
+//   scatter  one workgroup per chunk, one wavefront per 64 slots: ranks its slots in slot order
+//            with a ballot "match-any" loop, so equal experts keep their original order (stable),
+//            and writes sorted_slot / slot_to_row.
 // A problem of at most kChunk slots is done by one workgroup in a single launch.
 #include "moe_common.h"
 #include "moe_layout.h"
@@ -88,10 +88,18 @@ __global__ __launch_bounds__(1024) void permute_scan_kernel(int32_t *__restrict_
   const int e = threadIdx.x;
   int count = 0;
   if (e < E) {
-    for (int c = 0; c < n_chunks; c++) {
-      int x = chunk_counts[(size_t)c * E + e];
-      chunk_counts[(size_t)c * E + e] = count;   // rank of the chunk's first slot inside expert e
-      count += x;
+    // sixteen independent loads at a time (a load-add-store chain per chunk would pay one memory
+    // round trip per chunk)
+    constexpr int B = 16;
+    for (int c0 = 0; c0 < n_chunks; c0 += B) {
+      int x[B];
+#pragma unroll
+      for (int i = 0; i < B; i++) x[i] = c0 + i < n_chunks ? chunk_counts[(size_t)(c0 + i) * E + e] : 0;
+#pragma unroll
+      for (int i = 0; i < B; i++) {
+        if (c0 + i < n_chunks) chunk_counts[(size_t)(c0 + i) * E + e] = count;   // rank of the chunk's first slot inside expert e
+        count += x[i];
+      }
     }
   }
   int total;
@@ -110,31 +118,39 @@ __global__ __launch_bounds__(1024) void permute_scan_kernel(int32_t *__restrict_
   }
 }
 
-__global__ __launch_bounds__(64) void permute_scatter_kernel(const int32_t *__restrict__ ids, int TK, int E,
-                                                             const int32_t *__restrict__ chunk_counts,
-                                                             const int32_t *__restrict__ expert_offsets,
-                                                             int32_t *__restrict__ sorted_slot,
-                                                             int32_t *__restrict__ slot_to_row) {
+// One workgroup per chunk, one wavefront per 64 consecutive slots of it: every wavefront ranks its
+// slots among themselves, leaves its per-expert counts in LDS, and adds the counts of the
+// wavefronts before it - all slots of the chunk are placed in one round.
+__global__ __launch_bounds__(kChunk) void permute_scatter_kernel(const int32_t *__restrict__ ids, int TK, int E,
+                                                                 const int32_t *__restrict__ chunk_counts,
+                                                                 const int32_t *__restrict__ expert_offsets,
+                                                                 int32_t *__restrict__ sorted_slot,
+                                                                 int32_t *__restrict__ slot_to_row) {
+  constexpr int NWV = kChunk / 64;
   __shared__ int base[MOE_MAX_EXPERTS];
-  const int lane = threadIdx.x, c = blockIdx.x;
-  for (int e = lane; e < E; e += 64) base[e] = expert_offsets[e] + chunk_counts[(size_t)c * E + e];
-  __syncthreads();
-  const int lo = c * kChunk;
-  const int hi = min(lo + kChunk, TK);
-  for (int s0 = lo; s0 < hi; s0 += 64) {
-    const int s = s0 + lane;
-    int v = (s < hi) ? ids[s] : -1;
-    const bool valid = (s < hi) && v >= 0 && v < E;
-    int rank, cnt;
-    bool is_last;
-    match_rank(v, valid, lane, rank, cnt, is_last);
-    int row = valid ? base[v] + rank : -1;
-    __syncthreads();
-    if (valid && is_last) base[v] += cnt;
-    __syncthreads();
-    if (valid && row < TK) sorted_slot[row] = s;
-    if (s < hi) slot_to_row[s] = row;
+  __shared__ int wcount[NWV][MOE_MAX_EXPERTS];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = blockIdx.x;
+  for (int e = tid; e < E; e += kChunk) {
+    base[e] = expert_offsets[e] + chunk_counts[(size_t)c * E + e];
+#pragma unroll
+    for (int w = 0; w < NWV; w++) wcount[w][e] = 0;
   }
+  const int s = c * kChunk + tid;
+  const int v = s < TK ? ids[s] : -1;
+  const bool valid = s < TK && v >= 0 && v < E;
+  int rank, cnt;
+  bool is_last;
+  match_rank(v, valid, lane, rank, cnt, is_last);
+  __syncthreads();
+  if (valid && is_last) wcount[wave][v] = cnt;
+  __syncthreads();
+  int row = -1;
+  if (valid) {
+    row = base[v] + rank;
+    for (int w = 0; w < wave; w++) row += wcount[w][v];
+  }
+  if (valid && row < TK) sorted_slot[row] = s;
+  if (s < TK) slot_to_row[s] = row;
 }
 
 // Whole permutation of at most kChunk slots by one workgroup, one slot per thread: the rank of a
@@ -209,7 +225,7 @@ int permute_launch(hipStream_t st, const int32_t *ids, int T, int K, int E, int 
   permute_count_kernel<<<ws.n_chunks, 64, 0, st>>>(ids, TK, E, ws.chunk_counts);
   permute_scan_kernel<<<1, 1024, 0, st>>>(ws.chunk_counts, ws.n_chunks, E, tile_m, ws.max_tiles, expert_offsets,
                                           ws.tile_prefix, ws.tile_expert);
-  permute_scatter_kernel<<<ws.n_chunks, 64, 0, st>>>(ids, TK, E, ws.chunk_counts, expert_offsets, sorted_slot,
+  permute_scatter_kernel<<<ws.n_chunks, kChunk, 0, st>>>(ids, TK, E, ws.chunk_counts, expert_offsets, sorted_slot,
                                                      slot_to_row);
   return (int)hipGetLastError();
 }
