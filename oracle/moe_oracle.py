@@ -18,6 +18,8 @@ What follows which reference lines (paths relative to the reference root):
   route_sigmoid_recipe        python/regression/test_llm/test_torch_ops.py:441-456
   permute_literal             torch_tpu/csrc/ops/my_ops/fusedMoE.pl:624-756
   permute_counting_sort       the same permutation as a stable counting sort
+  mlp_w8a16_dq_ref            python/regression/test_llm/test_mlp_w8a16_dq.py:53-81
+  mm_w8a16_dq_ref             python/regression/test_llm/test_mm_w8a16_dq.py:52-60
 
 Pinned by tests/test_oracle.py against: the reference's routing tables and its
 ``err_data`` vector (tests/golden/reference_fixtures.json), brute force on tiny
@@ -28,7 +30,7 @@ dense MLP).
 Parity unpinned (the reference holds no source, test or vector for them; they are
 defined here from the workload description and closed forms only):
   act_quant_group128, quant_weight_block128, experts_w8a8_fp32, moe_w8a8_fp32,
-  route_softmax_topk, route_sigmoid_grouped (bias handling).
+  mlp_w8a8_fp32, mm_w8a8_fp32, route_softmax_topk, route_sigmoid_grouped (bias handling).
 """
 from __future__ import annotations
 
@@ -350,6 +352,39 @@ def experts_w8a8_fp32(x, select_experts, w13q, w13s, w2q, w2s, block=BLOCK, retu
     if return_mid:
         return out, (xq, xs, hq_all.reshape(T, K, I), hs_all.reshape(T, K, -1))
     return out
+
+
+# --------------------------------------------------------------------------- #
+# dense layers (the same arithmetic with one expert that owns every row)
+# --------------------------------------------------------------------------- #
+def mlp_w8a16_dq_ref(x, gate_weight, up_weight, down_weight, gate_scale, up_scale, down_scale, block=BLOCK):
+    """Reference form: block-dequantise each weight into bf16 (block loop), then a bf16
+    F.linear / F.silu chain.  gate/up [I, H], down [H, I] in checkpoint orientation."""
+    x = x.to(torch.bfloat16)
+    g = F.silu(F.linear(x, weight_dequant_literal(gate_weight, gate_scale, block)))
+    u = F.linear(x, weight_dequant_literal(up_weight, up_scale, block))
+    return F.linear(g * u, weight_dequant_literal(down_weight, down_scale, block))
+
+
+def mm_w8a16_dq_ref(x, weight, scale, block=BLOCK):
+    """Reference form: block-dequantise w [N, K] into bf16, then F.linear in bf16 (ragged N allowed)."""
+    return F.linear(x.to(torch.bfloat16), weight_dequant_literal(weight, scale, block))
+
+
+def mm_w8a8_fp32(x, wq, ws, block=BLOCK):
+    """x [M, K] bf16 quantised per row and 128 columns, times dequantised w [N, K]^T, all in fp32."""
+    xq, xs = act_quant_group128(x, block)
+    return act_dequant_group128(xq, xs, block) @ dequant_block(wq, ws, block).T
+
+
+def mlp_w8a8_fp32(x, w13q, w13s, w2q, w2s, block=BLOCK, return_mid=False, mid=None):
+    """Dense gated MLP on quantised operands: experts_w8a8_fp32 with a single expert and a single
+    slot per row.  w13q [2I, H], w2q [H, I]."""
+    sel = torch.zeros(x.shape[0], 1, dtype=torch.int32)
+    r = experts_w8a8_fp32(x, sel, w13q[None], w13s[None], w2q[None], w2s[None], block, return_mid, mid)
+    if return_mid:
+        return r[0][:, 0], r[1]
+    return r[:, 0]
 
 
 def e4m3_step(code_u8: torch.Tensor) -> torch.Tensor:

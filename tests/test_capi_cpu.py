@@ -53,6 +53,9 @@ def test_argument_errors_are_codes_not_crashes(pkg):
     assert lib.moe_route_topk(None, fake, 0, None, 1, 8, 9, 0, 1, 1, 1, 1.0, fake, fake, None) == E_SHAPE
     assert lib.moe_route_topk(None, fake, 0, None, 1, 8, 2, 9, 1, 1, 1, 1.0, fake, fake, None) == E_MODE
     assert lib.moe_permute(None, fake, 4, 2, 8, fake, fake, fake, fake, 16) == E_WS
+    assert lib.moe_mm_fp8(None, fake, 4, 200, fake, fake, 64, fake, fake, 1 << 20) == E_ALIGN    # K % 128
+    assert lib.moe_mm_fp8(None, fake, 4, 256, fake, fake, 8, fake, fake, 1 << 20) == E_SHAPE     # N < 16
+    assert lib.moe_mlp_fp8(None, fake, 4, 256, fake, fake, fake, fake, 128, fake, fake, 16) == E_WS
     assert lib.moe_permute(None, fake, 4, 2, 5000, fake, fake, fake, fake, 1 << 20) == E_SHAPE
     ws = lib.moe_fused_experts_workspace_bytes(4, 256, 512, 8, 2, 0)
     assert ws > 0 and ws % 256 == 0
@@ -102,6 +105,8 @@ def test_my_ops_are_registered_with_reference_arity(pkg):
     assert len(ops.fused_moe_fused_experts_v2.default._schema.arguments) == 27
     assert len(ops.noaux_tc_topk.default._schema.arguments) == 6
     assert len(ops.fused_moe_grouped_topk.default._schema.arguments) == 10
+    assert len(ops.mlp_w8a16_dq_forward.default._schema.arguments) == 9     # ops.hpp:279-288
+    assert len(ops.mm_w8a16_dq_forward.default._schema.arguments) == 5      # ops.hpp:290-295
     with pytest.raises(RuntimeError, match="closed-source"):
         ops.fused_moe_grouped_topk(*[torch.zeros(1)] * 10)
     z = torch.zeros(1, 1, 128, dtype=torch.bfloat16)

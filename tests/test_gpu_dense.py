@@ -1,0 +1,81 @@
+"""GPU parity of the dense block-scaled FP8 layers (my_ops.mm_w8a16_dq_forward, mlp_w8a16_dq_forward)
+against the oracle, on the reference's own shape grids and data recipes
+(python/regression/test_llm/test_mm_w8a16_dq.py:101-109, test_deepseek_mm.py:125-132,194-200,
+test_mlp_w8a16_dq.py:141-148: x ~ N(0,1) bf16, weights N(0,1) cast to e4m3fn, scales N(0,1) bf16)."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 2e-2, 1e-2          # on outputs normalised to unit rms
+MAX_OUTSIDE = 5e-3               # MLP only: share of elements a one-step flip of a re-quantised code may move
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def normalised_outside(got, ref):
+    rms = ref.pow(2).mean().sqrt().clamp_min(1e-12)
+    g, r = got / rms, ref / rms
+    return ((g - r).abs() > ATOL + RTOL * r.abs()).float().mean().item()
+
+
+MM_SHAPES = [(32, 7168, 1536), (32, 7168, 576), (32, 2048, 7168), (64, 4096, 2048), (128, 7168, 1536),
+             (256, 4096, 1024), (1, 256, 16), (200, 384, 272)]
+
+
+@pytest.mark.parametrize("M,K,N", MM_SHAPES)
+def test_mm_w8a16_dq_forward(pkg, oracle, dev, M, K, N):
+    say("mm", M, K, N)
+    g = torch.Generator().manual_seed(1000 + M + N)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = torch.randn(N, K, generator=g).to(torch.float8_e4m3fn)
+    s = torch.randn((N + 127) // 128, K // 128, generator=g).to(torch.bfloat16)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    r = torch.ops.my_ops.mm_w8a16_dq_forward(x.to(dev), w.to(dev), s.to(dev), out, 128)
+    torch.cuda.synchronize()
+    assert r.data_ptr() == out.data_ptr()
+    got = out.float().cpu()
+    assert torch.isfinite(got).all()
+    # the reference's criterion against its own bf16 ground truth
+    assert oracle.cos_sim(oracle.mm_w8a16_dq_ref(x, w, s).float().flatten(), got.flatten()) >= 0.99
+    # the same quantised operands multiplied in fp32: every element within tolerance
+    ref = oracle.mm_w8a8_fp32(x, w, s.float())
+    assert normalised_outside(got, ref) == 0.0
+
+
+@pytest.mark.parametrize("M,H,I", [(32, 7168, 2304), (32, 7168, 256), (64, 4096, 2048), (1, 256, 128), (200, 512, 384)])
+def test_mlp_w8a16_dq_forward(pkg, oracle, dev, M, H, I):
+    say("mlp", M, H, I)
+    g = torch.Generator().manual_seed(2000 + M + I)
+    x = torch.randn(M, H, generator=g).to(torch.bfloat16)
+    wg = torch.randn(I, H, generator=g).to(torch.float8_e4m3fn)
+    wu = torch.randn(I, H, generator=g).to(torch.float8_e4m3fn)
+    wd = torch.randn(H, I, generator=g).to(torch.float8_e4m3fn)
+    sg = torch.randn(I // 128, H // 128, generator=g).to(torch.bfloat16)
+    su = torch.randn(I // 128, H // 128, generator=g).to(torch.bfloat16)
+    sd = torch.randn(H // 128, I // 128, generator=g).to(torch.bfloat16)
+    out = torch.empty(M, H, dtype=torch.bfloat16, device=dev)
+    # the reference hands the down projection and its scales over transposed (non-contiguous views)
+    torch.ops.my_ops.mlp_w8a16_dq_forward(x.to(dev), wg.to(dev), wu.to(dev), wd.T.to(dev), sg.to(dev), su.to(dev),
+                                          sd.T.to(dev), out, 128)
+    torch.cuda.synchronize()
+    got = out.float().cpu()
+    assert torch.isfinite(got).all()
+    assert oracle.cos_sim(oracle.mlp_w8a16_dq_ref(x, wg, wu, wd, sg, su, sd).float().flatten(), got.flatten()) >= 0.99
+    w13q, w13s = torch.cat([wg, wu], 0), torch.cat([sg, su], 0).float()
+    ref, mid = oracle.mlp_w8a8_fp32(x, w13q, w13s, wd, sd.float(), return_mid=True)
+    assert normalised_outside(got, ref) <= MAX_OUTSIDE
+    assert oracle.cal_diff(ref, got)[0] < 1e-4
+
+
+def test_dense_ops_reject_what_they_do_not_support(pkg, dev):
+    x = torch.zeros(4, 256, dtype=torch.bfloat16, device=dev)
+    w = torch.zeros(128, 256, dtype=torch.float8_e4m3fn, device=dev)
+    s = torch.ones(1, 2, dtype=torch.bfloat16, device=dev)
+    out = torch.empty(4, 128, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(RuntimeError):
+        torch.ops.my_ops.mm_w8a16_dq_forward(x, w, s, out, 64)
+    with pytest.raises(RuntimeError):
+        torch.ops.my_ops.mm_w8a16_dq_forward(x, w.view(torch.uint8), s, out, 128)

@@ -381,3 +381,55 @@ def test_metrics(oracle):
     assert cd == pytest.approx(0.0) and rmse == 0 and amax == 0
     cd, rmse, amax = oracle.cal_diff(t, torch.tensor([3.0, 2.0]))
     assert amax == 2.0 and rmse == pytest.approx(math.sqrt(2.0)) and cd == pytest.approx(1 - 2 * 17 / 38)
+
+
+# ----------------------------------------------------------------------------- dense layers
+def test_dense_refs_reduce_to_library_routines(oracle):
+    """scale == 1: the reference-form dense layers are plain F.linear chains on the cast weights;
+    a ragged output width (576 = 4.5 blocks) uses the fifth scale row for its last 64 rows."""
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(5)
+    M, K, N = 6, 256, 576
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = torch.randn(N, K, generator=g).to(torch.float8_e4m3fn)
+    ones = torch.ones(5, 2, dtype=torch.bfloat16)
+    assert torch.equal(oracle.mm_w8a16_dq_ref(x, w, ones), F.linear(x, w.to(torch.bfloat16)))
+    s = ones.clone()
+    s[4, :] = 2.0                                                  # only rows 512..575 are doubled
+    y = oracle.mm_w8a16_dq_ref(x, w, s).float()
+    y1 = F.linear(x, w.to(torch.bfloat16)).float()
+    assert torch.equal(y[:, :512], y1[:, :512]) and torch.equal(y[:, 512:], 2 * y1[:, 512:])
+    I = 128
+    wg = torch.randn(I, K, generator=g).to(torch.float8_e4m3fn)
+    wu = torch.randn(I, K, generator=g).to(torch.float8_e4m3fn)
+    wd = torch.randn(K, I, generator=g).to(torch.float8_e4m3fn)
+    one_a, one_b = torch.ones(1, 2, dtype=torch.bfloat16), torch.ones(2, 1, dtype=torch.bfloat16)
+    want = F.linear(F.silu(F.linear(x, wg.to(torch.bfloat16))) * F.linear(x, wu.to(torch.bfloat16)), wd.to(torch.bfloat16))
+    assert torch.equal(oracle.mlp_w8a16_dq_ref(x, wg, wu, wd, one_a, one_a, one_b), want)
+
+
+def test_dense_w8a8_against_brute_force(oracle):
+    """mm_w8a8_fp32 on a tiny case, element by element in python floats from the quantised operands;
+    mlp_w8a8_fp32 == the single-expert MoE (already pinned) and its pieces chain through mm_w8a8_fp32."""
+    g = torch.Generator().manual_seed(6)
+    M, K, N = 3, 256, 16
+    x = (torch.randn(M, K, generator=g) * 3).to(torch.bfloat16)
+    wq, ws = oracle.quant_weight_block128(torch.randn(128, K, generator=g) * 0.05)
+    wq, ws = wq[:N], ws                                            # ragged: 16 rows of one 128-row block
+    got = oracle.mm_w8a8_fp32(x, wq, ws)
+    xq, xs = oracle.act_quant_group128(x)
+    tab = oracle.e4m3_decode_table()
+    for m in range(M):
+        for n in range(N):
+            acc = 0.0
+            for k in range(K):
+                a = float(tab[int(xq.view(torch.uint8)[m, k])]) * float(xs[m, k // 128])
+                b = float(tab[int(wq.view(torch.uint8)[n, k])]) * float(ws[0, k // 128])
+                acc += a * b
+            assert abs(acc - float(got[m, n])) <= 1e-5 * max(1.0, abs(acc))
+    E, H, I = 1, 256, 128
+    w13q, w13s, w2q, w2s = oracle.make_layer(E, H, I, seed=7)
+    xx = torch.randn(5, H, generator=g).to(torch.bfloat16)
+    y, (xq2, xs2, hq, hs) = oracle.mlp_w8a8_fp32(xx, w13q[0], w13s[0], w2q[0], w2s[0], return_mid=True)
+    h = oracle.act_dequant_group128(hq[:, 0].view(torch.float8_e4m3fn), hs[:, 0])
+    assert torch.allclose(y, h @ oracle.dequant_block(w2q[0], w2s[0]).T, rtol=1e-6, atol=1e-6)

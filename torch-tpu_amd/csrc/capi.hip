@@ -135,3 +135,84 @@ extern "C" int moe_fused_experts_fp8(void *stream, const void *x_bf16, int T, in
   }
   return moe_weighted_reduce(stream, y, routing_weights, has_shared ? w.sh_y : nullptr, T, K, H, out_bf16);
 }
+
+// ---- dense block-scaled FP8 linear layers: the grouped kernels with one "expert" that owns every row ----
+
+namespace moe {
+struct DenseWs {
+  uint8_t *xq;
+  float *xs;
+  uint8_t *hq;
+  float *hs;
+  size_t bytes;
+};
+static DenseWs dense_layout(void *base, int M, int K, int I) {
+  DenseWs w{};
+  size_t off = 0;
+  auto take = [&](size_t n) {
+    void *p = base ? (void *)((uint8_t *)base + off) : nullptr;
+    off += align_up(n ? n : 1, 256);
+    return p;
+  };
+  w.xq = (uint8_t *)take((size_t)M * K);
+  w.xs = (float *)take((size_t)M * scale_pitch(K / kBlock) * 4);
+  if (I > 0) {
+    w.hq = (uint8_t *)take((size_t)M * I);
+    w.hs = (float *)take((size_t)M * scale_pitch(I / kBlock) * 4);
+  }
+  w.bytes = off;
+  return w;
+}
+}  // namespace moe
+
+extern "C" size_t moe_mm_fp8_workspace_bytes(int M, int K) {
+  if (M < 0 || K < 1) return 0;
+  return moe::dense_layout(nullptr, M, K, 0).bytes;
+}
+
+extern "C" int moe_mm_fp8(void *stream, const void *x_bf16, int M, int K, const uint8_t *w, const float *w_scale,
+                          int N, void *out_bf16, void *workspace, size_t workspace_bytes) {
+  using namespace moe;
+  if (!x_bf16 || !w || !w_scale || !out_bf16 || !workspace) return MOE_E_NULL;
+  if (M < 0 || K < 1 || N < 16 || K > 32768 || N > (1 << 20)) return MOE_E_SHAPE;
+  if (K % kBlock || N % 16) return MOE_E_ALIGN;
+  if ((double)M * K >= 2147483648.0 || (double)M * N >= 2147483648.0 || (double)N * K >= 4294967296.0) return MOE_E_SHAPE;
+  if (((uintptr_t)workspace % 256) || ((uintptr_t)x_bf16 % 16) || ((uintptr_t)out_bf16 % 8) || ((uintptr_t)w % 16))
+    return MOE_E_ALIGN;
+  DenseWs d = dense_layout(workspace, M, K, 0);
+  if (workspace_bytes < d.bytes) return MOE_E_WORKSPACE;
+  if (M == 0) return MOE_OK;
+  int rc = moe_act_quant(stream, x_bf16, M, K, d.xq, d.xs);
+  if (rc) return rc;
+  return gemm2_launch((hipStream_t)stream, d.xq, d.xs, M, M, N, w, w_scale, K, 1, 1, nullptr, nullptr, nullptr, 0,
+                      (uint16_t *)out_bf16, nullptr, nullptr, 0, nullptr, nullptr, nullptr);
+}
+
+extern "C" size_t moe_mlp_fp8_workspace_bytes(int M, int H, int I) {
+  if (M < 0 || H < 1 || I < 1) return 0;
+  return moe::dense_layout(nullptr, M, H, I).bytes;
+}
+
+extern "C" int moe_mlp_fp8(void *stream, const void *x_bf16, int M, int H, const uint8_t *w13, const float *w13_scale,
+                           const uint8_t *w2, const float *w2_scale, int I, void *out_bf16, void *workspace,
+                           size_t workspace_bytes) {
+  using namespace moe;
+  if (!x_bf16 || !w13 || !w13_scale || !w2 || !w2_scale || !out_bf16 || !workspace) return MOE_E_NULL;
+  if (M < 0 || H < 1 || I < 1 || H > 32768 || I > 32768) return MOE_E_SHAPE;
+  if (H % kBlock || I % kBlock) return MOE_E_ALIGN;
+  if ((double)M * H >= 2147483648.0 || (double)M * I >= 2147483648.0) return MOE_E_SHAPE;
+  if (((uintptr_t)workspace % 256) || ((uintptr_t)x_bf16 % 16) || ((uintptr_t)out_bf16 % 8) || ((uintptr_t)w13 % 16) ||
+      ((uintptr_t)w2 % 16))
+    return MOE_E_ALIGN;
+  DenseWs d = dense_layout(workspace, M, H, I);
+  if (workspace_bytes < d.bytes) return MOE_E_WORKSPACE;
+  if (M == 0) return MOE_OK;
+  hipStream_t st = (hipStream_t)stream;
+  int rc = moe_act_quant(stream, x_bf16, M, H, d.xq, d.xs);
+  if (rc) return rc;
+  rc = gemm1_launch(st, d.xq, d.xs, M, H, w13, w13_scale, I, 1, 1, nullptr, nullptr, nullptr, 0, d.hq, d.hs, nullptr,
+                    nullptr, nullptr, nullptr);
+  if (rc) return rc;
+  return gemm2_launch(st, d.hq, d.hs, M, M, H, w2, w2_scale, I, 1, 1, nullptr, nullptr, nullptr, 0, (uint16_t *)out_bf16,
+                      nullptr, nullptr, 0, nullptr, nullptr, nullptr);
+}

@@ -200,7 +200,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   __syncthreads();
 
   const int NKB = a.Kd >> 7;
-  const int n_wblk = a.n_rows_w >> 7;                 // weight-scale rows per expert
+  const int n_wblk = (a.n_rows_w + 127) >> 7;         // weight-scale rows per expert
 
   // ---- per-lane source addresses ------------------------------------------------------------
   // GATED: tiles 0..WT/2-1 are gate columns, WT/2..WT-1 the matching up columns.

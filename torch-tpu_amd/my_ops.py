@@ -32,6 +32,11 @@ _lib.define("fused_moe_grouped_topk(Tensor topk_experts_res, Tensor topk_weights
             "Tensor right_bf16, Tensor topk_weights_res, Tensor left, Tensor right, Tensor max, Tensor matmul_res, "
             "Tensor softmax_res) -> Tensor")
 
+_lib.define("mlp_w8a16_dq_forward(Tensor input, Tensor gate_weight, Tensor up_weight, Tensor down_weight, "
+            "Tensor gate_scale, Tensor up_scale, Tensor down_scale, Tensor(a!) output, int blocksize) -> Tensor(a!)")
+_lib.define("mm_w8a16_dq_forward(Tensor input, Tensor weight, Tensor scale, Tensor(a!) output, int blocksize) "
+            "-> Tensor(a!)")
+
 # packed copies of reference-layout weights, keyed by the identity of the six tensors
 _pack_cache: dict = {}
 
@@ -93,7 +98,53 @@ def _grouped_topk(*args):
                        "undocumented; use noaux_tc_topk or torch_tpu_amd.moe_route instead")
 
 
+_dense_cache: dict = {}
+
+
+def _dense_packed(key_tensors, make):
+    key = tuple((t.data_ptr(), t._version, tuple(t.shape), tuple(t.stride())) for t in key_tensors)
+    hit = _dense_cache.get(key)
+    if hit is None:
+        if len(_dense_cache) > 32:
+            _dense_cache.clear()
+        hit = make()
+        _dense_cache[key] = hit
+    return hit
+
+
+def _check_dense(blocksize, *fp8):
+    if blocksize != 128:
+        raise RuntimeError("only blocksize 128 is supported")
+    for t in fp8:
+        if t.dtype != torch.float8_e4m3fn:
+            raise RuntimeError("weights must be float8_e4m3fn")
+
+
+def _mlp_w8a16_dq_forward(input, gate_weight, up_weight, down_weight, gate_scale, up_scale, down_scale, output,
+                          blocksize):
+    """torch_tpu/csrc/ops/my_ops/MlpW8A16Dq.cpp:189-241: gate/up [I,H], down passed transposed as
+    [I,H] (python/regression/test_llm/test_mlp_w8a16_dq.py:106-109), scales likewise; output [M,H]."""
+    _check_dense(blocksize, gate_weight, up_weight, down_weight)
+    w13, w13s, w2, w2s = _dense_packed(
+        (gate_weight, up_weight, down_weight, gate_scale, up_scale, down_scale),
+        lambda: (torch.cat([gate_weight, up_weight], 0).contiguous(),
+                 torch.cat([gate_scale, up_scale], 0).to(torch.float32).contiguous(),
+                 down_weight.t().contiguous(), down_scale.t().to(torch.float32).contiguous()))
+    ops.mlp_fp8(input.contiguous(), w13, w13s, w2, w2s, out=output)
+    return output
+
+
+def _mm_w8a16_dq_forward(input, weight, scale, output, blocksize):
+    """torch_tpu/csrc/ops/my_ops/MmW8A16Dq.cpp:185-228: weight [N,K], scale [ceil(N/bs), K/bs], output [M,N]."""
+    _check_dense(blocksize, weight)
+    w, ws = _dense_packed((weight, scale), lambda: (weight.contiguous(), scale.to(torch.float32).contiguous()))
+    ops.mm_fp8(input.contiguous(), w, ws, out=output)
+    return output
+
+
 _lib.impl("fused_moe_fused_experts", _fused_experts, "CompositeExplicitAutograd")
+_lib.impl("mlp_w8a16_dq_forward", _mlp_w8a16_dq_forward, "CompositeExplicitAutograd")
+_lib.impl("mm_w8a16_dq_forward", _mm_w8a16_dq_forward, "CompositeExplicitAutograd")
 _lib.impl("fused_moe_fused_experts_v2", _fused_experts_v2, "CompositeExplicitAutograd")
 _lib.impl("noaux_tc_topk", ops.noaux_tc_topk, "CompositeExplicitAutograd")
 _lib.impl("fused_moe_grouped_topk", _grouped_topk, "CompositeExplicitAutograd")

@@ -205,6 +205,52 @@ def fused_experts_fp8(x, w13, w13_scale, w2, w2_scale, ids, routing_weights=None
     return out
 
 
+# --------------------------------------------------------------------------- dense layers
+def mm_fp8(x, w, w_scale, out=None, workspace=None):
+    """Dense block-scaled linear layer: x [M,K] bf16, w [N,K] e4m3fn, fp32 scales [ceil(N/128), K/128]
+    -> out [M,N] bf16.  The activations are quantised per row and 128 columns first."""
+    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], "x must be [M,K] and w [N,K]")
+    M, K = x.shape
+    N = w.shape[0]
+    _need(tuple(w_scale.shape) == ((N + 127) // 128, K // 128), "w_scale must be [ceil(N/128), K/128]")
+    if out is None:
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=x.device)
+    _need(tuple(out.shape) == (M, N), "out must be [M,N]")
+    need = lib.moe_mm_fp8_workspace_bytes(M, K)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+    _need(workspace.numel() * workspace.element_size() >= need, "workspace too small")
+    rc = lib.moe_mm_fp8(_stream(), _dev(x, "x", torch.bfloat16), M, K, _dev(w, "w", _FP8),
+                        _dev(w_scale, "w_scale", torch.float32), N, _dev(out, "out", torch.bfloat16),
+                        _dev(workspace, "workspace"), workspace.numel() * workspace.element_size())
+    check(rc, "mm_fp8")
+    return out
+
+
+def mlp_fp8(x, w13, w13_scale, w2, w2_scale, out=None, workspace=None):
+    """Dense gated MLP: x [M,H] bf16, w13 [2I,H] (gate rows then up rows), w2 [H,I], fp32 128x128
+    block scales -> out [M,H] bf16 = (silu(x Wg^T) * (x Wu^T)) Wd^T, FP8 matrix products."""
+    _need(x.dim() == 2 and w13.dim() == 2 and w2.dim() == 2, "x, w13, w2 must be 2-d")
+    M, H = x.shape
+    I = w13.shape[0] // 2
+    _need(tuple(w13.shape) == (2 * I, H) and tuple(w2.shape) == (H, I), "w13 must be [2I,H] and w2 [H,I]")
+    _need(tuple(w13_scale.shape) == (2 * I // 128, H // 128) and tuple(w2_scale.shape) == (H // 128, I // 128),
+          "bad scale shapes")
+    if out is None:
+        out = torch.empty(M, H, dtype=torch.bfloat16, device=x.device)
+    _need(tuple(out.shape) == (M, H), "out must be [M,H]")
+    need = lib.moe_mlp_fp8_workspace_bytes(M, H, I)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+    _need(workspace.numel() * workspace.element_size() >= need, "workspace too small")
+    rc = lib.moe_mlp_fp8(_stream(), _dev(x, "x", torch.bfloat16), M, H, _dev(w13, "w13", _FP8),
+                         _dev(w13_scale, "w13_scale", torch.float32), _dev(w2, "w2", _FP8),
+                         _dev(w2_scale, "w2_scale", torch.float32), I, _dev(out, "out", torch.bfloat16),
+                         _dev(workspace, "workspace"), workspace.numel() * workspace.element_size())
+    check(rc, "mlp_fp8")
+    return out
+
+
 def gemm1_swiglu(xq, xs, w13, w13_scale, ids_shape, sorted_slot, offsets, permute_ws):
     """Stage: first grouped GEMM + SwiGLU + re-quantisation -> (hq [T*K, I] e4m3fn, hs [T*K, I/128])."""
     T, K = ids_shape
