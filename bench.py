@@ -234,6 +234,39 @@ def bench_decode(pkg, moe, cfg, dev, steps, warmup):
     return res
 
 
+def _lib():
+    from torch_tpu_amd._lib import lib
+    return lib
+
+
+def bench_dense(pkg, dev, steps, warmup):
+    """The dense block-scaled layers (same kernels, one expert): DeepSeek-V3 shapes of the reference's
+    dense tests at a decode and a prefill batch."""
+    res = []
+    g = torch.Generator(device=dev).manual_seed(7)
+    for kind, M, K, N in (("mm", 32, 7168, 1536), ("mm", 4096, 7168, 1536), ("mm", 4096, 2048, 7168),
+                          ("mlp", 32, 7168, 18432), ("mlp", 4096, 7168, 18432)):
+        x = torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16)
+        if kind == "mm":
+            w, ws = make_weights(pkg, 1, N, K, dev, 31)
+            w, ws = w[0], ws[0]
+            out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+            wsp = torch.empty(_lib().moe_mm_fp8_workspace_bytes(M, K), dtype=torch.uint8, device=dev)
+            fn = lambda: pkg.mm_fp8(x, w, ws, out=out, workspace=wsp)
+            flops, nbytes = 2.0 * M * K * N, N * K + 2 * M * K + 2 * M * N
+        else:
+            I = N
+            w13, w13s = make_weights(pkg, 1, 2 * I, K, dev, 32)
+            w2, w2s = make_weights(pkg, 1, K, I, dev, 33)
+            out = torch.empty(M, K, dtype=torch.bfloat16, device=dev)
+            wsp = torch.empty(_lib().moe_mlp_fp8_workspace_bytes(M, K, I), dtype=torch.uint8, device=dev)
+            fn = lambda: pkg.mlp_fp8(x, w13[0], w13s[0], w2[0], w2s[0], out=out, workspace=wsp)
+            flops, nbytes = 6.0 * M * K * I, 3 * K * I + 4 * M * K
+        sec = time_steps(fn, max(steps, 10), warmup)
+        res.append(dict(op=kind, M=M, K=K, N=N, ms=sec * 1e3, tflops=flops / sec / 1e12, hbm_gbs=nbytes / sec / 1e9))
+    return res
+
+
 def cpu_baseline(pkg, moe, cfg, x, sample_tokens):
     """The CPU oracle (routing, per-expert dequantise + fp32 matmul, weighted reduce) timed on the
     first `sample_tokens` tokens of the batch; the same pass doubles as a parity check of the
@@ -325,6 +358,8 @@ def main():
     }
     if not args.no_decode and args.workload == "c3_prefill":
         result["decode"] = bench_decode(pkg, moe, cfg, dev, args.steps, args.warmup)
+    if not args.no_decode and args.workload == "c3_prefill":
+        result["dense"] = bench_dense(pkg, dev, args.steps, args.warmup)
     if not args.no_cpu:
         base, parity = cpu_baseline(pkg, moe, cfg, x, min(args.cpu_sample, T))
         result["cpu_baseline"] = base

@@ -132,11 +132,21 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   // than one row tile, the weight strip.
   const int n_routed = a.fixed_expert >= 0 ? (a.rows_a + BM - 1) / BM : min(a.tile_prefix[a.E], a.max_mtiles);
   const int n_mtiles = n_routed + (a.sh_rows + BM - 1) / BM;
-  const int n_work = n_mtiles * a.n_strips;
-  const int per_xcd = (n_work + 7) >> 3;
-  if ((int)(blockIdx.x >> 3) >= per_xcd) return;
-  const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (logical >= n_work) return;
+  // Each XCD takes an equal share of the shared expert's work items (full tiles: the heaviest, so
+  // they go first) and then an equal, contiguous share of the routed ones.
+  const int n_routed_work = n_routed * a.n_strips, n_shared_work = (n_mtiles - n_routed) * a.n_strips;
+  const int per_xcd_r = (n_routed_work + 7) >> 3, per_xcd_s = (n_shared_work + 7) >> 3;
+  const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+  const int my_shared = min(max(n_shared_work - xcd * per_xcd_s, 0), per_xcd_s);
+  int logical;
+  if (idx < my_shared) {
+    logical = n_routed_work + xcd * per_xcd_s + idx;
+  } else {
+    const int j = idx - my_shared;
+    if (j >= per_xcd_r) return;
+    logical = xcd * per_xcd_r + j;
+    if (logical >= n_routed_work) return;
+  }
   // Inside one expert the (row tile, strip) pairs are walked in blocks of up to kBlockM row tiles x
   // kBlockS strips, so that the ~32 workgroups an XCD runs at a time share a few token tiles and a few
   // weight strips through its L2 instead of streaming 32 different strips.
@@ -393,7 +403,9 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     int kb = 0, stage = 0, stage_req = DEPTH;
     for (; kb + DEPTH < NKB; kb++) {
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 1) * L_STEP) : "memory");
+#ifndef MOE_DBG_NOBARRIER
       __syncthreads();
+#endif
       if ((kb & 15) == 0 && (kb >> 4) + 1 < n_chunks) request_scales((kb >> 4) + 1);
       request(kb + DEPTH, stage_req);
       compute(stage, kb, wlo[0], whi[0]);
@@ -608,7 +620,7 @@ static int launch_gemm(hipStream_t st, GemmArgs &a, int tile_m, int max_mtiles) 
   a.n_strips = GATED ? a.N / 128 : (a.N + 255) / 256;
   a.max_mtiles = max_mtiles - (a.sh_rows + tile_m - 1) / tile_m;
   long total = (long)max_mtiles * a.n_strips;
-  total = (total + 7) / 8 * 8;
+  total = (total + 7) / 8 * 8 + 16;                  // the per-XCD split rounds two shares up
   if (total <= 0 || total > 0x7fffffffl) return MOE_E_SHAPE;
   a.total_blocks = (int)total;
   dim3 grid((unsigned)total);
