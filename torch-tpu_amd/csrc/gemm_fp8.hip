@@ -83,6 +83,7 @@ struct GemmSmem {
   int arow[BM];                                  // source row in aq / as for each tile row
   int oslot[BM];                                 // second GEMM: output row of each tile row
   float amax[NW][BM];                            // GATED epilogue: per-wavefront partial amax
+  float2 fsc[4][BM];                             // large tiles: scale products of four steps, one pair per tile row
   float sb[2][kMaxKB + 4];                       // weight-block scales of the strip for every 128-step, then zeros
 };
 
@@ -429,9 +430,9 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     // Requests past the last step re-read it (cheap cache hits) instead of branching; a step past
     // an odd count multiplies by the zero weight scale stored behind the table.  The loop body is
     // instantiated per number of live m-tiles, so there is no branch between matrix instructions.
-    static_assert(DEPTH == 2 || DEPTH == 3, "the register ring holds two or three steps");
+    static_assert(DEPTH == 2, "the register ring holds two steps");
     constexpr int R = DEPTH;                             // ring slots = steps per pass of the unrolled loop
-    constexpr int XB = R == 2 ? 4 : 3;                   // token operand buffers; R * LIVE is a multiple of it
+    constexpr int XB = 4;                                // token operand buffers; R * LIVE is a multiple of it
     constexpr int L_WAIT = NTOK + 2 * WT * (R - 1);      // loads younger than the ones a step boundary needs
     const int last = NKB - 1;
     const int o0 = (lg ^ (li & 7)) << 4, o1 = ((lg + 4) ^ (li & 7)) << 4;
@@ -452,32 +453,47 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
       __syncthreads();
       if (n_chunks > 1) request_scales(1);
       request(min(3, last), 3);
+      // Scale products: what a lane multiplies a matrix-instruction result with is (activation scale
+      // of its token and step) x (weight-block scale of its tile and step).  One thread per tile row
+      // forms both products of a step once, two steps ahead, instead of every wavefront forming them
+      // for every m-tile (one multiply less per matrix instruction on the shared issue port).
+      auto produce_f = [&](int k) {
+        if (tid < BM) {
+          const int kc = min(k, last);                   // past the end: a finite scale times the zero behind the table
+          const float sa = sm.sac[(kc >> 4) & 1][(tid >> 4) * 256 + ((kc & 12) << 4) + (tid & 15) * 4 + (kc & 3)];
+          sm.fsc[k & 3][tid] = make_float2(sa * sm.sb[0][k], sa * sm.sb[1][k]);
+        }
+      };
+      produce_f(0);
+      produce_f(1);
+      produce_f(2);
+      __syncthreads();
       auto read_x = [&](int kb, int mt) {
         const uint8_t *t = sm.tok[kb & 3] + li * 128 + mt * 2048;
         return concat8(*(const v4i *)(t + o0), *(const v4i *)(t + o1));
       };
-      auto read_sa = [&](int kb, int mt) {
-        kb = min(kb, last);                              // a step past the end: any finite scale (times zero)
-        return sm.sac[(kb >> 4) & 1][mt * 256 + ((kb & 12) << 4) + li * 4 + (kb & 3)];
+      // GATED: both products (gate tiles use .x, up tiles .y); second GEMM: the one of this wavefront's column block
+      auto read_f = [&](int kb, int mt) {
+        if (GATED) return sm.fsc[kb & 3][mt * 16 + li];
+        const float f = ((const float *)&sm.fsc[kb & 3][mt * 16 + li])[sb_row0];
+        return make_float2(f, f);
       };
       v8i x[XB];
-      float sa_[XB], sc[R][2], f_[2][2];
+      float2 fb[XB];
       v4f p[2][WT];
 #pragma unroll
       for (int q = 0; q < PD; q++) {
         const int qq = q < LIVE ? q : q - LIVE, kk = q < LIVE ? 0 : 1;
-        x[q] = read_x(kk, LIVE - 1 - qq); sa_[q] = read_sa(kk, LIVE - 1 - qq);
+        x[q] = read_x(kk, LIVE - 1 - qq); fb[q] = read_f(kk, LIVE - 1 - qq);
       }
-      sc[0][0] = sm.sb[sb_row0][0]; sc[0][1] = sm.sb[sb_row1][0];
       // the multiply-add slot of the very first m-tile adds zero
 #pragma unroll
       for (int j = 0; j < WT; j++) p[1][j] = (v4f){0.f, 0.f, 0.f, 0.f};
-      f_[1][0] = f_[1][1] = 0.f;
+      fb[XB - 1] = make_float2(0.f, 0.f);
       for (int s0 = 0; s0 < NKB; s0 += R) {
 #pragma unroll
         for (int h = 0; h < R; h++) {
           const int kb = s0 + h;
-          sc[(h + 1) % R][0] = sm.sb[sb_row0][kb + 1]; sc[(h + 1) % R][1] = sm.sb[sb_row1][kb + 1];
           v8i wc[WT];
 #pragma unroll
           for (int j = 0; j < WT; j++) wc[j] = concat8(wlo[h][j], whi[h][j]);
@@ -491,19 +507,17 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
               const int qq = q + PD < LIVE ? q + PD : q + PD - LIVE;
               const int kk = q + PD < LIVE ? kb : kb + 1;
               x[(g + PD) % XB] = read_x(kk, LIVE - 1 - qq);
-              sa_[(g + PD) % XB] = read_sa(kk, LIVE - 1 - qq);
+              fb[(g + PD) % XB] = read_f(kk, LIVE - 1 - qq);
             }
 #pragma unroll
             for (int j = 0; j < WT; j++) {
               const v4f zero = {0.f, 0.f, 0.f, 0.f};
               p[g & 1][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wc[j], x[g % XB], zero, 0, 0, 0, 0, 0, 0);
             }
-            f_[g & 1][0] = sa_[g % XB] * sc[h][0];
-            f_[g & 1][1] = sa_[g % XB] * sc[h][1];
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int j = 0; j < WT; j++) {
-              const float f = (GATED && j >= WT / 2) ? f_[(g + 1) & 1][1] : f_[(g + 1) & 1][0];
+              const float f = (GATED && j >= WT / 2) ? fb[(g + XB - 1) % XB].y : fb[(g + XB - 1) % XB].x;
 #pragma unroll
               for (int r = 0; r < 4; r++) acc[tp][j][r] = fmaf(p[(g + 1) & 1][j][r], f, acc[tp][j][r]);
               // pins the multiply-adds here: without it they are sunk below the whole step's matrix
@@ -524,6 +538,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
           asm volatile("s_waitcnt vmcnt(%0)" ::"n"(L_WAIT) : "memory");
           arrived_weights(wlo[(h + 1) % R], whi[(h + 1) % R]);
           __syncthreads();
+          produce_f(kb + 3);
           if (((kb + 1) & 15) == 0 && ((kb + 1) >> 4) + 1 < n_chunks) request_scales(((kb + 1) >> 4) + 1);
 #if !defined(MOE_DBG_NOLOAD) && !defined(MOE_DBG_NOTOK)
           request(min(kb + 4, last), kb & 3);
@@ -539,7 +554,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
       // m-tile 0 of the last step is still pending
 #pragma unroll
       for (int j = 0; j < WT; j++) {
-        const float f = (GATED && j >= WT / 2) ? f_[1][1] : f_[1][0];
+        const float f = (GATED && j >= WT / 2) ? fb[XB - 1].y : fb[XB - 1].x;
 #pragma unroll
         for (int r = 0; r < 4; r++) acc[0][j][r] = fmaf(p[1][j][r], f, acc[0][j][r]);
       }
