@@ -73,7 +73,7 @@ def build_layer(pkg, cfg, dev):
     if cfg.get("zipf"):
         # popularity ~ rank^-s through a logit offset; a few experts are switched off entirely
         rank = torch.randperm(E, generator=g, device=dev).float() + 1
-        bias = -cfg["zipf"] * torch.log(rank) * 2.0
+        bias = -cfg["zipf"] * torch.log(rank)
         bias[torch.randperm(E, generator=g, device=dev)[:cfg["empty"]]] = -1e9
     elif cfg["route"] == "sigmoid":
         bias = torch.zeros(E, device=dev)           # uniform correction bias

@@ -439,3 +439,86 @@ def test_hip_graph_replay_matches_eager(pkg, oracle, dev):
             scratch = moe(xs[(rep + 1) % 3])            # eager work between replays
             torch.cuda.synchronize()
             del scratch
+
+
+def _layer_on_device(pkg, dev, E, H, I, seed):
+    def weights(n, k, sd):
+        gg = torch.Generator(device=dev).manual_seed(sd)
+        q = torch.empty(E, n, k, dtype=torch.float8_e4m3fn, device=dev)
+        s = torch.empty(E, n // 128, k // 128, dtype=torch.float32, device=dev)
+        step = max(1, (1 << 27) // (n * k))
+        for e0 in range(0, E, step):
+            e1 = min(E, e0 + step)
+            w = (torch.randn(e1 - e0, n, k, generator=gg, device=dev) * 0.02).to(torch.bfloat16)
+            q[e0:e1], s[e0:e1] = pkg.quant_weight_block128(w)
+        return q, s
+    w13, w13s = weights(2 * I, H, seed)
+    w2, w2s = weights(H, I, seed + 1)
+    return w13, w13s, w2, w2s
+
+
+def _full_size_checks(pkg, oracle, dev, x, layer, ids, w, pick):
+    """Size-independent properties of the expert computation plus a few tokens against the oracle."""
+    w13, w13s, w2, w2s = layer
+    T = x.shape[0]
+    y = pkg.fused_experts_fp8(x, w13, w13s, w2, w2s, ids)
+    out = pkg.fused_experts_fp8(x, w13, w13s, w2, w2s, ids, w)
+    torch.cuda.synchronize()
+    assert torch.isfinite(y.float()).all()
+    torch.testing.assert_close(out.float(), torch.einsum("tk,tkh->th", w, y.float()), rtol=1e-2, atol=1e-2)
+    sub = torch.arange(0, T, max(1, T // 97), device=dev)
+    y_sub = pkg.fused_experts_fp8(x[sub].contiguous(), w13, w13s, w2, w2s, ids[sub].contiguous())
+    assert torch.equal(y_sub.view(torch.int16), y[sub].view(torch.int16)), "a token's result depends on the batch"
+    y_rev = pkg.fused_experts_fp8(x[sub].contiguous(), w13, w13s, w2, w2s, ids[sub].flip(1).contiguous())
+    assert torch.equal(y_rev.flip(1).view(torch.int16), y[sub].view(torch.int16)), "a token's result depends on slot order"
+    # only the experts those tokens use are brought to the host
+    sel = ids[pick.to(dev)].cpu()
+    used = torch.unique(sel).tolist()
+    remap = {e: i for i, e in enumerate(used)}
+    sel_local = torch.tensor([[remap[int(e)] for e in row] for row in sel], dtype=torch.int32)
+    idx = torch.tensor(used, device=dev)
+    small = tuple(t[idx].cpu() for t in layer)
+    ref = oracle.experts_w8a8_fp32(x[pick.to(dev)].cpu(), sel_local, *small)
+    got = y[pick.to(dev)].float().cpu()
+    assert outside_fraction(got, ref) <= MAX_OUTSIDE
+    assert oracle.cal_diff(ref, got)[0] < 1e-5
+
+
+def test_full_size_properties_mixtral_shape(pkg, oracle, dev):
+    """Mixtral-8x7B layer shape (8 experts, top-2, 1024 rows per expert: the matrix-core-bound case) at T=4096."""
+    say("full size C2")
+    T, H, I, E, K = 4096, 4096, 14336, 8, 2
+    layer = _layer_on_device(pkg, dev, E, H, I, 31)
+    g = torch.Generator(device=dev).manual_seed(33)
+    x = torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16)
+    logits = (torch.randn(T, E, generator=g, device=dev)).float()
+    w, ids = pkg.moe_route(logits, K, "softmax", None, 1, 1, True, 1.0)
+    w_ref, ids_ref = oracle.route_softmax_topk(logits.cpu(), K, True)
+    assert torch.equal(ids.cpu(), ids_ref) and torch.allclose(w.cpu(), w_ref, rtol=1e-5, atol=1e-7)
+    ss, off, s2r = pkg.moe_permute(ids, E)
+    ss_ref, off_ref, s2r_ref = oracle.permute_counting_sort(ids_ref, E)
+    assert torch.equal(ss.cpu(), ss_ref) and torch.equal(off.cpu(), off_ref) and torch.equal(s2r.cpu(), s2r_ref)
+    _full_size_checks(pkg, oracle, dev, x, layer, ids, w, torch.tensor([7, 1900, 4095]))
+
+
+def test_full_size_properties_skewed_load(pkg, oracle, dev):
+    """Qwen3-30B-A3B layer shape, T=16384, popularity ~ rank^-1.2 and 13 experts that receive nothing: experts
+    with thousands of rows (many row tiles) next to experts with a handful, and empty ones."""
+    say("full size C5")
+    T, H, I, E, K = 16384, 2048, 768, 128, 8
+    layer = _layer_on_device(pkg, dev, E, H, I, 41)
+    g = torch.Generator(device=dev).manual_seed(43)
+    x = torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16)
+    rank = torch.randperm(E, generator=g, device=dev).float() + 1
+    bias = -1.2 * torch.log(rank)
+    bias[torch.randperm(E, generator=g, device=dev)[:13]] = -1e9
+    logits = torch.randn(T, E, generator=g, device=dev) * 0.9 + bias
+    w, ids = pkg.moe_route(logits, K, "softmax", None, 1, 1, True, 1.0)
+    w_ref, ids_ref = oracle.route_softmax_topk(logits.cpu(), K, True)
+    assert torch.equal(ids.cpu(), ids_ref) and torch.allclose(w.cpu(), w_ref, rtol=1e-5, atol=1e-7)
+    ss, off, s2r = pkg.moe_permute(ids, E)
+    ss_ref, off_ref, s2r_ref = oracle.permute_counting_sort(ids_ref, E)
+    assert torch.equal(ss.cpu(), ss_ref) and torch.equal(off.cpu(), off_ref) and torch.equal(s2r.cpu(), s2r_ref)
+    counts = (off_ref[1:] - off_ref[:-1])
+    assert int((counts == 0).sum()) >= 13 and int(counts.max()) > 8000
+    _full_size_checks(pkg, oracle, dev, x, layer, ids, w, torch.tensor([0, 5000, 11111, 16383]))
