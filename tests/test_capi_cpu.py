@@ -5,6 +5,7 @@ import os
 import re
 
 import pytest
+import torch
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
@@ -113,3 +114,30 @@ def test_my_ops_are_registered_with_reference_arity(pkg):
     with pytest.raises(RuntimeError, match="int32"):
         ops.fused_moe_fused_experts(z, z[0], None, None, z, z, z, z, z, z, torch.zeros(1, 1, dtype=torch.int64),
                                     z[0], None, None, None, 128, 1, 1, True, 8, 4, None, None, None, False)
+
+
+def test_checkpoint_layout_conversion_is_pure_data_movement(pkg, oracle):
+    """convert_hf_moe_layer stacks per-expert checkpoint tensors into the packed layout; the packed
+    tensors dequantise to exactly what the per-expert tensors dequantise to."""
+    E, H, I = 3, 256, 128
+    g = torch.Generator().manual_seed(3)
+    state, pre = {}, "model.layers.3.mlp."
+    for e in list(range(E)) + ["s"]:
+        base = pre + ("shared_experts." if e == "s" else f"experts.{e}.")
+        for proj, (n, k) in (("gate_proj", (I, H)), ("up_proj", (I, H)), ("down_proj", (H, I))):
+            q, s = oracle.quant_weight_block128(torch.randn(n, k, generator=g) * 0.05)
+            state[base + proj + ".weight"], state[base + proj + ".weight_scale_inv"] = q, s
+    state[pre + "gate.weight"] = torch.randn(E, H, generator=g)
+    state[pre + "gate.e_score_correction_bias"] = torch.randn(E, generator=g)
+    out = pkg.convert_hf_moe_layer(state, pre, E)
+    assert out["w13"].shape == (E, 2 * I, H) and out["w2"].shape == (E, H, I) and out["router_weight"].dtype == torch.bfloat16
+    for e in range(E):
+        gate = oracle.dequant_block(state[f"{pre}experts.{e}.gate_proj.weight"], state[f"{pre}experts.{e}.gate_proj.weight_scale_inv"])
+        up = oracle.dequant_block(state[f"{pre}experts.{e}.up_proj.weight"], state[f"{pre}experts.{e}.up_proj.weight_scale_inv"])
+        down = oracle.dequant_block(state[f"{pre}experts.{e}.down_proj.weight"], state[f"{pre}experts.{e}.down_proj.weight_scale_inv"])
+        w13 = oracle.dequant_block(out["w13"][e], out["w13_scale"][e])
+        assert torch.equal(w13[:I], gate) and torch.equal(w13[I:], up)
+        assert torch.equal(oracle.dequant_block(out["w2"][e], out["w2_scale"][e]), down)
+    sw13, sw13s, sw2, sw2s = out["shared"]
+    assert sw13.shape == (1, 2 * I, H) and sw2.shape == (1, H, I) and sw13s.dtype == torch.float32
+    assert torch.equal(out["bias"], state[pre + "gate.e_score_correction_bias"])

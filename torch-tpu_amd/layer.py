@@ -38,6 +38,44 @@ def quant_weight_block128(w: torch.Tensor):
     return q.reshape(*lead, N, K), scale
 
 
+def convert_hf_moe_layer(state: dict, prefix: str, num_experts: int, device=None):
+    """Checkpoint tensors of one DeepSeek-V3-style FP8 MoE layer -> the packed layout of the kernels.
+
+    Reads `{prefix}experts.{e}.{gate,up,down}_proj.weight` (e4m3fn `[out, in]`) and the matching
+    `.weight_scale_inv` (fp32 `[ceil(out/128), ceil(in/128)]`, the value a block is MULTIPLIED by),
+    `{prefix}gate.weight` (router, `[E, H]`), optionally `{prefix}gate.e_score_correction_bias` and
+    `{prefix}shared_experts.*`.  Returns a dict with router_weight, bias, w13, w13_scale, w2, w2_scale
+    and shared (a 4-tuple or None).  Pure data movement: codes and scales are not re-quantised.
+    The reference hands the same tensors to its op as separate gate / up / transposed-down arguments
+    (python/regression/test_llm/test_moe.py:285-288); torch_tpu_amd.pack_expert_weights packs that form."""
+    def get(name):
+        t = state[prefix + name]
+        return t.to(device) if device is not None else t
+
+    def stack(proj, suffix):
+        return torch.stack([get(f"experts.{e}.{proj}.{suffix}") for e in range(num_experts)])
+
+    w13 = torch.cat([stack("gate_proj", "weight"), stack("up_proj", "weight")], dim=1).contiguous()
+    w13_scale = torch.cat([stack("gate_proj", "weight_scale_inv"), stack("up_proj", "weight_scale_inv")],
+                          dim=1).to(torch.float32).contiguous()
+    w2 = stack("down_proj", "weight").contiguous()
+    w2_scale = stack("down_proj", "weight_scale_inv").to(torch.float32).contiguous()
+    for t in (w13, w2):
+        if t.dtype != torch.float8_e4m3fn:
+            raise RuntimeError("expert weights must be float8_e4m3fn (convert bf16 checkpoints with quant_weight_block128)")
+    shared = None
+    if prefix + "shared_experts.gate_proj.weight" in state:
+        sg, su, sd = (get(f"shared_experts.{p}.weight") for p in ("gate_proj", "up_proj", "down_proj"))
+        sgs, sus, sds = (get(f"shared_experts.{p}.weight_scale_inv") for p in ("gate_proj", "up_proj", "down_proj"))
+        shared = (torch.cat([sg, su], 0)[None].contiguous(), torch.cat([sgs, sus], 0)[None].to(torch.float32).contiguous(),
+                  sd[None].contiguous(), sds[None].to(torch.float32).contiguous())
+    bias = state.get(prefix + "gate.e_score_correction_bias")
+    if bias is not None:
+        bias = (bias.to(device) if device is not None else bias).to(torch.float32).contiguous()
+    return dict(router_weight=get("gate.weight").to(torch.bfloat16).contiguous(), bias=bias, w13=w13, w13_scale=w13_scale,
+                w2=w2, w2_scale=w2_scale, shared=shared)
+
+
 class FusedMoE:
     """Router + routed experts (+ shared expert) of one MoE layer, inference only.
 
@@ -64,7 +102,7 @@ class FusedMoE:
         return self._ws
 
     def route(self, x):
-        logits = torch.matmul(x, self.router_weight.t()).float()
+        logits = torch.matmul(x, self.router_weight.t())           # bf16; the routing kernel widens it
         bias = self.bias
         if self.mode == "softmax" and bias is not None:
             logits, bias = logits + bias, None          # a softmax router's bias is part of the logits
