@@ -251,7 +251,7 @@ def bench_dense(pkg, dev, steps, warmup):
             w, ws = make_weights(pkg, 1, N, K, dev, 31)
             w, ws = w[0], ws[0]
             out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
-            wsp = torch.empty(_lib().moe_mm_fp8_workspace_bytes(M, K), dtype=torch.uint8, device=dev)
+            wsp = torch.empty(_lib().moe_mm_fp8_workspace_bytes(M, K, N), dtype=torch.uint8, device=dev)
             fn = lambda: pkg.mm_fp8(x, w, ws, out=out, workspace=wsp)
             flops, nbytes = 2.0 * M * K * N, N * K + 2 * M * K + 2 * M * N
         else:

@@ -169,14 +169,16 @@ int moe_weighted_reduce(void *stream, const void *y_bf16, const float *routing_w
  * moe_mm_fp8 replaces at::mm_w8a16_dq_forward -> tpudnnMmW8A16DqAsync
  * (torch_tpu/csrc/ops/my_ops/MmW8A16Dq.cpp:185-228): out [M, N] bf16 = x [M, K] bf16 times the
  * transpose of w [N, K] fp8 with fp32 scales [ceil(N/128), K/128].  K a multiple of 128, N a
- * multiple of 16.
+ * multiple of 16.  Up to 128 rows a per-wavefront kernel slices the reduction over the chip and a
+ * second kernel adds the slices in a fixed order (for the MLP the SwiGLU and re-quantisation ride in that
+ * reduction); above that the grouped kernel runs with one expert.
  * moe_mlp_fp8 replaces at::mlp_w8a16_dq_forward -> tpudnnMlpW8A16DqAsync
  * (torch_tpu/csrc/ops/my_ops/MlpW8A16Dq.cpp:189-241): out [M, H] bf16 =
  * (silu(x Wg^T) * (x Wu^T)) Wd^T with w13 [2I, H] = gate rows then up rows, w2 [H, I].
  * Unlike the reference (bf16 activations against de-quantised weights) both quantise the
  * activations per row and 128 columns, as the expert path does; the matrix products run in FP8.
  */
-size_t moe_mm_fp8_workspace_bytes(int M, int K);
+size_t moe_mm_fp8_workspace_bytes(int M, int K, int N);
 int moe_mm_fp8(void *stream, const void *x_bf16, int M, int K, const uint8_t *w, const float *w_scale, int N,
                void *out_bf16, void *workspace, size_t workspace_bytes);
 size_t moe_mlp_fp8_workspace_bytes(int M, int H, int I);

@@ -22,7 +22,7 @@ def normalised_outside(got, ref):
 
 
 MM_SHAPES = [(32, 7168, 1536), (32, 7168, 576), (32, 2048, 7168), (64, 4096, 2048), (128, 7168, 1536),
-             (256, 4096, 1024), (1, 256, 16), (200, 384, 272)]
+             (256, 4096, 1024), (1, 256, 16), (200, 384, 272), (100, 4096, 8192), (128, 1024, 64)]
 
 
 @pytest.mark.parametrize("M,K,N", MM_SHAPES)
@@ -45,7 +45,8 @@ def test_mm_w8a16_dq_forward(pkg, oracle, dev, M, K, N):
     assert normalised_outside(got, ref) == 0.0
 
 
-@pytest.mark.parametrize("M,H,I", [(32, 7168, 2304), (32, 7168, 256), (64, 4096, 2048), (1, 256, 128), (200, 512, 384)])
+@pytest.mark.parametrize("M,H,I", [(32, 7168, 2304), (32, 7168, 256), (64, 4096, 2048), (1, 256, 128), (200, 512, 384),
+                                   (32, 4096, 8192), (100, 1024, 1024)])
 def test_mlp_w8a16_dq_forward(pkg, oracle, dev, M, H, I):
     say("mlp", M, H, I)
     g = torch.Generator().manual_seed(2000 + M + I)

@@ -16,6 +16,12 @@ int gemm2_launch(hipStream_t st, const uint8_t *hq, const float *hs, int rows_a,
                  const PermuteWs *pw, int fixed_expert, uint16_t *y, const uint8_t *sh_hq, const float *sh_hs,
                  int sh_rows, const uint8_t *sh_w2, const float *sh_w2s, uint16_t *sh_y);
 
+size_t dense_small_partial_bytes(int M, int K, int N, bool keep_partial);
+int dense_small_launch(hipStream_t st, const uint8_t *xq, const float *xs, int M, int K, const uint8_t *w, const float *ws,
+                       int N, uint16_t *out, float *partial, int *n_splits_out);
+int swiglu_quant_reduce_launch(hipStream_t st, const float *partial, int n_splits, int M, int I, uint8_t *hq, float *hs);
+constexpr int kDenseSmallRows = 128;        // up to this many rows the per-wavefront dense kernel is used
+
 // Carves the caller's workspace.  Every piece starts on a 256-byte boundary.
 struct FusedWs {
   void *permute;
@@ -144,9 +150,11 @@ struct DenseWs {
   float *xs;
   uint8_t *hq;
   float *hs;
+  float *partial;     // slices of the (only or second) product
+  float *partial1;    // MLP: slices of the first product
   size_t bytes;
 };
-static DenseWs dense_layout(void *base, int M, int K, int I) {
+static DenseWs dense_layout(void *base, int M, int K, int I, int N = 0) {
   DenseWs w{};
   size_t off = 0;
   auto take = [&](size_t n) {
@@ -160,14 +168,22 @@ static DenseWs dense_layout(void *base, int M, int K, int I) {
     w.hq = (uint8_t *)take((size_t)M * I);
     w.hs = (float *)take((size_t)M * scale_pitch(I / kBlock) * 4);
   }
+  if (N > 0 && M <= kDenseSmallRows) {
+    if (I > 0) {      // MLP: K = H, N = H; first product [M, 2I] over H, second [M, H] over I
+      w.partial1 = (float *)take(dense_small_partial_bytes(M, K, 2 * I, true));
+      w.partial = (float *)take(dense_small_partial_bytes(M, I, N, false));
+    } else {
+      w.partial = (float *)take(dense_small_partial_bytes(M, K, N, false));
+    }
+  }
   w.bytes = off;
   return w;
 }
 }  // namespace moe
 
-extern "C" size_t moe_mm_fp8_workspace_bytes(int M, int K) {
-  if (M < 0 || K < 1) return 0;
-  return moe::dense_layout(nullptr, M, K, 0).bytes;
+extern "C" size_t moe_mm_fp8_workspace_bytes(int M, int K, int N) {
+  if (M < 0 || K < 1 || N < 16 || K % moe::kBlock || N % 16) return 0;
+  return moe::dense_layout(nullptr, M, K, 0, N).bytes;
 }
 
 extern "C" int moe_mm_fp8(void *stream, const void *x_bf16, int M, int K, const uint8_t *w, const float *w_scale,
@@ -179,18 +195,20 @@ extern "C" int moe_mm_fp8(void *stream, const void *x_bf16, int M, int K, const 
   if ((double)M * K >= 2147483648.0 || (double)M * N >= 2147483648.0 || (double)N * K >= 4294967296.0) return MOE_E_SHAPE;
   if (((uintptr_t)workspace % 256) || ((uintptr_t)x_bf16 % 16) || ((uintptr_t)out_bf16 % 8) || ((uintptr_t)w % 16))
     return MOE_E_ALIGN;
-  DenseWs d = dense_layout(workspace, M, K, 0);
+  DenseWs d = dense_layout(workspace, M, K, 0, N);
   if (workspace_bytes < d.bytes) return MOE_E_WORKSPACE;
   if (M == 0) return MOE_OK;
   int rc = moe_act_quant(stream, x_bf16, M, K, d.xq, d.xs);
   if (rc) return rc;
+  if (M <= kDenseSmallRows)
+    return dense_small_launch((hipStream_t)stream, d.xq, d.xs, M, K, w, w_scale, N, (uint16_t *)out_bf16, d.partial, nullptr);
   return gemm2_launch((hipStream_t)stream, d.xq, d.xs, M, M, N, w, w_scale, K, 1, 1, nullptr, nullptr, nullptr, 0,
                       (uint16_t *)out_bf16, nullptr, nullptr, 0, nullptr, nullptr, nullptr);
 }
 
 extern "C" size_t moe_mlp_fp8_workspace_bytes(int M, int H, int I) {
   if (M < 0 || H < 1 || I < 1) return 0;
-  return moe::dense_layout(nullptr, M, H, I).bytes;
+  return moe::dense_layout(nullptr, M, H, I, H).bytes;
 }
 
 extern "C" int moe_mlp_fp8(void *stream, const void *x_bf16, int M, int H, const uint8_t *w13, const float *w13_scale,
@@ -204,12 +222,20 @@ extern "C" int moe_mlp_fp8(void *stream, const void *x_bf16, int M, int H, const
   if (((uintptr_t)workspace % 256) || ((uintptr_t)x_bf16 % 16) || ((uintptr_t)out_bf16 % 8) || ((uintptr_t)w13 % 16) ||
       ((uintptr_t)w2 % 16))
     return MOE_E_ALIGN;
-  DenseWs d = dense_layout(workspace, M, H, I);
+  DenseWs d = dense_layout(workspace, M, H, I, H);
   if (workspace_bytes < d.bytes) return MOE_E_WORKSPACE;
   if (M == 0) return MOE_OK;
   hipStream_t st = (hipStream_t)stream;
   int rc = moe_act_quant(stream, x_bf16, M, H, d.xq, d.xs);
   if (rc) return rc;
+  if (M <= kDenseSmallRows) {
+    int n1 = 0;
+    rc = dense_small_launch(st, d.xq, d.xs, M, H, w13, w13_scale, 2 * I, nullptr, d.partial1, &n1);
+    if (rc) return rc;
+    rc = swiglu_quant_reduce_launch(st, d.partial1, n1, M, I, d.hq, d.hs);
+    if (rc) return rc;
+    return dense_small_launch(st, d.hq, d.hs, M, I, w2, w2_scale, H, (uint16_t *)out_bf16, d.partial, nullptr);
+  }
   rc = gemm1_launch(st, d.xq, d.xs, M, H, w13, w13_scale, I, 1, 1, nullptr, nullptr, nullptr, 0, d.hq, d.hs, nullptr,
                     nullptr, nullptr, nullptr);
   if (rc) return rc;

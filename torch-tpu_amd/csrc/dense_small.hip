@@ -1,0 +1,247 @@
+// Dense block-scaled FP8 linear layer at decode batch sizes (M <= 128): out [M, N] = x [M, K] . w [N, K]^T.
+//
+// With so few rows the work is streaming the weights once, and the grouped kernel's 256-column
+// strips leave most of the chip idle (N = 1536 gives six workgroups).  Here one WAVEFRONT is the
+// unit: it owns one 16-row weight tile for a slice of the reduction and up to 64 token rows, keeps
+// everything in registers (no LDS, no barrier, operands loaded straight into matrix-instruction
+// layout), and several wavefronts per SIMD hide each other's load latency.  Slices of the
+// reduction are summed by a second, tiny kernel in a fixed order, so results are reproducible.
+#include "moe_common.h"
+#include "moe_layout.h"
+#include "../../include/moe_hip.h"
+
+namespace moe {
+
+struct SmallArgs {
+  const uint8_t *xq;     // [M, K] fp8
+  const float *xs;       // [M, xs_pitch] fp32
+  const uint8_t *w;      // [N, K] fp8
+  const float *ws;       // [ceil(N/128), K/128] fp32
+  float *partial;        // [n_splits, M, N] fp32 (n_splits > 1)
+  uint16_t *out;         // [M, N] bf16 (n_splits == 1)
+  int xs_pitch, M, K, N, NKB;
+  int split_len;         // reduction steps per slice
+  int n_splits, n_mchunks;
+  int keep_partial;      // write fp32 slices even when there is only one (a fused reduction follows)
+};
+
+__device__ __forceinline__ v8i cat8(v4i a, v4i b) {
+  v8i r;
+  r[0] = a[0]; r[1] = a[1]; r[2] = a[2]; r[3] = a[3];
+  r[4] = b[0]; r[5] = b[1]; r[6] = b[2]; r[7] = b[3];
+  return r;
+}
+
+// MT   m-tiles of 16 token rows per work item
+// NTW  weight tiles of 16 rows per work item: every token operand loaded from L2 serves NTW matrix
+//      instructions (wide layers), or 1 to get the most work items out of a narrow layer
+template <int MT, int NTW>
+__global__ __launch_bounds__(256) void dense_small_kernel(const SmallArgs a) {
+  constexpr int U = NTW == 1 ? 4 : 2;                    // reduction steps loaded together
+  const int lane = threadIdx.x & 63, li = lane & 15, lg = lane >> 4;
+  const int n_tiles = a.N / (16 * NTW);
+  long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);  // (row chunk, slice, weight tile group), the last fastest
+  const int nt = (int)(item % n_tiles);
+  item /= n_tiles;
+  const int sp = (int)(item % a.n_splits);
+  const int mc = (int)(item / a.n_splits);
+  if (mc >= a.n_mchunks) return;
+  const int kb0 = sp * a.split_len, kb1 = min(kb0 + a.split_len, a.NKB);
+  if (kb0 >= kb1) return;
+  // lane (li, lg) holds row li of an operand tile and 16-byte reduction chunks lg and lg + 4
+  const uint8_t *wp = a.w + (size_t)(nt * 16 * NTW + li) * a.K + lg * 16;
+  const size_t wtile = (size_t)16 * a.K;                 // bytes between consecutive weight tiles
+  const float *wsp = a.ws + (size_t)((nt * NTW) >> 3) * a.NKB;   // a group of tiles lies inside one 128-row block
+  const uint8_t *xp[MT];
+  const float *sap[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; mt++) {
+    const int row = min(mc * 16 * MT + mt * 16 + li, a.M - 1);
+    xp[mt] = a.xq + (size_t)row * a.K + lg * 16;
+    sap[mt] = a.xs + (size_t)row * a.xs_pitch;
+  }
+  v4f acc[NTW][MT];
+#pragma unroll
+  for (int j = 0; j < NTW; j++)
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) acc[j][mt] = (v4f){0.f, 0.f, 0.f, 0.f};
+  for (int kb = kb0; kb < kb1; kb += U) {
+    v4i wl[U][NTW], wh[U][NTW], xl[U][MT], xh[U][MT];
+    float f[U][MT];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const int kk = min(kb + u, kb1 - 1);               // past the slice: the last step again, times zero
+      const float sb = kb + u < kb1 ? wsp[kk] : 0.f;
+#pragma unroll
+      for (int j = 0; j < NTW; j++) {
+        wl[u][j] = *(const v4i *)(wp + j * wtile + (size_t)kk * 128);
+        wh[u][j] = *(const v4i *)(wp + j * wtile + (size_t)kk * 128 + 64);
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) {
+        xl[u][mt] = *(const v4i *)(xp[mt] + (size_t)kk * 128);
+        xh[u][mt] = *(const v4i *)(xp[mt] + (size_t)kk * 128 + 64);
+        f[u][mt] = sap[mt][kk] * sb;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) {
+        const v8i xc = cat8(xl[u][mt], xh[u][mt]);
+#pragma unroll
+        for (int j = 0; j < NTW; j++) {
+          const v4f zero = {0.f, 0.f, 0.f, 0.f};
+          const v4f p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(cat8(wl[u][j], wh[u][j]), xc, zero, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+          for (int r = 0; r < 4; r++) acc[j][mt][r] = fmaf(p[r], f[u][mt], acc[j][mt][r]);
+        }
+      }
+    }
+  }
+  // a lane holds output columns (tile)*16 + 4*lg .. +3 of token row li of each m-tile
+#pragma unroll
+  for (int mt = 0; mt < MT; mt++) {
+    const int row = mc * 16 * MT + mt * 16 + li;
+    if (row >= a.M) continue;
+#pragma unroll
+    for (int j = 0; j < NTW; j++) {
+      const size_t o = (size_t)row * a.N + (nt * NTW + j) * 16 + lg * 4;
+      if (a.n_splits == 1 && !a.keep_partial) {
+        v2i v;
+        v[0] = (int)((uint32_t)f32_to_bf16(acc[j][mt][0]) | ((uint32_t)f32_to_bf16(acc[j][mt][1]) << 16));
+        v[1] = (int)((uint32_t)f32_to_bf16(acc[j][mt][2]) | ((uint32_t)f32_to_bf16(acc[j][mt][3]) << 16));
+        *(v2i *)(a.out + o) = v;
+      } else {
+        *(v4f *)(a.partial + (size_t)sp * a.M * a.N + o) = acc[j][mt];
+      }
+    }
+  }
+}
+
+// out[m, n] = bf16(sum over slices in slice order), four columns per lane
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ partial, int n_splits, size_t mn,
+                                                           uint16_t *__restrict__ out) {
+  const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i >= mn) return;
+  v4f s = *(const v4f *)(partial + i);
+  for (int k = 1; k < n_splits; k++) {
+    const v4f t = *(const v4f *)(partial + (size_t)k * mn + i);
+    s[0] += t[0]; s[1] += t[1]; s[2] += t[2]; s[3] += t[3];
+  }
+  v2i v;
+  v[0] = (int)((uint32_t)f32_to_bf16(s[0]) | ((uint32_t)f32_to_bf16(s[1]) << 16));
+  v[1] = (int)((uint32_t)f32_to_bf16(s[2]) | ((uint32_t)f32_to_bf16(s[3]) << 16));
+  *(v2i *)(out + i) = v;
+}
+
+// Gated-MLP middle stage on the slices of the first product [n_splits, M, 2I] (gate columns, then up
+// columns): h = silu(sum gate) * (sum up), re-quantised per row and 128 columns.  Sixteen lanes share
+// one (row, 128-column group), eight columns each.
+__global__ __launch_bounds__(256) void swiglu_quant_reduce_kernel(const float *__restrict__ partial, int n_splits, int M,
+                                                                 int I, int hs_pitch, uint8_t *__restrict__ hq,
+                                                                 float *__restrict__ hs) {
+  const size_t grp = ((size_t)blockIdx.x * 256 + threadIdx.x) >> 4;
+  const int sub = threadIdx.x & 15;
+  const int groups_per_row = I / kBlock;
+  const bool live = grp < (size_t)M * groups_per_row;
+  float h[8];
+  float amax = 0.f;
+  size_t row = 0;
+  int col = 0;
+  if (live) {
+    row = grp / groups_per_row;
+    col = (int)(grp % groups_per_row) * kBlock + sub * 8;
+    float g[8], u[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) g[i] = u[i] = 0.f;
+    const size_t mn = (size_t)M * 2 * I;
+    for (int k = 0; k < n_splits; k++) {
+      const float *p = partial + (size_t)k * mn + row * 2 * I + col;
+      const v4f g0 = *(const v4f *)p, g1 = *(const v4f *)(p + 4), u0 = *(const v4f *)(p + I), u1 = *(const v4f *)(p + I + 4);
+#pragma unroll
+      for (int i = 0; i < 4; i++) { g[i] += g0[i]; g[4 + i] += g1[i]; u[i] += u0[i]; u[4 + i] += u1[i]; }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      h[i] = (g[i] / (1.0f + expf(-g[i]))) * u[i];
+      amax = fmaxf(amax, fabsf(h[i]));
+    }
+  }
+  amax = max_over_row16(amax);
+  if (!live) return;
+  const float sc = group_scale(amax);
+  v2i o;
+  o[0] = (int)pack4_fp8(h[0] / sc, h[1] / sc, h[2] / sc, h[3] / sc);
+  o[1] = (int)pack4_fp8(h[4] / sc, h[5] / sc, h[6] / sc, h[7] / sc);
+  *(v2i *)(hq + row * I + col) = o;
+  if (sub == 0) hs[row * hs_pitch + col / kBlock] = sc;
+}
+
+// How the reduction is sliced: enough wavefront-sized work items to fill the chip (the reference's
+// launcher weighs the same split-N against split-K trade-off on the host, MmW8A16Dq.cpp:94-142).
+void dense_small_plan(int M, int K, int N, int *n_splits, int *split_len, int *rows_per_item, int *n_mchunks,
+                      int *tiles_per_item) {
+  const int NKB = K / kBlock;
+  const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+  const int chunks = (M + 16 * mt - 1) / (16 * mt);
+  // four weight tiles per item when the layer is wide enough to still fill the chip with short slices
+  const int ntw = (N % 64 == 0 && (long)(N / 64) * chunks * (NKB / 8) >= 1024) ? 4 : 1;
+  *tiles_per_item = ntw;
+  const long tiles = (long)(N / (16 * ntw)) * chunks;
+  long want = (2048 + tiles - 1) / tiles;                // ~2 wavefronts per SIMD over 256 CUs
+  if (want < 1) want = 1;
+  int len = (int)((NKB + want - 1) / want);
+  len = (len + 3) / 4 * 4;                               // whole load batches
+  if (len > NKB) len = NKB;
+  *split_len = len;
+  *n_splits = (NKB + len - 1) / len;
+  *rows_per_item = 16 * mt;
+  *n_mchunks = chunks;
+}
+
+size_t dense_small_partial_bytes(int M, int K, int N, bool keep_partial) {
+  int s, l, r, c, t;
+  dense_small_plan(M, K, N, &s, &l, &r, &c, &t);
+  return (s > 1 || keep_partial) ? (size_t)s * M * N * 4 : 0;
+}
+
+// out != nullptr: bf16 result (slices added by a second kernel); out == nullptr: the fp32 slices stay in
+// `partial` for the caller's own reduction, their number is returned through n_splits_out.
+int dense_small_launch(hipStream_t st, const uint8_t *xq, const float *xs, int M, int K, const uint8_t *w, const float *ws,
+                       int N, uint16_t *out, float *partial, int *n_splits_out) {
+  SmallArgs a{};
+  a.keep_partial = out == nullptr;
+  int rows, ntw;
+  dense_small_plan(M, K, N, &a.n_splits, &a.split_len, &rows, &a.n_mchunks, &ntw);
+  a.xq = xq; a.xs = xs; a.xs_pitch = scale_pitch(K / kBlock); a.w = w; a.ws = ws; a.partial = partial; a.out = out;
+  a.M = M; a.K = K; a.N = N; a.NKB = K / kBlock;
+  const long items = (long)(N / (16 * ntw)) * a.n_splits * a.n_mchunks;
+  const long blocks = (items + 3) / 4;
+  if (blocks > 0x7fffffffl) return MOE_E_SHAPE;
+  const unsigned g = (unsigned)blocks;
+  if (ntw == 1) {
+    if (rows == 16) dense_small_kernel<1, 1><<<g, 256, 0, st>>>(a);
+    else if (rows == 32) dense_small_kernel<2, 1><<<g, 256, 0, st>>>(a);
+    else dense_small_kernel<4, 1><<<g, 256, 0, st>>>(a);
+  } else {
+    if (rows == 16) dense_small_kernel<1, 4><<<g, 256, 0, st>>>(a);
+    else if (rows == 32) dense_small_kernel<2, 4><<<g, 256, 0, st>>>(a);
+    else dense_small_kernel<4, 4><<<g, 256, 0, st>>>(a);
+  }
+  if (n_splits_out) *n_splits_out = a.n_splits;
+  if (a.n_splits > 1 && out != nullptr) {
+    const size_t mn = (size_t)M * N;
+    splitk_reduce_kernel<<<(unsigned)((mn / 4 + 255) / 256), 256, 0, st>>>(partial, a.n_splits, mn, out);
+  }
+  return (int)hipGetLastError();
+}
+
+int swiglu_quant_reduce_launch(hipStream_t st, const float *partial, int n_splits, int M, int I, uint8_t *hq, float *hs) {
+  const size_t lanes = (size_t)M * (I / kBlock) * 16;
+  swiglu_quant_reduce_kernel<<<(unsigned)((lanes + 255) / 256), 256, 0, st>>>(partial, n_splits, M, I,
+                                                                             scale_pitch(I / kBlock), hq, hs);
+  return (int)hipGetLastError();
+}
+
+}  // namespace moe

@@ -216,7 +216,7 @@ def mm_fp8(x, w, w_scale, out=None, workspace=None):
     if out is None:
         out = torch.empty(M, N, dtype=torch.bfloat16, device=x.device)
     _need(tuple(out.shape) == (M, N), "out must be [M,N]")
-    need = lib.moe_mm_fp8_workspace_bytes(M, K)
+    need = lib.moe_mm_fp8_workspace_bytes(M, K, N)
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
     _need(workspace.numel() * workspace.element_size() >= need, "workspace too small")
