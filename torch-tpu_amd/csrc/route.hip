@@ -46,6 +46,22 @@ __device__ __forceinline__ Best wave_argmax(Best b) {
   return r;
 }
 
+// Arg-max inside each half of the wavefront (lanes 0-31 and 32-63 separately); every lane ends up with
+// the winner of its own half.
+__device__ __forceinline__ Best half_argmax(Best b, int lane) {
+  argmax_step<0x111, 0xf>(b);   // row_shr:1
+  argmax_step<0x112, 0xf>(b);   // row_shr:2
+  argmax_step<0x114, 0xf>(b);   // row_shr:4
+  argmax_step<0x118, 0xf>(b);   // row_shr:8
+  argmax_step<0x142, 0xa>(b);   // row_bcast:15 into rows 1 and 3: lanes 31 and 63 hold the halves' winners
+  Best lo, hi;
+  lo.v = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, b.v), 31));
+  lo.i = __builtin_amdgcn_readlane(b.i, 31);
+  hi.v = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, b.v), 63));
+  hi.i = __builtin_amdgcn_readlane(b.i, 63);
+  return lane < 32 ? lo : hi;
+}
+
 __device__ __forceinline__ float round_to_bf16(float f) { return bf16_to_f32(f32_to_bf16(f)); }
 
 // Select top_k of one row.  v[j] holds element lane + 64*j (only j < per_lane are used,
@@ -64,34 +80,50 @@ __device__ __forceinline__ void select_row(float (&v)[PER_LANE], int E, int lane
   if (n_groups > 1) {
     const int per = E / n_groups;
     float gscore = 0.f;          // lane g keeps the score of group g (n_groups <= 64)
-    for (int g = 0; g < n_groups; g++) {
-      const int lo = g * per, hi = lo + per;
-      float sum = 0.f;
-      int first = -1;
-      for (int pass = 0; pass < 2; pass++) {
-        Best b{0.f, 0x7fffffff};
+    if (per == 32 && E == 64 * PER_LANE) {
+      // Groups of 32 (the DeepSeek-V3 shape): register j of lanes 0-31 is group 2j, of lanes 32-63
+      // group 2j+1, so both halves reduce at once and no range scan is needed.
 #pragma unroll
-        for (int j = 0; j < PER_LANE; j++) {
-          int e = lane + 64 * j;
-          if (e >= lo && e < hi && e != first && !(dead >> j & 1))
-            if (better(v[j], e, b.v, b.i)) { b.v = v[j]; b.i = e; }
-        }
-        b = wave_argmax(b);
-        if (b.i != 0x7fffffff) sum = (pass == 0) ? b.v : sum + b.v;
-        first = b.i;
+      for (int j = 0; j < PER_LANE; j++) {
+        const int e = lane + 64 * j;
+        Best b1 = half_argmax(Best{v[j], e}, lane);
+        Best b2 = half_argmax(Best{v[j], e == b1.i ? 0x7fffffff : e}, lane);
+        float sum = b1.v + (b2.i != 0x7fffffff ? b2.v : 0.f);
+        if (round_bf16) sum = round_to_bf16(sum);
+        const float lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sum), 0));
+        const float hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sum), 32));
+        if (lane == 2 * j) gscore = lo;
+        if (lane == 2 * j + 1) gscore = hi;
       }
-      if (round_bf16) sum = round_to_bf16(sum);
-      if (lane == g) gscore = sum;
+    } else {
+      for (int g = 0; g < n_groups; g++) {
+        const int lo = g * per, hi = lo + per;
+        float sum = 0.f;
+        int first = -1;
+        for (int pass = 0; pass < 2; pass++) {
+          Best b{0.f, 0x7fffffff};
+#pragma unroll
+          for (int j = 0; j < PER_LANE; j++) {
+            int e = lane + 64 * j;
+            if (e >= lo && e < hi && e != first && !(dead >> j & 1))
+              if (better(v[j], e, b.v, b.i)) { b.v = v[j]; b.i = e; }
+          }
+          b = wave_argmax(b);
+          if (b.i != 0x7fffffff) sum = (pass == 0) ? b.v : sum + b.v;
+          first = b.i;
+        }
+        if (round_bf16) sum = round_to_bf16(sum);
+        if (lane == g) gscore = sum;
+      }
     }
-    uint64_t keep = 0;
-    bool taken = false;
-    for (int s = 0; s < topk_groups; s++) {
-      Best b{gscore, (lane < n_groups && !taken) ? lane : 0x7fffffff};
-      b = wave_argmax(b);
-      if (b.i == 0x7fffffff) break;
-      keep |= 1ull << b.i;
-      if (lane == b.i) taken = true;
+    // the topk_groups best groups: lane g counts the groups that come before its own in
+    // "greater score, then lower index" order
+    int rank = 0;
+    for (int g = 0; g < n_groups; g++) {
+      const float s = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, gscore), g));
+      rank += (s > gscore || (s == gscore && g < lane)) ? 1 : 0;
     }
+    const uint64_t keep = __ballot(lane < n_groups && rank < topk_groups);
 #pragma unroll
     for (int j = 0; j < PER_LANE; j++) {
       int e = lane + 64 * j;
