@@ -45,6 +45,7 @@ struct GemmArgs {
   const int32_t *expert_offsets;
   const int32_t *tile_prefix;
   const int32_t *tile_expert;
+  const int32_t *tile_desc;     // [tiles][8], see the permutation
   uint8_t *hq;                  // GATED: [TK, N] fp8
   float *hs;                    // GATED: [TK, N/128]
   uint16_t *y;                  // !GATED: [TK, N] bf16 in slot order
@@ -119,7 +120,9 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   constexpr int NT = 64 * NW;                         // threads
   constexpr int WT = 16 / NW;                         // weight tiles per wavefront
   constexpr int STAGES = WREG ? 4 : DEPTH + 1;        // token tiles staged in LDS
-  __shared__ GemmSmem<MT, NW, STAGES, WREG ? 1 : STAGES, WREG ? 64 : 2048> sm;
+  using Smem = GemmSmem<MT, NW, STAGES, WREG ? 1 : STAGES, WREG ? 64 : 2048>;
+  static_assert(sizeof(Smem) <= 160 * 1024, "one workgroup's LDS");
+  __shared__ Smem sm;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -153,7 +156,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   // weight strips through its L2 instead of streaming 32 different strips.
   constexpr int kBlockM = 6, kBlockS = 5;
   const int g0 = logical / a.n_strips;                // some row tile of the expert this work item is in
-  int e, first_mtile, n_mt;                           // expert, its first row tile, its row tiles
+  int e, first_mtile, n_mt, e_row0 = 0, e_rows = 0;   // expert, its first row tile, its row tiles, first row, rows
   const bool shared = g0 >= n_routed;                 // a tile of the shared expert
   const bool direct = shared || a.fixed_expert >= 0;  // rows are taken in order, no permutation
   if (shared) {
@@ -161,10 +164,15 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   } else if (a.fixed_expert >= 0) {
     e = a.fixed_expert; first_mtile = 0; n_mt = n_routed;
   } else {
-    e = a.tile_expert[g0];
+    // one 32-byte record holds everything about the expert this tile belongs to
+    const v4i d0 = *(const v4i *)(a.tile_desc + (size_t)g0 * 8);
+    const v4i d1 = *(const v4i *)(a.tile_desc + (size_t)g0 * 8 + 4);
+    e = d0[0];
     if (e < 0 || e >= a.E) return;
-    first_mtile = a.tile_prefix[e];
-    n_mt = min(a.tile_prefix[e + 1], a.max_mtiles) - first_mtile;
+    first_mtile = d0[1];
+    n_mt = min(d0[1] + d0[2], a.max_mtiles) - first_mtile;
+    e_row0 = d0[3];
+    e_rows = d1[0];
   }
   int mtile, strip;
   {
@@ -187,8 +195,8 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     row0 = mtile * BM;
     rows = min(BM, a.rows_a - row0);
   } else {
-    row0 = a.expert_offsets[e] + (mtile - first_mtile) * BM;
-    rows = min(BM, a.expert_offsets[e + 1] - row0);
+    row0 = e_row0 + (mtile - first_mtile) * BM;
+    rows = min(BM, e_row0 + e_rows - row0);
   }
   const uint8_t *const aq = shared ? a.sh_aq : a.aq;
   const float *const as = shared ? a.sh_as : a.as;
@@ -676,6 +684,7 @@ int gemm1_launch(hipStream_t st, const uint8_t *xq, const float *xs, int T, int 
   a.aq = xq; a.as = xs; a.w = w13; a.ws = w13s;
   a.sorted_slot = sorted_slot; a.expert_offsets = expert_offsets;
   a.tile_prefix = pw ? pw->tile_prefix : nullptr; a.tile_expert = pw ? pw->tile_expert : nullptr;
+  a.tile_desc = pw ? pw->tile_desc : nullptr;
   a.hq = hq; a.hs = hs; a.y = nullptr;
   a.as_pitch = scale_pitch(H / kBlock); a.hs_pitch = scale_pitch(I / kBlock);
   a.Kd = H; a.N = I; a.n_rows_w = 2 * I; a.rows_a = T; a.topk = K; a.E = E; a.fixed_expert = fixed_expert;
@@ -693,6 +702,7 @@ int gemm2_launch(hipStream_t st, const uint8_t *hq, const float *hs, int rows_a,
   a.aq = hq; a.as = hs; a.w = w2; a.ws = w2s;
   a.sorted_slot = sorted_slot; a.expert_offsets = expert_offsets;
   a.tile_prefix = pw ? pw->tile_prefix : nullptr; a.tile_expert = pw ? pw->tile_expert : nullptr;
+  a.tile_desc = pw ? pw->tile_desc : nullptr;
   a.hq = nullptr; a.hs = nullptr; a.y = y;
   a.as_pitch = scale_pitch(I / kBlock); a.hs_pitch = 0;
   a.Kd = I; a.N = H; a.n_rows_w = H; a.rows_a = rows_a; a.topk = K; a.E = E; a.fixed_expert = fixed_expert;

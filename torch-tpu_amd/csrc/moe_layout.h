@@ -32,6 +32,7 @@ struct PermuteWs {
   int32_t *chunk_counts;   // [n_chunks, E]
   int32_t *tile_prefix;    // [E + 1] first tile of each expert; [E] = number of tiles
   int32_t *tile_expert;    // [max_tiles]
+  int32_t *tile_desc;      // [max_tiles][8]: expert, its first tile, its tiles, its first row, its rows, 0, 0, 0
   int n_chunks;
   int max_tiles;
 };
@@ -49,7 +50,7 @@ static inline size_t permute_ws_bytes(int T, int K, int E) {
   long tk = (long)T * K;
   size_t n_chunks = (size_t)((tk + kChunk - 1) / kChunk);
   if (n_chunks == 0) n_chunks = 1;
-  size_t ints = n_chunks * (size_t)E + (size_t)(E + 1) + (size_t)permute_max_tiles(T, K, E);
+  size_t ints = n_chunks * (size_t)E + (size_t)(E + 1) + 9 * (size_t)permute_max_tiles(T, K, E) + 8;
   return align_up(ints * 4, 256);
 }
 
@@ -62,6 +63,8 @@ static inline PermuteWs permute_ws_layout(void *ws, int T, int K, int E) {
   p.chunk_counts = (int32_t *)ws;
   p.tile_prefix = p.chunk_counts + (size_t)p.n_chunks * E;
   p.tile_expert = p.tile_prefix + (E + 1);
+  // 32-byte aligned: one descriptor is fetched with a single scalar load
+  p.tile_desc = (int32_t *)(((uintptr_t)(p.tile_expert + p.max_tiles) + 31) & ~(uintptr_t)31);
   return p;
 }
 

@@ -72,18 +72,26 @@ __device__ __forceinline__ int block_exclusive_scan(int x, int *lds_wave_sums, i
   return base + inc - x;
 }
 
-__device__ __forceinline__ void write_tiles(int e, int count, int first_tile, int tile_m, int32_t *tile_expert,
-                                            int max_tiles) {
+// every row tile of expert e gets the expert's whole description: the GEMM workgroups, which only know
+// "some tile of my expert", find their tile, rows and neighbours from one 32-byte record
+__device__ __forceinline__ void write_tiles(int e, int count, int first_row, int first_tile, int tile_m,
+                                            int32_t *tile_expert, int32_t *tile_desc, int max_tiles) {
   int nt = (count + tile_m - 1) / tile_m;
   for (int j = 0; j < nt; j++)
-    if (first_tile + j < max_tiles) tile_expert[first_tile + j] = e;
+    if (first_tile + j < max_tiles) {
+      tile_expert[first_tile + j] = e;
+      v4i *d = (v4i *)(tile_desc + (size_t)(first_tile + j) * 8);
+      d[0] = (v4i){e, first_tile, nt, first_row};
+      d[1] = (v4i){count, 0, 0, 0};
+    }
 }
 
 __global__ __launch_bounds__(1024) void permute_scan_kernel(int32_t *__restrict__ chunk_counts, int n_chunks, int E,
                                                             int tile_m, int max_tiles,
                                                             int32_t *__restrict__ expert_offsets,
                                                             int32_t *__restrict__ tile_prefix,
-                                                            int32_t *__restrict__ tile_expert) {
+                                                            int32_t *__restrict__ tile_expert,
+                                                            int32_t *__restrict__ tile_desc) {
   __shared__ int wave_sums[16];
   const int e = threadIdx.x;
   int count = 0;
@@ -110,7 +118,7 @@ __global__ __launch_bounds__(1024) void permute_scan_kernel(int32_t *__restrict_
   if (e < E) {
     expert_offsets[e] = off;
     tile_prefix[e] = first_tile;
-    write_tiles(e, count, first_tile, tile_m, tile_expert, max_tiles);
+    write_tiles(e, count, off, first_tile, tile_m, tile_expert, tile_desc, max_tiles);
   }
   if (e == 0) {
     expert_offsets[E] = total;
@@ -162,7 +170,8 @@ __global__ __launch_bounds__(kChunk) void permute_small_kernel(const int32_t *__
                                                               int32_t *__restrict__ expert_offsets,
                                                               int32_t *__restrict__ slot_to_row,
                                                               int32_t *__restrict__ tile_prefix,
-                                                              int32_t *__restrict__ tile_expert) {
+                                                              int32_t *__restrict__ tile_expert,
+                                                              int32_t *__restrict__ tile_desc) {
   __shared__ int hist[MOE_MAX_EXPERTS];
   __shared__ int offs[MOE_MAX_EXPERTS];
   __shared__ int sid[kChunk];
@@ -201,7 +210,7 @@ __global__ __launch_bounds__(kChunk) void permute_small_kernel(const int32_t *__
       offs[e] = base + inc - c;
       expert_offsets[e] = base + inc - c;
       tile_prefix[e] = tbase + tinc - t;
-      write_tiles(e, c, tbase + tinc - t, tile_m, tile_expert, max_tiles);
+      write_tiles(e, c, base + inc - c, tbase + tinc - t, tile_m, tile_expert, tile_desc, max_tiles);
     }
     carry += tot; tcarry += ttot;
     __syncthreads();
@@ -219,12 +228,12 @@ int permute_launch(hipStream_t st, const int32_t *ids, int T, int K, int E, int 
   const int TK = T * K;
   if (TK <= kChunk) {
     permute_small_kernel<<<1, kChunk, 0, st>>>(ids, TK, E, tile_m, ws.max_tiles, sorted_slot, expert_offsets, slot_to_row,
-                                           ws.tile_prefix, ws.tile_expert);
+                                           ws.tile_prefix, ws.tile_expert, ws.tile_desc);
     return (int)hipGetLastError();
   }
   permute_count_kernel<<<ws.n_chunks, 64, 0, st>>>(ids, TK, E, ws.chunk_counts);
   permute_scan_kernel<<<1, 1024, 0, st>>>(ws.chunk_counts, ws.n_chunks, E, tile_m, ws.max_tiles, expert_offsets,
-                                          ws.tile_prefix, ws.tile_expert);
+                                          ws.tile_prefix, ws.tile_expert, ws.tile_desc);
   permute_scatter_kernel<<<ws.n_chunks, kChunk, 0, st>>>(ids, TK, E, ws.chunk_counts, expert_offsets, sorted_slot,
                                                      slot_to_row);
   return (int)hipGetLastError();
