@@ -164,6 +164,18 @@ int moe_weighted_reduce(void *stream, const void *y_bf16, const float *routing_w
                         const void *shared_y_bf16, int T, int K, int H, void *out_bf16);
 
 /*
+ * The same expert computation on un-quantised weights: the reference's op with its scale arguments
+ * absent (fusedMoE.cpp:117-236 with gate/up/down_scales undefined; python/test/fused_moe_bf16.py:113-122).
+ * x [T,H] bf16, w13 [E,2I,H] bf16 (gate rows, then up rows), w2 [E,H,I] bf16; products in bf16 matrix
+ * instructions with fp32 accumulation, bf16 intermediate.  H and I multiples of 128, no shared expert.
+ */
+size_t moe_fused_experts_bf16_workspace_bytes(int T, int H, int I, int E, int K);
+int moe_fused_experts_bf16(void *stream, const void *x_bf16, int T, int H, const void *w13_bf16,
+                           const void *w2_bf16, int I, int E, const int32_t *ids,
+                           const float *routing_weights, int K, void *out_bf16, int out_mode,
+                           void *workspace, size_t workspace_bytes);
+
+/*
  * Dense block-scaled FP8 layers: the same kernels with a single "expert" that owns every row.
  *
  * moe_mm_fp8 replaces at::mm_w8a16_dq_forward -> tpudnnMmW8A16DqAsync

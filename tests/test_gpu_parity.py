@@ -522,3 +522,44 @@ def test_full_size_properties_skewed_load(pkg, oracle, dev):
     counts = (off_ref[1:] - off_ref[:-1])
     assert int((counts == 0).sum()) >= 13 and int(counts.max()) > 8000
     _full_size_checks(pkg, oracle, dev, x, layer, ids, w, torch.tensor([0, 5000, 11111, 16383]))
+
+
+# ----------------------------------------------------------------------------- un-quantised experts
+@pytest.mark.parametrize("T,H,I,E,K", [(1, 7168, 256, 1, 1), (1, 7168, 256, 16, 8), (1, 7168, 256, 256, 8),
+                                       (2, 4096, 384, 2, 2), (8, 4096, 384, 128, 8), (22, 4096, 384, 128, 8),
+                                       (300, 512, 256, 8, 2), (2000, 256, 128, 4, 2)])
+def test_experts_with_bf16_weights(pkg, oracle, dev, T, H, I, E, K):
+    """The reference's op with the scale arguments absent (python/test/fused_moe_bf16.py:148-208: its shape grid and
+    data recipe - everything N(0,1) - plus two larger batches for the big tiles), against the reference's bf16
+    chain; its criterion is cos_diff <= 1e-4."""
+    say("bf16 experts", T, H, I, E, K)
+    g = torch.Generator().manual_seed(1000 + T + E)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    w0 = torch.randn(E, I, H, generator=g).to(torch.bfloat16)
+    w1 = torch.randn(E, I, H, generator=g).to(torch.bfloat16)
+    w2 = torch.randn(E, H, I, generator=g).to(torch.bfloat16)
+    ids, w = distinct_ids(T, E, K, seed=T + 7)
+    out = torch.empty(T, K, H, dtype=torch.bfloat16, device=dev)
+    r = torch.ops.my_ops.fused_moe_fused_experts(
+        out, x.to(dev), None, None, w0.to(dev), w1.to(dev), w2.transpose(1, 2).to(dev), None, None, None,
+        ids.to(dev), w.to(torch.bfloat16).to(dev), None, None, None, 128, E, K, False, 1, 1, None, None, None, False)
+    torch.cuda.synchronize()
+    assert r.data_ptr() == out.data_ptr()
+    got = out.float().cpu()
+    assert torch.isfinite(got).all()
+    ref = oracle.experts_ref_bf16(x, ids, w0, w1, w2, None, None, None).float()
+    cos_diff = oracle.cal_diff(ref, got)[0]
+    assert cos_diff <= 1e-4, cos_diff
+    # element-wise: the chain rounds to bf16 three times (two linears, one product) where the kernel keeps fp32
+    # until the intermediate, so a few bf16 steps of the row's scale are allowed
+    rms = ref.pow(2).mean().sqrt()
+    assert ((got - ref).abs() <= 3e-2 * ref.abs() + 3e-2 * rms).float().mean() > 0.999
+    # weighted form
+    out2 = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    torch.ops.my_ops.fused_moe_fused_experts(
+        out2, x.to(dev), None, None, w0.to(dev), w1.to(dev), w2.transpose(1, 2).to(dev), None, None, None,
+        ids.to(dev), w.to(torch.bfloat16).to(dev), None, None, None, 128, E, K, False, 1, 1, None, None, None, False)
+    torch.cuda.synchronize()
+    want = torch.einsum("tk,tkh->th", w.to(torch.bfloat16).float(), got)
+    rms2 = want.pow(2).mean().sqrt()
+    assert ((out2.float().cpu() - want).abs() <= 2e-2 * want.abs() + 2e-2 * rms2).all()

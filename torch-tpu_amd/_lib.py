@@ -32,6 +32,9 @@ SIGNATURES = {
     "moe_gemm2": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
                           c_void_p, c_void_p, c_void_p, c_void_p]),
     "moe_weighted_reduce": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "moe_fused_experts_bf16_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
+    "moe_fused_experts_bf16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
+                                       c_void_p, c_int, c_void_p, c_int, c_void_p, c_size_t]),
     "moe_mm_fp8_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "moe_mm_fp8": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_size_t]),
     "moe_mlp_fp8_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),

@@ -10,11 +10,11 @@ int permute_launch(hipStream_t st, const int32_t *ids, int T, int K, int E, int 
 int gemm1_launch(hipStream_t st, const uint8_t *xq, const float *xs, int T, int H, const uint8_t *w13,
                  const float *w13s, int I, int E, int K, const int32_t *sorted_slot, const int32_t *expert_offsets,
                  const PermuteWs *pw, int fixed_expert, uint8_t *hq, float *hs, const uint8_t *sh_w13,
-                 const float *sh_w13s, uint8_t *sh_hq, float *sh_hs);
+                 const float *sh_w13s, uint8_t *sh_hq, float *sh_hs, bool bf16 = false);
 int gemm2_launch(hipStream_t st, const uint8_t *hq, const float *hs, int rows_a, int T, int H, const uint8_t *w2,
                  const float *w2s, int I, int E, int K, const int32_t *sorted_slot, const int32_t *expert_offsets,
                  const PermuteWs *pw, int fixed_expert, uint16_t *y, const uint8_t *sh_hq, const float *sh_hs,
-                 int sh_rows, const uint8_t *sh_w2, const float *sh_w2s, uint16_t *sh_y);
+                 int sh_rows, const uint8_t *sh_w2, const float *sh_w2s, uint16_t *sh_y, bool bf16 = false);
 
 size_t dense_small_partial_bytes(int M, int K, int N, bool keep_partial);
 int dense_small_launch(hipStream_t st, const uint8_t *xq, const float *xs, int M, int K, const uint8_t *w, const float *ws,
@@ -241,4 +241,71 @@ extern "C" int moe_mlp_fp8(void *stream, const void *x_bf16, int M, int H, const
   if (rc) return rc;
   return gemm2_launch(st, d.hq, d.hs, M, M, H, w2, w2_scale, I, 1, 1, nullptr, nullptr, nullptr, 0, (uint16_t *)out_bf16,
                       nullptr, nullptr, 0, nullptr, nullptr, nullptr);
+}
+
+// ---- un-quantised experts: bf16 weights, bf16 activations, no scales ----
+
+namespace moe {
+struct Bf16Ws {
+  void *permute;
+  int32_t *sorted_slot, *expert_offsets, *slot_to_row;
+  uint16_t *h, *y;
+  size_t bytes;
+};
+static Bf16Ws bf16_layout(void *base, int T, int H, int I, int E, int K) {
+  Bf16Ws w{};
+  size_t off = 0;
+  auto take = [&](size_t n) {
+    void *p = base ? (void *)((uint8_t *)base + off) : nullptr;
+    off += align_up(n ? n : 1, 256);
+    return p;
+  };
+  const size_t TK = (size_t)T * K;
+  w.permute = take(permute_ws_bytes(T, K, E));
+  w.sorted_slot = (int32_t *)take(TK * 4);
+  w.expert_offsets = (int32_t *)take((size_t)(E + 1) * 4);
+  w.slot_to_row = (int32_t *)take(TK * 4);
+  w.h = (uint16_t *)take(TK * I * 2);
+  w.y = (uint16_t *)take(TK * H * 2);
+  w.bytes = off;
+  return w;
+}
+}  // namespace moe
+
+extern "C" size_t moe_fused_experts_bf16_workspace_bytes(int T, int H, int I, int E, int K) {
+  if (T < 0 || H < 1 || I < 1 || E < 1 || K < 1) return 0;
+  return moe::bf16_layout(nullptr, T, H, I, E, K).bytes;
+}
+
+extern "C" int moe_fused_experts_bf16(void *stream, const void *x_bf16, int T, int H, const void *w13_bf16,
+                                      const void *w2_bf16, int I, int E, const int32_t *ids,
+                                      const float *routing_weights, int K, void *out_bf16, int out_mode,
+                                      void *workspace, size_t workspace_bytes) {
+  using namespace moe;
+  if (!x_bf16 || !w13_bf16 || !w2_bf16 || !ids || !out_bf16 || !workspace) return MOE_E_NULL;
+  if (out_mode != 0 && out_mode != 1) return MOE_E_MODE;
+  if (out_mode == 1 && !routing_weights) return MOE_E_NULL;
+  if (T < 0 || H < 1 || I < 1 || E < 1 || E > MOE_MAX_EXPERTS || K < 1 || K > MOE_MAX_TOPK || K > E) return MOE_E_SHAPE;
+  if ((long)T * K > (1l << 30) || H > 16384 || I > 16384) return MOE_E_SHAPE;
+  if (H % kBlock || I % kBlock) return MOE_E_ALIGN;
+  if ((double)T * H * 2 >= 2147483648.0 || (double)T * K * I * 2 >= 2147483648.0) return MOE_E_SHAPE;
+  if (((uintptr_t)workspace % 256) || ((uintptr_t)x_bf16 % 16) || ((uintptr_t)out_bf16 % 16) ||
+      ((uintptr_t)w13_bf16 % 16) || ((uintptr_t)w2_bf16 % 16))
+    return MOE_E_ALIGN;
+  Bf16Ws w = bf16_layout(workspace, T, H, I, E, K);
+  if (workspace_bytes < w.bytes) return MOE_E_WORKSPACE;
+  if (T == 0) return MOE_OK;
+  hipStream_t st = (hipStream_t)stream;
+  PermuteWs pw = permute_ws_layout(w.permute, T, K, E);
+  int rc = permute_launch(st, ids, T, K, E, choose_tile_m(T, K, E), w.sorted_slot, w.expert_offsets, w.slot_to_row, pw);
+  if (rc) return rc;
+  rc = gemm1_launch(st, (const uint8_t *)x_bf16, nullptr, T, H, (const uint8_t *)w13_bf16, nullptr, I, E, K, w.sorted_slot,
+                    w.expert_offsets, &pw, -1, (uint8_t *)w.h, nullptr, nullptr, nullptr, nullptr, nullptr, true);
+  if (rc) return rc;
+  uint16_t *y = out_mode == 0 ? (uint16_t *)out_bf16 : w.y;
+  rc = gemm2_launch(st, (const uint8_t *)w.h, nullptr, T * K, T, H, (const uint8_t *)w2_bf16, nullptr, I, E, K,
+                    w.sorted_slot, w.expert_offsets, &pw, -1, y, nullptr, nullptr, 0, nullptr, nullptr, nullptr, true);
+  if (rc) return rc;
+  if (out_mode == 0) return MOE_OK;
+  return moe_weighted_reduce(stream, y, routing_weights, nullptr, T, K, H, out_bf16);
 }

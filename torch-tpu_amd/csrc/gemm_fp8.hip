@@ -111,10 +111,32 @@ __device__ __forceinline__ v8i concat8(v4i lo, v4i hi) {
   return r;
 }
 
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+
+// bf16 operands: the two 16-byte chunks a lane holds of a 128-byte step are the lane's share of two
+// 32-element matrix instructions; all first halves are issued before the second halves so that an
+// accumulator is not needed again right away
+template <int WT>
+__device__ __forceinline__ void mma_bf16(v4f (&acc)[WT], const v8i (&w)[WT], const v8i &x) {
+  const v4i xl = {x[0], x[1], x[2], x[3]}, xh = {x[4], x[5], x[6], x[7]};
+#pragma unroll
+  for (int j = 0; j < WT; j++) {
+    const v4i wl = {w[j][0], w[j][1], w[j][2], w[j][3]};
+    acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wl), __builtin_bit_cast(v8bf, xl), acc[j], 0, 0, 0);
+  }
+#pragma unroll
+  for (int j = 0; j < WT; j++) {
+    const v4i wh = {w[j][4], w[j][5], w[j][6], w[j][7]};
+    acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wh), __builtin_bit_cast(v8bf, xh), acc[j], 0, 0, 0);
+  }
+}
+
 // MT     token m-tiles (of 16 rows) per workgroup
 // NW     wavefronts per workgroup (4 or 8); each owns WT = 16 / NW of the strip's 16 weight tiles
 // DEPTH  128-steps of weights kept in flight per wavefront (register ring)
-template <int MT, int NW, int DEPTH, bool GATED, bool WREG>
+// BF16   un-quantised mode: both operands are bf16 (a 128-byte step is 64 elements = two
+//        v_mfma_f32_16x16x32_bf16 accumulating in place), no scales, bf16 intermediate
+template <int MT, int NW, int DEPTH, bool GATED, bool WREG, bool BF16 = false>
 __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a) {
   constexpr int BM = 16 * MT;
   constexpr int NT = 64 * NW;                         // threads
@@ -238,7 +260,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   // The strip's weight-block scales for all steps go to LDS once (two rows: gate/up blocks for
   // the gated GEMM, the strip's two 128-column blocks otherwise): uniform values re-read per
   // step from LDS instead of through the vector-memory queue.
-  {
+  if constexpr (!BF16) {
     const int blk0 = GATED ? strip : min(strip * 2, n_wblk - 1);
     const int blk1 = GATED ? (a.N >> 7) + strip : min(strip * 2 + 1, n_wblk - 1);
     for (int i = tid; i < 2 * NKB; i += NT) {
@@ -317,6 +339,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     for (int j = 0; j < WT; j++) asm volatile("" : "+v"(lo[j]), "+v"(hi[j]));
   };
   auto request_scales = [&](int chunk) {
+    if constexpr (BF16) return;
 #pragma unroll
     for (int u = 0; u < NSC; u++) {
       const float *base = as + chunk * 16;
@@ -356,7 +379,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
       if (WREG) wc[j] = concat8(lo[j], hi[j]);
       else wc[j] = concat8(*(const v4i *)(wbase + j * 2048), *(const v4i *)(wbase + j * 2048 + 1024));
     }
-    const float s0 = sm.sb[sb_row0][kb], s1 = sm.sb[sb_row1][kb];
+    const float s0 = BF16 ? 0.f : sm.sb[sb_row0][kb], s1 = BF16 ? 0.f : sm.sb[sb_row1][kb];
     const uint8_t *tbase = sm.tok[stage] + li * 128;
     const int o0 = (lg ^ (li & 7)) << 4, o1 = ((lg + 4) ^ (li & 7)) << 4;
     const float *sap = sm.sac[(kb >> 4) & 1] + ((kb & 12) << 4) + li * 4 + (kb & 3);
@@ -369,9 +392,15 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
         for (int mi = 0; mi < MG; mi++) {
           const int mt = mg * MG + mi;
           x[mi] = concat8(*(const v4i *)(tbase + mt * 2048 + o0), *(const v4i *)(tbase + mt * 2048 + o1));
-          sa_[mi] = sap[mt * 256];
+          sa_[mi] = BF16 ? 0.f : sap[mt * 256];
         }
         __builtin_amdgcn_sched_barrier(0);
+        if constexpr (BF16) {
+#pragma unroll
+          for (int mi = 0; mi < MG; mi++) mma_bf16<WT>(acc[mg * MG + mi], wc, x[mi]);
+          __builtin_amdgcn_sched_barrier(0);
+          continue;
+        }
         v4f p[MG][WT];
 #pragma unroll
         for (int mi = 0; mi < MG; mi++) {
@@ -466,6 +495,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
       // forms both products of a step once, two steps ahead, instead of every wavefront forming them
       // for every m-tile (one multiply less per matrix instruction on the shared issue port).
       auto produce_f = [&](int k) {
+        if constexpr (BF16) return;
         if (tid < BM) {
           const int kc = min(k, last);                   // past the end: a finite scale times the zero behind the table
           const float sa = sm.sac[(kc >> 4) & 1][(tid >> 4) * 256 + ((kc & 12) << 4) + (tid & 15) * 4 + (kc & 3)];
@@ -482,6 +512,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
       };
       // GATED: both products (gate tiles use .x, up tiles .y); second GEMM: the one of this wavefront's column block
       auto read_f = [&](int kb, int mt) {
+        if (BF16) return make_float2(0.f, 0.f);
         if (GATED) return sm.fsc[kb & 3][mt * 16 + li];
         const float f = ((const float *)&sm.fsc[kb & 3][mt * 16 + li])[sb_row0];
         return make_float2(f, f);
@@ -516,6 +547,11 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
               const int kk = q + PD < LIVE ? kb : kb + 1;
               x[(g + PD) % XB] = read_x(kk, LIVE - 1 - qq);
               fb[(g + PD) % XB] = read_f(kk, LIVE - 1 - qq);
+            }
+            if constexpr (BF16) {                        // accumulates in place: nothing is pending afterwards
+              mma_bf16<WT>(acc[LIVE - 1 - q], wc, x[g % XB]);
+              __builtin_amdgcn_sched_barrier(0);
+              return;
             }
 #pragma unroll
             for (int j = 0; j < WT; j++) {
@@ -578,7 +614,28 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   __syncthreads();
 
   // ---- epilogue -------------------------------------------------------------------------------
-  if (GATED) {
+  if (GATED && BF16) {
+    constexpr int G = WT / 2;                          // gate tiles per wavefront
+    uint16_t *const h = (uint16_t *)(shared ? a.sh_hq : a.hq);
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) {
+      const int i = mt * 16 + li;
+      if (i >= rows) continue;
+#pragma unroll
+      for (int j = 0; j < G; j++) {
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const float g = acc[mt][j][r], u = acc[mt][j + G][r];
+          v[r] = (g / (1.0f + expf(-g))) * u;
+        }
+        v2i o;
+        o[0] = (int)((uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16));
+        o[1] = (int)((uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16));
+        *(v2i *)(h + (size_t)(row0 + i) * a.N + strip * 128 + wave * (16 * G) + j * 16 + lg * 4) = o;
+      }
+    }
+  } else if (GATED) {
     constexpr int G = WT / 2;                          // gate tiles per wavefront
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
@@ -638,7 +695,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
 
 // Launch shape per tile height.  Eight wavefronts (two per SIMD, two weight tiles each) keep
 // more loads in flight for the bandwidth-bound shapes.
-template <bool GATED>
+template <bool GATED, bool BF16 = false>
 static int launch_gemm(hipStream_t st, GemmArgs &a, int tile_m, int max_mtiles) {
   a.n_strips = GATED ? a.N / 128 : (a.N + 255) / 256;
   a.max_mtiles = max_mtiles - (a.sh_rows + tile_m - 1) / tile_m;
@@ -647,7 +704,7 @@ static int launch_gemm(hipStream_t st, GemmArgs &a, int tile_m, int max_mtiles) 
   if (total <= 0 || total > 0x7fffffffl) return MOE_E_SHAPE;
   a.total_blocks = (int)total;
   dim3 grid((unsigned)total);
-#define MOE_GEMM(MT, NW, D, WREG) grouped_gemm_kernel<MT, NW, D, GATED, WREG><<<grid, dim3(64 * NW), 0, st>>>(a)
+#define MOE_GEMM(MT, NW, D, WREG) grouped_gemm_kernel<MT, NW, D, GATED, WREG, BF16><<<grid, dim3(64 * NW), 0, st>>>(a)
   // small tiles: both operands through LDS (few registers, deeper pipeline); large tiles: weights in
   // a register ring so that LDS holds three stages of the bigger token tile
   switch (tile_m) {
@@ -678,7 +735,7 @@ static int check_dims(int T, int H, int I, int E, int K) {
 int gemm1_launch(hipStream_t st, const uint8_t *xq, const float *xs, int T, int H, const uint8_t *w13,
                  const float *w13s, int I, int E, int K, const int32_t *sorted_slot, const int32_t *expert_offsets,
                  const PermuteWs *pw, int fixed_expert, uint8_t *hq, float *hs, const uint8_t *sh_w13,
-                 const float *sh_w13s, uint8_t *sh_hq, float *sh_hs) {
+                 const float *sh_w13s, uint8_t *sh_hq, float *sh_hs, bool bf16) {
   GemmArgs a{};
   if (sh_w13) { a.sh_aq = xq; a.sh_as = xs; a.sh_w = sh_w13; a.sh_ws = sh_w13s; a.sh_hq = sh_hq; a.sh_hs = sh_hs; a.sh_rows = T; }
   a.aq = xq; a.as = xs; a.w = w13; a.ws = w13s;
@@ -687,16 +744,17 @@ int gemm1_launch(hipStream_t st, const uint8_t *xq, const float *xs, int T, int 
   a.tile_desc = pw ? pw->tile_desc : nullptr;
   a.hq = hq; a.hs = hs; a.y = nullptr;
   a.as_pitch = scale_pitch(H / kBlock); a.hs_pitch = scale_pitch(I / kBlock);
-  a.Kd = H; a.N = I; a.n_rows_w = 2 * I; a.rows_a = T; a.topk = K; a.E = E; a.fixed_expert = fixed_expert;
+  a.Kd = bf16 ? 2 * H : H; a.N = I; a.n_rows_w = 2 * I; a.rows_a = T; a.topk = K; a.E = E; a.fixed_expert = fixed_expert;
   const int tile_m = choose_tile_m(T, K, E);
   const int max_mtiles = fixed_expert >= 0 ? (T + tile_m - 1) / tile_m : pw->max_tiles;
+  if (bf16) return launch_gemm<true, true>(st, a, tile_m, max_mtiles + (a.sh_rows + tile_m - 1) / tile_m);
   return launch_gemm<true>(st, a, tile_m, max_mtiles + (a.sh_rows + tile_m - 1) / tile_m);
 }
 
 int gemm2_launch(hipStream_t st, const uint8_t *hq, const float *hs, int rows_a, int T, int H, const uint8_t *w2,
                  const float *w2s, int I, int E, int K, const int32_t *sorted_slot, const int32_t *expert_offsets,
                  const PermuteWs *pw, int fixed_expert, uint16_t *y, const uint8_t *sh_hq, const float *sh_hs,
-                 int sh_rows, const uint8_t *sh_w2, const float *sh_w2s, uint16_t *sh_y) {
+                 int sh_rows, const uint8_t *sh_w2, const float *sh_w2s, uint16_t *sh_y, bool bf16) {
   GemmArgs a{};
   if (sh_w2) { a.sh_aq = sh_hq; a.sh_as = sh_hs; a.sh_w = sh_w2; a.sh_ws = sh_w2s; a.sh_y = sh_y; a.sh_rows = sh_rows; }
   a.aq = hq; a.as = hs; a.w = w2; a.ws = w2s;
@@ -705,9 +763,10 @@ int gemm2_launch(hipStream_t st, const uint8_t *hq, const float *hs, int rows_a,
   a.tile_desc = pw ? pw->tile_desc : nullptr;
   a.hq = nullptr; a.hs = nullptr; a.y = y;
   a.as_pitch = scale_pitch(I / kBlock); a.hs_pitch = 0;
-  a.Kd = I; a.N = H; a.n_rows_w = H; a.rows_a = rows_a; a.topk = K; a.E = E; a.fixed_expert = fixed_expert;
+  a.Kd = bf16 ? 2 * I : I; a.N = H; a.n_rows_w = H; a.rows_a = rows_a; a.topk = K; a.E = E; a.fixed_expert = fixed_expert;
   const int tile_m = choose_tile_m(T, K, E);
   const int max_mtiles = fixed_expert >= 0 ? (rows_a + tile_m - 1) / tile_m : pw->max_tiles;
+  if (bf16) return launch_gemm<false, true>(st, a, tile_m, max_mtiles + (a.sh_rows + tile_m - 1) / tile_m);
   return launch_gemm<false>(st, a, tile_m, max_mtiles + (a.sh_rows + tile_m - 1) / tile_m);
 }
 
@@ -726,7 +785,7 @@ extern "C" int moe_gemm1_swiglu(void *stream, const uint8_t *xq, const float *xs
   if (T == 0) return MOE_OK;
   PermuteWs pw = permute_ws_layout(const_cast<void *>(permute_workspace), T, K, E);
   return gemm1_launch((hipStream_t)stream, xq, xs, T, H, w13, w13_scale, I, E, K, sorted_slot, expert_offsets, &pw, -1,
-                      hq, hs, nullptr, nullptr, nullptr, nullptr);
+                      hq, hs, nullptr, nullptr, nullptr, nullptr, false);
 }
 
 extern "C" int moe_gemm2(void *stream, const uint8_t *hq, const float *hs, int T, int H, const uint8_t *w2,
@@ -741,5 +800,5 @@ extern "C" int moe_gemm2(void *stream, const uint8_t *hq, const float *hs, int T
   if (T == 0) return MOE_OK;
   PermuteWs pw = permute_ws_layout(const_cast<void *>(permute_workspace), T, K, E);
   return gemm2_launch((hipStream_t)stream, hq, hs, T * K, T, H, w2, w2_scale, I, E, K, sorted_slot, expert_offsets, &pw,
-                      -1, (uint16_t *)y_bf16, nullptr, nullptr, 0, nullptr, nullptr, nullptr);
+                      -1, (uint16_t *)y_bf16, nullptr, nullptr, 0, nullptr, nullptr, nullptr, false);
 }

@@ -41,6 +41,20 @@ _lib.define("mm_w8a16_dq_forward(Tensor input, Tensor weight, Tensor scale, Tens
 _pack_cache: dict = {}
 
 
+_dense_cache: dict = {}
+
+
+def _dense_packed(key_tensors, make):
+    key = tuple((t.data_ptr(), t._version, tuple(t.shape), tuple(t.stride())) for t in key_tensors)
+    hit = _dense_cache.get(key)
+    if hit is None:
+        if len(_dense_cache) > 32:
+            _dense_cache.clear()
+        hit = make()
+        _dense_cache[key] = hit
+    return hit
+
+
 def _packed(gate, up, down, gs, us, ds):
     key = tuple((t.data_ptr(), t._version, tuple(t.shape)) for t in (gate, up, down, gs, us, ds))
     hit = _pack_cache.get(key)
@@ -67,8 +81,21 @@ def _fused_experts(output, input, output_sample, input_sample, gate_weights, up_
                                "undefined; it is not supported")
     if save_mid_res:
         raise RuntimeError("save_mid_res is not supported")
+    if gate_scales is None and up_scales is None and down_scales is None:
+        # un-quantised experts (python/test/fused_moe_bf16.py:113-122): bf16 weights, same op
+        for t in (gate_weights, up_weights, down_weights):
+            if t.dtype != torch.bfloat16:
+                raise RuntimeError("weights without scales must be bfloat16")
+        w13, w2 = _dense_packed((gate_weights, up_weights, down_weights),
+                                lambda: (torch.cat([gate_weights, up_weights], dim=1).contiguous(),
+                                         down_weights.transpose(1, 2).contiguous()))
+        if w13.shape[0] != num_experts or select_experts.shape[1] != num_experts_per_tok:
+            raise RuntimeError("num_experts / num_experts_per_tok do not match the tensors")
+        rw = routing_weights.to(torch.float32) if output.dim() == 2 else None
+        ops.fused_experts_bf16(input, w13, w2, select_experts, rw, out=output)
+        return output
     if gate_scales is None or up_scales is None or down_scales is None:
-        raise RuntimeError("bf16 (un-quantised) expert weights are not supported: pass fp8 weights with block scales")
+        raise RuntimeError("either all three weight tensors carry block scales or none does")
     if blocksize != 128:
         raise RuntimeError("blocksize must be 128")
     w13, w13s, w2, w2s = _packed(gate_weights, up_weights, down_weights, gate_scales, up_scales, down_scales)
@@ -96,20 +123,6 @@ def _fused_experts_v2(output, input, output_sample, input_sample, gate_weights, 
 def _grouped_topk(*args):
     raise RuntimeError("fused_moe_grouped_topk: the reference's fused router is closed-source, untested and "
                        "undocumented; use noaux_tc_topk or torch_tpu_amd.moe_route instead")
-
-
-_dense_cache: dict = {}
-
-
-def _dense_packed(key_tensors, make):
-    key = tuple((t.data_ptr(), t._version, tuple(t.shape), tuple(t.stride())) for t in key_tensors)
-    hit = _dense_cache.get(key)
-    if hit is None:
-        if len(_dense_cache) > 32:
-            _dense_cache.clear()
-        hit = make()
-        _dense_cache[key] = hit
-    return hit
 
 
 def _check_dense(blocksize, *fp8):
