@@ -331,6 +331,18 @@ def test_my_ops_drop_in_reference_layout(pkg, oracle, dev):
     torch.ops.my_ops.fused_moe_fused_experts_v2(*args, scratch[0], scratch[1], scratch[2], scratch[3], *tail)
     torch.cuda.synchronize()
     assert torch.equal(out.float().cpu(), got)
+    # the reference's own arithmetic (weights de-quantised into bf16, bf16 activations) meets the reference's own
+    # criterion, cos_sim > 0.99 and cos_diff < 1e-4 (test_moe.py:308)
+    pkg.set_expert_numerics("w8a16")
+    try:
+        out.zero_()
+        torch.ops.my_ops.fused_moe_fused_experts(*args, scratch[0], scratch[1], *tail)
+        torch.cuda.synchronize()
+    finally:
+        pkg.set_expert_numerics("w8a8")
+    got16 = out.float().cpu()
+    assert oracle.cos_sim(ref_bf16.numpy(), got16.numpy()) > 0.99
+    assert oracle.cal_diff(ref_bf16, got16)[0] < 1e-4
 
 
 def test_layer_module_end_to_end_toy_config(pkg, oracle, dev):

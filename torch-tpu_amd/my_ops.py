@@ -37,6 +37,29 @@ _lib.define("mlp_w8a16_dq_forward(Tensor input, Tensor gate_weight, Tensor up_we
 _lib.define("mm_w8a16_dq_forward(Tensor input, Tensor weight, Tensor scale, Tensor(a!) output, int blocksize) "
             "-> Tensor(a!)")
 
+# How quantised expert weights are multiplied.  "w8a8" (default): activations are quantised to FP8 per
+# token and 128 columns and the products run on the FP8 matrix path - the path this package is about.
+# "w8a16": the reference's own arithmetic (python/regression/test_llm/test_moe.py:10-98) - weights are
+# de-quantised ONCE into bf16 (bf16(fp8) * bf16 scale, cached, twice the bytes) and the un-quantised
+# kernels run on bf16 activations; meant for validating against the reference's criterion
+# (cos_diff < 1e-4, test_moe.py:308), not for serving.
+_numerics = "w8a8"
+
+
+def set_expert_numerics(mode: str) -> None:
+    global _numerics
+    if mode not in ("w8a8", "w8a16"):
+        raise ValueError("mode must be 'w8a8' or 'w8a16'")
+    _numerics = mode
+
+
+def _dequant_bf16(w, s):
+    """[E, N, K] fp8 with [E, ceil(N/128), ceil(K/128)] scales -> bf16, as the reference's weight_dequant does."""
+    E, N, K = w.shape
+    full = s.to(torch.bfloat16).repeat_interleave(128, dim=1)[:, :N].repeat_interleave(128, dim=2)[:, :, :K]
+    return (w.to(torch.float32) * full.to(torch.float32)).to(torch.bfloat16)
+
+
 # packed copies of reference-layout weights, keyed by the identity of the six tensors
 _pack_cache: dict = {}
 
@@ -98,6 +121,14 @@ def _fused_experts(output, input, output_sample, input_sample, gate_weights, up_
         raise RuntimeError("either all three weight tensors carry block scales or none does")
     if blocksize != 128:
         raise RuntimeError("blocksize must be 128")
+    if _numerics == "w8a16":
+        w13, w2 = _dense_packed(
+            (gate_weights, up_weights, down_weights, gate_scales, up_scales, down_scales),
+            lambda: (torch.cat([_dequant_bf16(gate_weights, gate_scales), _dequant_bf16(up_weights, up_scales)], 1).contiguous(),
+                     _dequant_bf16(down_weights, down_scales).transpose(1, 2).contiguous()))
+        rw = routing_weights.to(torch.float32) if output.dim() == 2 else None
+        ops.fused_experts_bf16(input, w13, w2, select_experts, rw, out=output)
+        return output
     w13, w13s, w2, w2s = _packed(gate_weights, up_weights, down_weights, gate_scales, up_scales, down_scales)
     if w13.shape[0] != num_experts or select_experts.shape[1] != num_experts_per_tok:
         raise RuntimeError("num_experts / num_experts_per_tok do not match the tensors")
