@@ -16,12 +16,17 @@
 //                         this split makes the 128-bit LDS reads of the token tile conflict-free)
 //   lane l of the result: c[r] = (weight row 4*(l / 16) + r, token l % 16)
 //
-// Data movement per step: the token tile is shared by all wavefronts and goes HBM/L2 -> LDS
-// with direct-to-LDS loads (no registers held while in flight, XOR swizzle applied on the source
-// side) through DEPTH + 1 stages; each wavefront's WT = 16 / NW weight tiles are used by nobody
-// else and go HBM -> registers in operand layout through a DEPTH-deep register ring (WREG) or,
-// for small row tiles, -> LDS the same way as the tokens.  Requests run DEPTH steps ahead of
-// the matrix work and are waited for with hand-placed s_waitcnt; one barrier per step.
+// Data movement per step: the token tile is shared by all wavefronts and goes L2 -> LDS with
+// direct-to-LDS loads (no registers held while in flight, XOR swizzle applied on the source
+// side); each wavefront's WT = 16 / NW weight tiles are used by nobody else and go HBM ->
+// registers in operand layout through a two-step register ring (WREG, row tiles of 128 / 192)
+// or, for small row tiles, -> LDS the same way as the tokens.  Activation scales come sixteen
+// steps at a time into a double-buffered LDS table.  Requests run ahead of the matrix work and
+// are waited for with hand-placed s_waitcnt; one barrier per step.  The large-tile loop is one
+// software pipeline over all m-tiles of all steps (see the loop itself).
+//
+// BF16 = true: the same tiles and pipelines on un-quantised operands (no scales, two
+// v_mfma_f32_16x16x32_bf16 per 128-byte step accumulating in place, bf16 intermediate).
 //
 // GATED = true  (first GEMM): the strip is 128 gate columns plus the 128 matching up columns of
 //   W13; wavefront w owns gate columns 16w..16w+15 and the same up columns.  Epilogue:
@@ -88,9 +93,6 @@ struct GemmSmem {
   float sb[2][kMaxKB + 4];                       // weight-block scales of the strip for every 128-step, then zeros
 };
 
-#ifndef MOE_W_MOD
-#define MOE_W_MOD ""
-#endif
 typedef __attribute__((address_space(3))) uint8_t lds_byte;
 // byte offset of a __shared__ object inside the workgroup's LDS allocation (what M0 wants)
 __device__ __forceinline__ uint32_t lds_offset(const void *p) { return (uint32_t)(uintptr_t)(lds_byte *)p; }
@@ -232,9 +234,6 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     const int p = row0 + min(i, rows - 1);
     int src = p;
     if (GATED && !direct) src = a.sorted_slot[p] / a.topk;
-#ifdef MOE_DBG_SAMETOK
-    src = i;
-#endif
     sm.arow[i] = min(max(src, 0), rows_a - 1);
     if (!GATED) sm.oslot[i] = direct ? p : a.sorted_slot[p];      // output row (slot) of each tile row
   }
@@ -330,7 +329,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
 #pragma unroll
     for (int j = 0; j < WT; j++) {
       const uint8_t *base = wtile[j] + (size_t)kb * 128;
-      asm volatile("global_load_dwordx4 %0, %2, %3" MOE_W_MOD "\n\tglobal_load_dwordx4 %1, %2, %3 offset:64" MOE_W_MOD
+      asm volatile("global_load_dwordx4 %0, %2, %3\n\tglobal_load_dwordx4 %1, %2, %3 offset:64"
                    : "=&v"(lo[j]), "=&v"(hi[j]) : "v"(woff), "s"(base) : "memory");
     }
   };
@@ -359,9 +358,9 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     for (int j = 0; j < WT; j++) {
       const uint8_t *base = wtile[j] + (size_t)kb * 128;
       const uint32_t m0 = wt_base + stage * kWtStage + j * 2048;
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" MOE_W_MOD "\n\t"
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t"
                    // the instruction offset moves the LDS address as well as the global one: 0x400 - 64
-                   "s_add_u32 m0, m0, 0x3c0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:64" MOE_W_MOD
+                   "s_add_u32 m0, m0, 0x3c0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:64"
                    ::"s"(m0), "v"(woff), "s"(base) : "memory", "m0", "scc");
     }
   };
@@ -441,9 +440,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     int kb = 0, stage = 0, stage_req = DEPTH;
     for (; kb + DEPTH < NKB; kb++) {
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 1) * L_STEP) : "memory");
-#ifndef MOE_DBG_NOBARRIER
       __syncthreads();
-#endif
       if ((kb & 15) == 0 && (kb >> 4) + 1 < n_chunks) request_scales((kb >> 4) + 1);
       request(kb + DEPTH, stage_req);
       compute(stage, kb, wlo[0], whi[0]);
@@ -570,23 +567,17 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
             }
             __builtin_amdgcn_sched_barrier(0);
           };
-#ifndef MOE_DBG_NOCOMPUTE
           tile(0, 0);
 #pragma unroll
           for (int q = 1; q < LIVE; q++) tile(q, LIVE - q);
-#endif
           // top of step kb + 1
-#if !defined(MOE_DBG_NOLOAD) && !defined(MOE_DBG_NOW)
           request_weights_reg(min(kb + R, last), wlo[h], whi[h]);
-#endif
           asm volatile("s_waitcnt vmcnt(%0)" ::"n"(L_WAIT) : "memory");
           arrived_weights(wlo[(h + 1) % R], whi[(h + 1) % R]);
           __syncthreads();
           produce_f(kb + 3);
           if (((kb + 1) & 15) == 0 && ((kb + 1) >> 4) + 1 < n_chunks) request_scales(((kb + 1) >> 4) + 1);
-#if !defined(MOE_DBG_NOLOAD) && !defined(MOE_DBG_NOTOK)
           request(min(kb + 4, last), kb & 3);
-#endif
           __builtin_amdgcn_sched_barrier(0);
         }
       }
@@ -678,11 +669,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
 #pragma unroll
       for (int j = 0; j < WT; j++) {
         const int col = strip * 256 + wave * (16 * WT) + j * 16 + lg * 4;
-#ifdef MOE_DBG_NOSTORE
-        if (valid && col < 0) {
-#else
         if (valid && col < a.N) {
-#endif
           v2i o;
           o[0] = (int)((uint32_t)f32_to_bf16(acc[mt][j][0]) | ((uint32_t)f32_to_bf16(acc[mt][j][1]) << 16));
           o[1] = (int)((uint32_t)f32_to_bf16(acc[mt][j][2]) | ((uint32_t)f32_to_bf16(acc[mt][j][3]) << 16));
@@ -712,10 +699,7 @@ static int launch_gemm(hipStream_t st, GemmArgs &a, int tile_m, int max_mtiles) 
     case 32: MOE_GEMM(2, 8, 3, false); break;
     case 64: MOE_GEMM(4, 8, 2, false); break;
     case 128: MOE_GEMM(8, 8, 2, true); break;
-    #ifndef MOE_D192
-#define MOE_D192 2
-#endif
-    case 192: MOE_GEMM(12, 8, MOE_D192, true); break;
+    case 192: MOE_GEMM(12, 8, 2, true); break;
     default: return MOE_E_SHAPE;
   }
 #undef MOE_GEMM
