@@ -327,8 +327,8 @@ def main():
     ap.add_argument("--cpu-sample", type=int, default=32)
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py measures ONE GPU: the path is single-device by design (expert-parallel sharding is "
-              "described in DESIGN.md, not built); run with --gpus 1", file=sys.stderr)
+        print("bench.py measures ONE GPU: the path is single-device by design (sharding the experts over several "
+              "GPUs is not built); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
     if not torch.cuda.is_available():
         print("bench.py needs a ROCm GPU", file=sys.stderr)
