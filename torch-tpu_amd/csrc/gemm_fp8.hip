@@ -83,7 +83,7 @@ constexpr int kMaxKB = 256;                 // reduction length limit: 256 * 128
 template <int MT, int NW, int STAGES, int WSTAGES, int WTILE = 2048>
 struct GemmSmem {
   static constexpr int BM = 16 * MT;
-  alignas(1024) uint8_t wt[WSTAGES][16 * WTILE];   // weight tiles: [tile][half][lane][16 bytes], read by their owner
+  alignas(1024) uint8_t wt[WSTAGES][16 * WTILE];   // weight tiles: [tile][row][swizzled 16-byte chunk], read by their owner
   alignas(1024) uint8_t tok[STAGES][BM * 128];   // token tiles, XOR-swizzled 16-byte chunks
   alignas(1024) float sac[2][MT * 256];          // activation scales, 16 steps at a time: [m-tile][4-step part][row][4]
   int arow[BM];                                  // source row in aq / as for each tile row
@@ -256,6 +256,8 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     wtile[j] = wq + ((size_t)e * a.n_rows_w + wrow) * a.Kd;
   }
   const uint32_t woff = (uint32_t)li * (uint32_t)a.Kd + lg * 16;   // lane's row and first 16-byte chunk in a tile
+  // direct-to-LDS weight loads: lane l fetches row l/8 (of 8) and the chunk that belongs at position l%8
+  const uint32_t wdma_off = (uint32_t)(lane >> 3) * (uint32_t)a.Kd + (((lane & 7) ^ (lane >> 3)) << 4);
   // The strip's weight-block scales for all steps go to LDS once (two rows: gate/up blocks for
   // the gated GEMM, the strip's two 128-column blocks otherwise): uniform values re-read per
   // step from LDS instead of through the vector-memory queue.
@@ -353,15 +355,17 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
       const uint32_t m0 = tok_base + stage * kTokStage + tok_m0[u];
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(tok_src[u]), "s"(base) : "memory", "m0");
     }
+    // weight tiles through LDS: like the token tile, an instruction moves 8 whole rows x 128 bytes
+    // (every cache line it touches is used completely) into swizzled [row][16-byte chunk] order
     if (!WREG)
 #pragma unroll
     for (int j = 0; j < WT; j++) {
       const uint8_t *base = wtile[j] + (size_t)kb * 128;
+      const uint8_t *base8 = base + (size_t)8 * a.Kd;
       const uint32_t m0 = wt_base + stage * kWtStage + j * 2048;
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t"
-                   // the instruction offset moves the LDS address as well as the global one: 0x400 - 64
-                   "s_add_u32 m0, m0, 0x3c0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:64"
-                   ::"s"(m0), "v"(woff), "s"(base) : "memory", "m0", "scc");
+                   "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %3"
+                   ::"s"(m0), "v"(wdma_off), "s"(base), "s"(base8) : "memory", "m0", "scc");
     }
   };
 
@@ -372,11 +376,12 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   constexpr int MG = MT < 4 ? MT : (MT % 4 == 0 && MT <= 8 ? 4 : (DEPTH >= 3 ? 2 : 3));
   auto compute = [&](int stage, int kb, const v4i(&lo)[WT], const v4i(&hi)[WT]) {
     v8i wc[WT];
-    const uint8_t *wbase = sm.wt[WREG ? 0 : stage] + wave * (WT * 2048) + lane * 16;
+    const uint8_t *wbase = sm.wt[WREG ? 0 : stage] + wave * (WT * 2048) + li * 128;
 #pragma unroll
     for (int j = 0; j < WT; j++) {
       if (WREG) wc[j] = concat8(lo[j], hi[j]);
-      else wc[j] = concat8(*(const v4i *)(wbase + j * 2048), *(const v4i *)(wbase + j * 2048 + 1024));
+      else wc[j] = concat8(*(const v4i *)(wbase + j * 2048 + ((lg ^ (li & 7)) << 4)),
+                           *(const v4i *)(wbase + j * 2048 + (((lg + 4) ^ (li & 7)) << 4)));
     }
     const float s0 = BF16 ? 0.f : sm.sb[sb_row0][kb], s1 = BF16 ? 0.f : sm.sb[sb_row1][kb];
     const uint8_t *tbase = sm.tok[stage] + li * 128;
