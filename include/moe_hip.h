@@ -198,6 +198,33 @@ int moe_mlp_fp8(void *stream, const void *x_bf16, int M, int H, const uint8_t *w
                 const uint8_t *w2, const float *w2_scale, int I, void *out_bf16, void *workspace,
                 size_t workspace_bytes);
 
+/*
+ * Router and experts of one layer in a single call, for decode-size batches: T * K <= 256 slots and
+ * E <= 256 experts (MOE_E_SHAPE beyond that - route, then moe_fused_experts_fp8, cover every size).
+ * Replaces, in one go, what the reference's callers chain on the host for every token batch
+ * (python/regression/test_llm/test_torch_ops.py:441-456: logits = x Wr^T in bf16 -> sigmoid -> top-k ->
+ * renormalise -> scale) and the expert op behind it (torch_tpu/csrc/ops/my_ops/fusedMoE.cpp:117-236).
+ * Two launches stand in front of the grouped GEMMs instead of five: the router logits (fp32 sums rounded
+ * to bf16) together with the activation quantisation, then routing and permutation.
+ * router_w_bf16 [E, H] bf16; router_bias [E] fp32 or NULL (selection only, as in moe_route_topk);
+ * mode MOE_ROUTE_SOFTMAX or MOE_ROUTE_SIGMOID; the other routing arguments as in moe_route_topk.
+ * out bf16 [T, H] (the weighted sum, shared expert added when its pointers are non-NULL).
+ * logits_out_bf16 [T, E], weights_out [T, K], ids_out [T, K]: optional copies of what the router
+ * produced (NULL to skip).  Given the same logits, ids and weights equal moe_route_topk's, and given the
+ * same ids and weights the output equals moe_fused_experts_fp8's, bit for bit.
+ * workspace: moe_decode_layer_fp8_workspace_bytes(...) bytes, 256-byte aligned.
+ */
+size_t moe_decode_layer_fp8_workspace_bytes(int T, int H, int I, int E, int K, int I_shared);
+int moe_decode_layer_fp8(void *stream, const void *x_bf16, int T, int H,
+                         const void *router_w_bf16, const float *router_bias, int E, int K, int mode,
+                         int n_groups, int topk_groups, int renorm, float scale,
+                         const uint8_t *w13, const float *w13_scale,
+                         const uint8_t *w2, const float *w2_scale, int I,
+                         const uint8_t *shared_w13, const float *shared_w13_scale,
+                         const uint8_t *shared_w2, const float *shared_w2_scale, int I_shared,
+                         void *out_bf16, void *logits_out_bf16, float *weights_out, int32_t *ids_out,
+                         void *workspace, size_t workspace_bytes);
+
 #ifdef __cplusplus
 }
 #endif

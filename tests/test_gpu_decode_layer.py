@@ -1,0 +1,201 @@
+"""Decode-size batches: the workgroup-per-token routing kernel and the one-call layer entry point
+(moe_decode_layer_fp8), through the C ABI, on a real MI355X.
+
+What must hold, bit for bit: the routing of a small batch equals the routing of the same rows inside
+a large batch (two different kernels) and the oracle's ids; given the logits the entry point produced, its
+ids and weights equal moe_route_topk's; given those, its output equals moe_fused_experts_fp8's.
+The logits themselves are a bf16 rounding of an fp32 dot product: checked against an fp64 product with
+the tolerance of that rounding.
+"""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+ROUTE_CASES = [
+    # E, K, mode, groups, kept groups, bias, ties
+    (8, 2, "softmax", 1, 1, False, False),
+    (128, 8, "softmax", 1, 1, False, True),
+    (200, 6, "softmax", 1, 1, True, False),
+    (256, 8, "sigmoid", 8, 4, True, False),
+    (256, 8, "sigmoid", 8, 4, False, True),
+    (96, 7, "sigmoid", 3, 2, True, True),
+    (64, 32, "scores", 4, 3, False, True),
+    (250, 5, "sigmoid", 1, 1, False, False),
+]
+
+
+@pytest.mark.parametrize("E,K,mode,G,TG,with_bias,ties", ROUTE_CASES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_small_batch_routing_equals_large_batch_routing(pkg, oracle, dev, E, K, mode, G, TG, with_bias, ties, dtype):
+    say("route small vs large", E, K, mode, G, TG, with_bias, ties, dtype)
+    T = 150                                            # above the small-batch limit: one wavefront per token
+    g = torch.Generator().manual_seed(E * 31 + K)
+    logits = torch.randn(T, E, generator=g) * 1.5
+    if mode == "scores":
+        logits = torch.rand(T, E, generator=g)
+    if ties:
+        logits[::2] = torch.round(logits[::2] * 2) / 2  # many exact ties, in the groups' sums as well
+        logits[3] = 0.25                                # one row of a single value
+    logits = logits.to(dtype).to(dev)
+    bias = (torch.randn(E, generator=g) * 0.1).to(dev) if with_bias else None
+    kw = dict(bias=bias, n_groups=G, topk_groups=TG, renorm=True, scale=2.5, return_scores=True)
+    w_big, i_big, s_big = pkg.moe_route(logits, K, mode, **kw)
+    for lo, n in ((0, 1), (1, 7), (8, 64), (100, 50)):
+        w, i, s = pkg.moe_route(logits[lo:lo + n].contiguous(), K, mode, **kw)
+        assert torch.equal(i, i_big[lo:lo + n]), (lo, n)
+        assert torch.equal(w, w_big[lo:lo + n]), (lo, n)
+        assert torch.equal(s, s_big[lo:lo + n]), (lo, n)
+    w_nr, i_nr = pkg.moe_route(logits[:9].contiguous(), K, mode, bias=bias, n_groups=G, topk_groups=TG, renorm=False)
+    w_nr_big, i_nr_big = pkg.moe_route(logits, K, mode, bias=bias, n_groups=G, topk_groups=TG, renorm=False)
+    assert torch.equal(i_nr, i_nr_big[:9]) and torch.equal(w_nr, w_nr_big[:9])
+    # and the ids are the oracle's, given the scores the device selected on
+    small = pkg.moe_route(logits[:40].contiguous(), K, mode, **kw)
+    scores = small[2].cpu()
+    b = None if bias is None else bias.cpu()
+    if mode == "softmax":
+        # selection looks at the logits (+ bias); a softmax is monotone, so any row-wise top-k of them will do
+        sel = logits[:40].float().cpu() + (0 if b is None else b)
+        order = torch.sort(sel, dim=-1, descending=True, stable=True).indices[:, :K].to(torch.int32)
+        assert torch.equal(small[1].cpu(), order)
+    else:
+        w_ref, i_ref = oracle.select_sigmoid_grouped(scores, b, K, G, TG, 2.5, True)
+        assert torch.equal(small[1].cpu(), i_ref)
+        assert torch.allclose(small[0].cpu(), w_ref, rtol=1e-5, atol=1e-7)
+
+
+def _shared(pkg, oracle, H, I_sh, seed, dev):
+    w13, w13s, w2, w2s = oracle.make_layer(1, H, I_sh, seed=seed)
+    return tuple(t.to(dev) for t in (w13, w13s, w2, w2s))
+
+
+LAYER_CASES = [
+    # T, H, I, E, K, mode, groups, kept, bias, shared I
+    (1, 7168, 256, 256, 8, "sigmoid", 8, 4, True, 256),
+    (8, 1024, 256, 64, 6, "softmax", 1, 1, False, 0),
+    (32, 512, 384, 8, 2, "softmax", 1, 1, False, 0),
+    (19, 1280, 128, 100, 4, "sigmoid", 4, 2, True, 384),
+    (32, 2304, 128, 256, 8, "sigmoid", 8, 4, False, 128),
+    (3, 8192 + 1024, 128, 16, 3, "sigmoid", 1, 1, False, 0),
+]
+
+
+@pytest.mark.parametrize("T,H,I,E,K,mode,G,TG,with_bias,I_sh", LAYER_CASES)
+def test_decode_layer_entry_point(pkg, oracle, dev, T, H, I, E, K, mode, G, TG, with_bias, I_sh):
+    say("decode layer", T, H, I, E, K, mode, G, TG, with_bias, I_sh)
+    small = 3 * E * H * I <= (1 << 26)
+    if small:
+        layer = oracle.make_layer(E, H, I, seed=T + E)
+        ld = tuple(t.to(dev) for t in layer)
+    else:                                   # too large to make on the host: random weights made on the device
+        gd = torch.Generator(device=dev).manual_seed(T + E)
+        w13 = (torch.randn(E, 2 * I, H, generator=gd, device=dev) * 0.02).to(torch.bfloat16)
+        w2 = (torch.randn(E, H, I, generator=gd, device=dev) * 0.02).to(torch.bfloat16)
+        ld = (*pkg.quant_weight_block128(w13), *pkg.quant_weight_block128(w2))
+        del w13, w2
+    g = torch.Generator().manual_seed(7 * T + E)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    wr = (torch.randn(E, H, generator=g) * 0.05).to(torch.bfloat16)
+    bias = (torch.randn(E, generator=g) * 0.05) if with_bias else None
+    xd, wrd = x.to(dev), wr.to(dev)
+    biasd = None if bias is None else bias.to(dev)
+    shared = _shared(pkg, oracle, H, I_sh, 99, dev) if I_sh else None
+    kw = dict(bias=biasd, n_groups=G, topk_groups=TG, renorm=True, scale=2.5 if mode == "sigmoid" else 1.0)
+
+    out, logits, w, ids = pkg.decode_layer_fp8(xd, wrd, *ld, K, mode, shared=shared, return_routing=True, **kw)
+    torch.cuda.synchronize()
+    # logits: bf16 rounding of the exact product
+    exact = x.double() @ wr.double().t()
+    err = (logits.double().cpu() - exact).abs()
+    bound = exact.abs() * 2.0 ** -8 + 1e-4 * x.double().norm(dim=1, keepdim=True) * wr.double().norm(dim=1)[None]
+    assert bool((err <= bound).all()), float((err - bound).max())
+    # routing: the stand-alone routing entry point on the same logits
+    w2_, ids2 = pkg.moe_route(logits, K, mode, **kw)
+    assert torch.equal(ids, ids2) and torch.equal(w, w2_)
+    # experts: the stand-alone expert entry point on the same routing
+    ref_out = pkg.fused_experts_fp8(xd, *ld, ids, w, shared=shared)
+    assert torch.equal(out.view(torch.int16), ref_out.view(torch.int16))
+    # a second call into the same workspace (the arrival counter starts over), without the optional outputs
+    ws = torch.empty(pkg.decode_layer_workspace_bytes(T, H, I, E, K, I_sh), dtype=torch.uint8, device=dev)
+    for _ in range(2):
+        again = pkg.decode_layer_fp8(xd, wrd, *ld, K, mode, shared=shared, workspace=ws, **kw)
+        assert torch.equal(again.view(torch.int16), out.view(torch.int16))
+    # the module takes this road by itself for such a batch
+    moe = pkg.FusedMoE(wrd, *ld, top_k=K, mode=mode, bias=biasd, n_groups=G, topk_groups=TG, renorm=True,
+                       scale=kw["scale"], shared=shared)
+    assert moe._one_call(T)
+    assert torch.equal(moe(xd).view(torch.int16), out.view(torch.int16))
+    # and the whole thing against the oracle, fed with the device's logits
+    lg = logits.float().cpu()
+    if mode == "softmax":
+        w_ref, ids_ref = oracle.route_softmax_topk(lg, K)
+    else:
+        w_ref, ids_ref = oracle.select_sigmoid_grouped(torch.sigmoid(lg), bias, K, G, TG, 2.5, True)
+    if not small:
+        return
+    if torch.equal(ids.cpu(), ids_ref):        # sigmoid on the device may differ in the last place; ids then may too
+        sh = None if shared is None else tuple(t.cpu() for t in shared)
+        ref = oracle.moe_w8a8_fp32(x, ids_ref, w_ref, *layer, shared=sh) if sh else oracle.moe_w8a8_fp32(x, ids_ref, w_ref, *layer)
+        got = out.float().cpu()
+        bad = (got - ref).abs() > 1e-2 + 2e-2 * ref.abs()
+        assert bad.float().mean().item() <= 2e-3
+    else:
+        assert mode == "sigmoid"
+
+
+def test_decode_layer_in_a_hip_graph(pkg, oracle, dev):
+    say("decode layer graph")
+    T, H, I, E, K = 4, 1024, 256, 64, 4
+    ld = tuple(t.to(dev) for t in oracle.make_layer(E, H, I, seed=5))
+    g = torch.Generator().manual_seed(5)
+    wr = (torch.randn(E, H, generator=g) * 0.05).to(torch.bfloat16).to(dev)
+    xs = [torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev) for _ in range(3)]
+    moe = pkg.FusedMoE(wr, *ld, top_k=K, mode="softmax")
+    eager = [moe(x).clone() for x in xs]
+    x_static = xs[0].clone()
+    out_static = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        moe(x_static, out=out_static)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        moe(x_static, out=out_static)
+    for rep in range(2):
+        for x, ref in zip(xs, eager):
+            x_static.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out_static.view(torch.int16), ref.view(torch.int16)), rep
+            assert torch.equal(moe(x).view(torch.int16), ref.view(torch.int16))     # eager work between replays
+
+
+def test_decode_layer_rejects_what_it_does_not_cover(pkg, oracle, dev):
+    say("decode layer errors")
+    H, I = 256, 128
+    g = torch.Generator().manual_seed(1)
+
+    def call(T, E, K):
+        ld = tuple(t.to(dev) for t in oracle.make_layer(E, H, I, seed=1))
+        wr = (torch.randn(E, H, generator=g) * 0.05).to(torch.bfloat16).to(dev)
+        x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+        return pkg.decode_layer_fp8(x, wr, *ld, K, "softmax")
+
+    with pytest.raises(RuntimeError):
+        call(33, 16, 8)             # 264 slots
+    assert not pkg.decode_layer_eligible(33, 16, 8) and pkg.decode_layer_eligible(32, 16, 8)
+    assert not pkg.decode_layer_eligible(1, 257, 8)
+    lib = pkg._lib.lib
+    assert lib.moe_decode_layer_fp8(None, 1, 33, H, 1, None, 16, 8, 0, 1, 1, 1, 1.0, 1, 1, 1, 1, I, None, None, None, None,
+                                    0, 1, None, None, None, 256, 1 << 30) == -2
+    assert lib.moe_decode_layer_fp8(None, 1, 1, H, 1, None, 300, 8, 0, 1, 1, 1, 1.0, 1, 1, 1, 1, I, None, None, None, None,
+                                    0, 1, None, None, None, 256, 1 << 30) == -2
+    out = call(2, 16, 8)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()

@@ -16,6 +16,11 @@ int gemm2_launch(hipStream_t st, const uint8_t *hq, const float *hs, int rows_a,
                  const PermuteWs *pw, int fixed_expert, uint16_t *y, const uint8_t *sh_hq, const float *sh_hs,
                  int sh_rows, const uint8_t *sh_w2, const float *sh_w2s, uint16_t *sh_y, bool bf16 = false);
 
+int decode_prep_launch(hipStream_t st, const uint16_t *x, int T, int H, const uint16_t *wr, const float *bias, int E, int K,
+                       int mode, int n_groups, int topk_groups, int renorm, float scale, uint16_t *logits, float *weights,
+                       int32_t *ids, int *arrivals, uint8_t *xq, float *xs, int tile_m, int32_t *sorted_slot,
+                       int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &pw);
+
 size_t dense_small_partial_bytes(int M, int K, int N, bool keep_partial);
 int dense_small_launch(hipStream_t st, const uint8_t *xq, const float *xs, int M, int K, const uint8_t *w, const float *ws,
                        int N, uint16_t *out, float *partial, int *n_splits_out);
@@ -62,6 +67,62 @@ static FusedWs fused_layout(void *base, int T, int H, int I, int E, int K, int I
   }
   w.bytes = off;
   return w;
+}
+
+// The grouped GEMMs and the weighted sum, once the permutation and the quantised activations are in the workspace.
+static int run_experts(void *stream, const FusedWs &w, const PermuteWs &pw, int T, int H, const uint8_t *w13,
+                       const float *w13_scale, const uint8_t *w2, const float *w2_scale, int I, int E, int K,
+                       const float *routing_weights, const uint8_t *shared_w13, const float *shared_w13_scale,
+                       const uint8_t *shared_w2, const float *shared_w2_scale, int I_sh, void *out_bf16, int out_mode) {
+  hipStream_t st = (hipStream_t)stream;
+  const bool has_shared = shared_w13 != nullptr;
+  // a shared expert of the routed experts' width rides in the routed launches (its tiles fill the
+  // machine together with theirs); any other width gets launches of its own
+  const bool fuse_shared = has_shared && I_sh == I;
+  int rc = gemm1_launch(st, w.xq, w.xs, T, H, w13, w13_scale, I, E, K, w.sorted_slot, w.expert_offsets, &pw, -1, w.hq, w.hs,
+                        fuse_shared ? shared_w13 : nullptr, shared_w13_scale, w.sh_hq, w.sh_hs);
+  if (rc) return rc;
+  uint16_t *y = out_mode == 0 ? (uint16_t *)out_bf16 : w.y;
+  rc = gemm2_launch(st, w.hq, w.hs, T * K, T, H, w2, w2_scale, I, E, K, w.sorted_slot, w.expert_offsets, &pw, -1, y,
+                    w.sh_hq, w.sh_hs, T, fuse_shared ? shared_w2 : nullptr, shared_w2_scale, w.sh_y);
+  if (rc) return rc;
+  if (out_mode == 0) return MOE_OK;
+  if (has_shared && !fuse_shared) {
+    rc = gemm1_launch(st, w.xq, w.xs, T, H, shared_w13, shared_w13_scale, I_sh, 1, 1, nullptr, nullptr, nullptr, 0,
+                      w.sh_hq, w.sh_hs, nullptr, nullptr, nullptr, nullptr);
+    if (rc) return rc;
+    rc = gemm2_launch(st, w.sh_hq, w.sh_hs, T, T, H, shared_w2, shared_w2_scale, I_sh, 1, 1, nullptr, nullptr, nullptr,
+                      0, w.sh_y, nullptr, nullptr, 0, nullptr, nullptr, nullptr);
+    if (rc) return rc;
+  }
+  return moe_weighted_reduce(stream, y, routing_weights, has_shared ? w.sh_y : nullptr, T, K, H, out_bf16);
+}
+
+// moe_decode_layer_fp8: the fused-experts workspace followed by the router's own pieces
+struct DecodeWs {
+  FusedWs fused;
+  uint16_t *logits;
+  float *weights;
+  int32_t *ids;
+  int *arrivals;
+  size_t bytes;
+};
+
+static DecodeWs decode_layout(void *base, int T, int H, int I, int E, int K, int I_sh) {
+  DecodeWs d{};
+  d.fused = fused_layout(base, T, H, I, E, K, I_sh);
+  size_t off = d.fused.bytes;
+  auto take = [&](size_t n) {
+    void *p = base ? (void *)((uint8_t *)base + off) : nullptr;
+    off += align_up(n ? n : 1, 256);
+    return p;
+  };
+  d.logits = (uint16_t *)take((size_t)T * E * 2);
+  d.weights = (float *)take((size_t)T * K * 4);
+  d.ids = (int32_t *)take((size_t)T * K * 4);
+  d.arrivals = (int *)take(4);
+  d.bytes = off;
+  return d;
 }
 
 }  // namespace moe
@@ -120,26 +181,51 @@ extern "C" int moe_fused_experts_fp8(void *stream, const void *x_bf16, int T, in
   if (rc) return rc;
   rc = moe_act_quant(stream, x_bf16, T, H, w.xq, w.xs);
   if (rc) return rc;
-  // a shared expert of the routed experts' width rides in the routed launches (its tiles fill the
-  // machine together with theirs); any other width gets launches of its own
-  const bool fuse_shared = has_shared && I_sh == I;
-  rc = gemm1_launch(st, w.xq, w.xs, T, H, w13, w13_scale, I, E, K, w.sorted_slot, w.expert_offsets, &pw, -1, w.hq, w.hs,
-                    fuse_shared ? shared_w13 : nullptr, shared_w13_scale, w.sh_hq, w.sh_hs);
-  if (rc) return rc;
-  uint16_t *y = out_mode == 0 ? (uint16_t *)out_bf16 : w.y;
-  rc = gemm2_launch(st, w.hq, w.hs, T * K, T, H, w2, w2_scale, I, E, K, w.sorted_slot, w.expert_offsets, &pw, -1, y,
-                    w.sh_hq, w.sh_hs, T, fuse_shared ? shared_w2 : nullptr, shared_w2_scale, w.sh_y);
-  if (rc) return rc;
-  if (out_mode == 0) return MOE_OK;
-  if (has_shared && !fuse_shared) {
-    rc = gemm1_launch(st, w.xq, w.xs, T, H, shared_w13, shared_w13_scale, I_sh, 1, 1, nullptr, nullptr, nullptr, 0,
-                      w.sh_hq, w.sh_hs, nullptr, nullptr, nullptr, nullptr);
-    if (rc) return rc;
-    rc = gemm2_launch(st, w.sh_hq, w.sh_hs, T, T, H, shared_w2, shared_w2_scale, I_sh, 1, 1, nullptr, nullptr, nullptr,
-                      0, w.sh_y, nullptr, nullptr, 0, nullptr, nullptr, nullptr);
-    if (rc) return rc;
+  return run_experts(stream, w, pw, T, H, w13, w13_scale, w2, w2_scale, I, E, K, routing_weights, shared_w13,
+                     shared_w13_scale, shared_w2, shared_w2_scale, I_sh, out_bf16, out_mode);
+}
+
+extern "C" size_t moe_decode_layer_fp8_workspace_bytes(int T, int H, int I, int E, int K, int I_shared) {
+  if (T < 0 || H < 1 || I < 1 || E < 1 || K < 1 || I_shared < 0) return 0;
+  return moe::decode_layout(nullptr, T, H, I, E, K, I_shared).bytes;
+}
+
+extern "C" int moe_decode_layer_fp8(void *stream, const void *x_bf16, int T, int H, const void *router_w_bf16,
+                                    const float *router_bias, int E, int K, int mode, int n_groups, int topk_groups,
+                                    int renorm, float scale, const uint8_t *w13, const float *w13_scale,
+                                    const uint8_t *w2, const float *w2_scale, int I, const uint8_t *shared_w13,
+                                    const float *shared_w13_scale, const uint8_t *shared_w2,
+                                    const float *shared_w2_scale, int I_shared, void *out_bf16, void *logits_out_bf16,
+                                    float *weights_out, int32_t *ids_out, void *workspace, size_t workspace_bytes) {
+  using namespace moe;
+  if (!x_bf16 || !router_w_bf16 || !w13 || !w13_scale || !w2 || !w2_scale || !out_bf16 || !workspace) return MOE_E_NULL;
+  if (T < 0 || H < 1 || I < 1 || E < 1 || E > 256 || K < 1 || K > MOE_MAX_TOPK || K > E) return MOE_E_SHAPE;
+  if ((long)T * K > kChunk) return MOE_E_SHAPE;
+  if (H % kBlock || I % kBlock) return MOE_E_ALIGN;
+  const bool has_shared = shared_w13 != nullptr;
+  if (has_shared) {
+    if (!shared_w13_scale || !shared_w2 || !shared_w2_scale) return MOE_E_NULL;
+    if (I_shared < 1) return MOE_E_SHAPE;
+    if (I_shared % kBlock) return MOE_E_ALIGN;
   }
-  return moe_weighted_reduce(stream, y, routing_weights, has_shared ? w.sh_y : nullptr, T, K, H, out_bf16);
+  const int I_sh = has_shared ? I_shared : 0;
+  if (((uintptr_t)workspace % 256) || ((uintptr_t)x_bf16 % 16) || ((uintptr_t)out_bf16 % 16) ||
+      ((uintptr_t)router_w_bf16 % 16) || ((uintptr_t)w13 % 16) || ((uintptr_t)w2 % 16))
+    return MOE_E_ALIGN;
+  DecodeWs d = decode_layout(workspace, T, H, I, E, K, I_sh);
+  if (workspace_bytes < d.bytes) return MOE_E_WORKSPACE;
+  if (T == 0) return MOE_OK;
+  const FusedWs &w = d.fused;
+  PermuteWs pw = permute_ws_layout(w.permute, T, K, E);
+  float *weights = weights_out ? weights_out : d.weights;
+  int rc = decode_prep_launch((hipStream_t)stream, (const uint16_t *)x_bf16, T, H, (const uint16_t *)router_w_bf16,
+                              router_bias, E, K, mode, n_groups, topk_groups, renorm, scale,
+                              logits_out_bf16 ? (uint16_t *)logits_out_bf16 : d.logits, weights,
+                              ids_out ? ids_out : d.ids, d.arrivals, w.xq, w.xs, choose_tile_m(T, K, E), w.sorted_slot,
+                              w.expert_offsets, w.slot_to_row, pw);
+  if (rc) return rc;
+  return run_experts(stream, w, pw, T, H, w13, w13_scale, w2, w2_scale, I, E, K, weights, shared_w13, shared_w13_scale,
+                     shared_w2, shared_w2_scale, I_sh, out_bf16, 1);
 }
 
 // ---- dense block-scaled FP8 linear layers: the grouped kernels with one "expert" that owns every row ----

@@ -12,6 +12,7 @@
 // A problem of at most kChunk slots is done by one workgroup in a single launch.
 #include "moe_common.h"
 #include "moe_layout.h"
+#include "permute_small.h"
 #include "../../include/moe_hip.h"
 
 namespace moe {
@@ -70,20 +71,6 @@ __device__ __forceinline__ int block_exclusive_scan(int x, int *lds_wave_sums, i
   __syncthreads();
   total = tot;
   return base + inc - x;
-}
-
-// every row tile of expert e gets the expert's whole description: the GEMM workgroups, which only know
-// "some tile of my expert", find their tile, rows and neighbours from one 32-byte record
-__device__ __forceinline__ void write_tiles(int e, int count, int first_row, int first_tile, int tile_m,
-                                            int32_t *tile_expert, int32_t *tile_desc, int max_tiles) {
-  int nt = (count + tile_m - 1) / tile_m;
-  for (int j = 0; j < nt; j++)
-    if (first_tile + j < max_tiles) {
-      tile_expert[first_tile + j] = e;
-      v4i *d = (v4i *)(tile_desc + (size_t)(first_tile + j) * 8);
-      d[0] = (v4i){e, first_tile, nt, first_row};
-      d[1] = (v4i){count, 0, 0, 0};
-    }
 }
 
 __global__ __launch_bounds__(1024) void permute_scan_kernel(int32_t *__restrict__ chunk_counts, int n_chunks, int E,
@@ -161,10 +148,6 @@ __global__ __launch_bounds__(kChunk) void permute_scatter_kernel(const int32_t *
   if (s < TK) slot_to_row[s] = row;
 }
 
-// Whole permutation of at most kChunk slots by one workgroup, one slot per thread: the rank of a
-// slot inside its expert is the number of earlier slots with the same id (every thread walks
-// the id list in LDS in step, so each read is a broadcast), the expert offsets are a block scan of
-// the histogram.
 __global__ __launch_bounds__(kChunk) void permute_small_kernel(const int32_t *__restrict__ ids, int TK, int E, int tile_m,
                                                               int max_tiles, int32_t *__restrict__ sorted_slot,
                                                               int32_t *__restrict__ expert_offsets,
@@ -172,55 +155,10 @@ __global__ __launch_bounds__(kChunk) void permute_small_kernel(const int32_t *__
                                                               int32_t *__restrict__ tile_prefix,
                                                               int32_t *__restrict__ tile_expert,
                                                               int32_t *__restrict__ tile_desc) {
-  __shared__ int hist[MOE_MAX_EXPERTS];
-  __shared__ int offs[MOE_MAX_EXPERTS];
-  __shared__ int sid[kChunk];
-  __shared__ int wave_sums[2][kChunk / 64];
+  __shared__ PermuteSmallSmem sm;
   const int s = threadIdx.x;
-  for (int e = s; e < E; e += kChunk) hist[e] = 0;
-  int v = (s < TK) ? ids[s] : -1;
-  const bool valid = v >= 0 && v < E;
-  sid[s] = valid ? v : -1;
-  __syncthreads();
-  if (valid) atomicAdd(&hist[v], 1);
-  int rank = 0;
-  for (int j = 0; j < s; j++) rank += (sid[j] == v);
-  __syncthreads();
-  // exclusive scans of the counts and of the tile counts over the experts, kChunk experts per pass
-  int carry = 0, tcarry = 0;
-  for (int e0 = 0; e0 < E; e0 += kChunk) {
-    const int e = e0 + s;
-    const int c = e < E ? hist[e] : 0;
-    const int t = (c + tile_m - 1) / tile_m;
-    int inc = c, tinc = t;
-    const int lane = s & 63, wave = s >> 6;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-      const int y = __shfl_up(inc, off, 64), ty = __shfl_up(tinc, off, 64);
-      if (lane >= off) { inc += y; tinc += ty; }
-    }
-    if (lane == 63) { wave_sums[0][wave] = inc; wave_sums[1][wave] = tinc; }
-    __syncthreads();
-    int base = carry, tbase = tcarry, tot = 0, ttot = 0;
-    for (int w = 0; w < kChunk / 64; w++) {
-      if (w < wave) { base += wave_sums[0][w]; tbase += wave_sums[1][w]; }
-      tot += wave_sums[0][w]; ttot += wave_sums[1][w];
-    }
-    if (e < E) {
-      offs[e] = base + inc - c;
-      expert_offsets[e] = base + inc - c;
-      tile_prefix[e] = tbase + tinc - t;
-      write_tiles(e, c, base + inc - c, tbase + tinc - t, tile_m, tile_expert, tile_desc, max_tiles);
-    }
-    carry += tot; tcarry += ttot;
-    __syncthreads();
-  }
-  if (s == 0) { expert_offsets[E] = carry; tile_prefix[E] = tcarry; }
-  if (s < TK) {
-    const int row = valid ? offs[v] + rank : -1;
-    if (valid && row < TK) sorted_slot[row] = s;
-    slot_to_row[s] = row;
-  }
+  permute_small_block(sm, (s < TK) ? ids[s] : -1, TK, E, tile_m, max_tiles, sorted_slot, expert_offsets, slot_to_row,
+                      tile_prefix, tile_expert, tile_desc);
 }
 
 int permute_launch(hipStream_t st, const int32_t *ids, int T, int K, int E, int tile_m, int32_t *sorted_slot,

@@ -4,38 +4,15 @@
 // Both move 16 bytes per lane per access; rows are contiguous so every access is coalesced.
 #include "moe_common.h"
 #include "moe_layout.h"
+#include "act_quant.h"
 #include "../../include/moe_hip.h"
 
 namespace moe {
 
-// 16 lanes share one 128-column group: 8 bf16 per lane.
 __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t *__restrict__ x, size_t n_groups,
                                                         int groups_per_row, int pitch, uint8_t *__restrict__ q,
                                                         float *__restrict__ s) {
-  const size_t g = ((size_t)blockIdx.x * 256 + threadIdx.x) >> 4;
-  const int sub = threadIdx.x & 15;
-  const bool live = g < n_groups;
-  float f[8];
-  float amax = 0.f;
-  if (live) {
-    v4i raw = *(const v4i *)(x + g * kBlock + sub * 8);
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      uint32_t w = (uint32_t)raw[i];
-      f[2 * i] = bf16_to_f32((uint16_t)(w & 0xffff));
-      f[2 * i + 1] = bf16_to_f32((uint16_t)(w >> 16));
-    }
-#pragma unroll
-    for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(f[i]));
-  }
-  amax = max_over_row16(amax);
-  if (!live) return;
-  const float sc = group_scale(amax);
-  v2i out;
-  out[0] = (int)pack4_fp8(f[0] / sc, f[1] / sc, f[2] / sc, f[3] / sc);
-  out[1] = (int)pack4_fp8(f[4] / sc, f[5] / sc, f[6] / sc, f[7] / sc);
-  *(v2i *)(q + g * kBlock + sub * 8) = out;
-  if (sub == 0) s[(g / groups_per_row) * pitch + g % groups_per_row] = sc;
+  act_quant_thread(x, n_groups, groups_per_row, pitch, q, s, (size_t)blockIdx.x * 256 + threadIdx.x);
 }
 
 // One lane produces 8 consecutive columns of one token.

@@ -5,6 +5,7 @@
 // "greater value, then lower index" as the order, so equal scores resolve to the lower index
 // on every lane identically and the K picks come out in descending order.
 #include "moe_common.h"
+#include "route_block.h"
 #include "../../include/moe_hip.h"
 
 namespace moe {
@@ -260,7 +261,23 @@ static int launch_noaux(hipStream_t st, const void *scores, int dtype, int T, in
   return (int)hipGetLastError();
 }
 
-static int check_route_shape(int T, int E, int K, int n_groups, int topk_groups) {
+// One workgroup per token: the short-chain form for batches of a few tokens (route_block.h).
+__global__ __launch_bounds__(kRouteBlock) void route_block_kernel(const void *__restrict__ logits, int logits_bf16,
+                                                                  const float *__restrict__ bias, int E, int K, int mode,
+                                                                  int n_groups, int topk_groups, int renorm, float scale,
+                                                                  float *__restrict__ weights_out,
+                                                                  int32_t *__restrict__ ids_out,
+                                                                  float *__restrict__ scores_out) {
+  __shared__ __attribute__((aligned(16))) RouteBlockSmem sm;
+  const size_t t = blockIdx.x;
+  const void *row = logits_bf16 ? (const void *)((const uint16_t *)logits + t * E) : (const void *)((const float *)logits + t * E);
+  route_block(sm, row, logits_bf16, bias, E, K, mode, n_groups, topk_groups, renorm, scale, weights_out + t * K,
+              ids_out + t * K, scores_out ? scores_out + t * E : nullptr);
+}
+
+constexpr int kRouteBlockMaxTokens = 64;   // up to here a launch is latency-bound and the workgroup-per-token form wins
+
+int check_route_shape(int T, int E, int K, int n_groups, int topk_groups) {
   if (T < 0 || E < 1 || E > MOE_MAX_EXPERTS || K < 1 || K > E || K > MOE_MAX_TOPK) return MOE_E_SHAPE;
   if (n_groups > 1) {
     if (n_groups > 64 || E % n_groups != 0 || topk_groups < 1 || topk_groups > n_groups) return MOE_E_SHAPE;
@@ -301,6 +318,11 @@ extern "C" int moe_route_topk(void *stream, const void *logits, int logits_dtype
   hipStream_t st = (hipStream_t)stream;
   dim3 grid((T + 3) / 4), block(256);
   const int bf = logits_dtype == MOE_DTYPE_BF16;
+  if (T <= kRouteBlockMaxTokens && E <= kRouteBlock) {
+    route_block_kernel<<<T, kRouteBlock, 0, st>>>(logits, bf, bias, E, K, mode, n_groups, topk_groups, renorm, scale,
+                                                  weights_out, ids_out, scores_out);
+    return (int)hipGetLastError();
+  }
 #define MOE_LAUNCH_ROUTE(P)                                                                                          \
   route_topk_kernel<P><<<grid, block, 0, st>>>(logits, bf, bias, T, E, K, mode, n_groups, topk_groups, renorm, scale, \
                                                weights_out, ids_out, scores_out)

@@ -205,6 +205,72 @@ def fused_experts_fp8(x, w13, w13_scale, w2, w2_scale, ids, routing_weights=None
     return out
 
 
+def decode_layer_eligible(T: int, E: int, K: int) -> bool:
+    """Shapes the one-call decode entry point takes (decode_layer_fp8)."""
+    return 1 <= T and T * K <= 256 and E <= 256
+
+
+def decode_layer_workspace_bytes(T, H, I, E, K, I_shared=0) -> int:
+    return lib.moe_decode_layer_fp8_workspace_bytes(T, H, I, E, K, I_shared)
+
+
+def decode_layer_fp8(x, router_weight, w13, w13_scale, w2, w2_scale, top_k: int, mode: str = "softmax", bias=None,
+                     n_groups: int = 1, topk_groups: int = 1, renorm: bool = True, scale: float = 1.0, shared=None,
+                     out=None, workspace=None, return_routing: bool = False):
+    """Router and experts of one layer in one call, for decode-size batches (T*top_k <= 256, E <= 256).
+
+    x [T,H] bf16, router_weight [E,H] bf16, the expert weights as in fused_experts_fp8.  Returns out [T,H] bf16,
+    or (out, logits bf16 [T,E], weights fp32 [T,k], ids int32 [T,k]) with return_routing."""
+    modes = {"softmax": ROUTE_SOFTMAX, "sigmoid": ROUTE_SIGMOID}
+    _need(mode in modes, f"unknown routing mode {mode!r}")
+    _need(x.dim() == 2 and w13.dim() == 3 and w2.dim() == 3 and router_weight.dim() == 2, "bad ranks")
+    T, H = x.shape
+    E, I2, H2 = w13.shape
+    I = I2 // 2
+    _need(decode_layer_eligible(T, E, top_k), "decode_layer_fp8 takes T*top_k <= 256 and E <= 256")
+    _need(H2 == H and tuple(w2.shape) == (E, H, I) and tuple(router_weight.shape) == (E, H), "weight shapes do not match x")
+    _need(H % 128 == 0 and I % 128 == 0, "H and I must be multiples of 128")
+    _need(tuple(w13_scale.shape) == (E, I2 // 128, H // 128), "w13_scale must be [E, 2I/128, H/128]")
+    _need(tuple(w2_scale.shape) == (E, H // 128, I // 128), "w2_scale must be [E, H/128, I/128]")
+    if out is None:
+        out = torch.empty(T, H, dtype=torch.bfloat16, device=x.device)
+    _need(tuple(out.shape) == (T, H), "out must be [T, H]")
+    bias_ptr = None
+    if bias is not None:
+        _need(bias.numel() == E, "bias must hold one value per expert")
+        bias_ptr = _dev(bias, "bias", torch.float32)
+    sh = [None, None, None, None]
+    I_sh = 0
+    if shared is not None:
+        s13, s13s, s2, s2s = shared
+        I_sh = s13.shape[1] // 2
+        _need(tuple(s13.shape) == (1, 2 * I_sh, H) and tuple(s2.shape) == (1, H, I_sh), "bad shared expert shapes")
+        _need(tuple(s13s.shape) == (1, 2 * I_sh // 128, H // 128) and tuple(s2s.shape) == (1, H // 128, I_sh // 128),
+              "bad shared expert scale shapes")
+        sh = [_dev(s13, "shared w13", _FP8), _dev(s13s, "shared w13 scale", torch.float32),
+              _dev(s2, "shared w2", _FP8), _dev(s2s, "shared w2 scale", torch.float32)]
+    need = decode_layer_workspace_bytes(T, H, I, E, top_k, I_sh)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+    _need(workspace.numel() * workspace.element_size() >= need, "workspace too small")
+    logits = weights = ids = None
+    if return_routing:
+        logits = torch.empty(T, E, dtype=torch.bfloat16, device=x.device)
+        weights = torch.empty(T, top_k, dtype=torch.float32, device=x.device)
+        ids = torch.empty(T, top_k, dtype=torch.int32, device=x.device)
+    rc = lib.moe_decode_layer_fp8(
+        _stream(), _dev(x, "x", torch.bfloat16), T, H, _dev(router_weight, "router_weight", torch.bfloat16), bias_ptr,
+        E, top_k, modes[mode], n_groups, topk_groups, int(renorm), float(scale),
+        _dev(w13, "w13", _FP8), _dev(w13_scale, "w13_scale", torch.float32),
+        _dev(w2, "w2", _FP8), _dev(w2_scale, "w2_scale", torch.float32), I,
+        sh[0], sh[1], sh[2], sh[3], I_sh, _dev(out, "out", torch.bfloat16),
+        logits.data_ptr() if return_routing else None, weights.data_ptr() if return_routing else None,
+        ids.data_ptr() if return_routing else None,
+        _dev(workspace, "workspace"), workspace.numel() * workspace.element_size())
+    check(rc, "decode_layer_fp8")
+    return (out, logits, weights, ids) if return_routing else out
+
+
 def fused_experts_bf16(x, w13, w2, ids, routing_weights=None, out=None, workspace=None):
     """The expert computation on un-quantised weights: x [T,H] bf16, w13 [E,2I,H] bf16 (gate rows, then
     up rows), w2 [E,H,I] bf16, ids [T,K] int32.  out [T,K,H]: per-slot results; out [T,H]: weighted sum."""
