@@ -107,14 +107,19 @@ __global__ __launch_bounds__(kRouteBlock) void route_permute_small_kernel(
   const int t = blockIdx.x;
   route_block(rs, logits + (size_t)t * E, 1, bias, E, K, mode, n_groups, topk_groups, renorm, scale,
               weights + (size_t)t * K, ids + (size_t)t * K, nullptr);
-  __threadfence();                      // this token's picks are visible device-wide before the arrival is counted
-  __syncthreads();
-  if (threadIdx.x == 0) is_last = atomicAdd(arrivals, 1) == (int)gridDim.x - 1;
-  __syncthreads();
-  if (!is_last) return;
-  __threadfence();
   const int s = threadIdx.x, TK = T * K;
-  const int v = s < TK ? __hip_atomic_load(ids + s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : -1;
+  int v;
+  if (gridDim.x == 1) {
+    v = s < TK ? rs.isel[s] : -1;       // one token: its picks are still in LDS
+  } else {
+    __threadfence();                    // this token's picks are visible device-wide before the arrival is counted
+    __syncthreads();
+    if (threadIdx.x == 0) is_last = atomicAdd(arrivals, 1) == (int)gridDim.x - 1;
+    __syncthreads();
+    if (!is_last) return;
+    __threadfence();
+    v = s < TK ? __hip_atomic_load(ids + s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : -1;
+  }
   permute_small_block(ps, v, TK, E, tile_m, max_tiles, sorted_slot, expert_offsets, slot_to_row, tile_prefix, tile_expert,
                       tile_desc);
 }

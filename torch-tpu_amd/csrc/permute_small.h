@@ -21,10 +21,10 @@ __device__ __forceinline__ void write_tiles(int e, int count, int first_row, int
     }
 }
 
-struct PermuteSmallSmem {
+struct __attribute__((aligned(16))) PermuteSmallSmem {
+  int sid[kChunk];
   int hist[MOE_MAX_EXPERTS];
   int offs[MOE_MAX_EXPERTS];
-  int sid[kChunk];
   int wave_sums[2][kChunk / 64];
 };
 
@@ -32,6 +32,7 @@ struct PermuteSmallSmem {
 // (`v` = the thread's expert id, anything outside [0, E) for "no slot"): the rank of a slot inside its
 // expert is the number of earlier slots with the same id (every thread walks the id list in LDS in
 // step, so each read is a broadcast), the expert offsets are a block scan of the histogram.
+// `sm` must sit on a 16-byte boundary.
 __device__ __forceinline__ void permute_small_block(PermuteSmallSmem &sm, int v, int TK, int E, int tile_m, int max_tiles,
                                                     int32_t *__restrict__ sorted_slot,
                                                     int32_t *__restrict__ expert_offsets,
@@ -43,11 +44,20 @@ __device__ __forceinline__ void permute_small_block(PermuteSmallSmem &sm, int v,
   for (int e = s; e < E; e += kChunk) sm.hist[e] = 0;
   const bool valid = s < TK && v >= 0 && v < E;
   if (!valid) v = -1;
-  sm.sid[s] = v;
+  // (expert, slot) as one integer: the slots of expert v that precede slot s are the entries in [v * kChunk, own)
+  const uint32_t own = valid ? (uint32_t)v * kChunk + s : 0x7fffffffu, lo = (uint32_t)v * kChunk;
+  sm.sid[s] = (int)own;
   __syncthreads();
   if (valid) atomicAdd(&sm.hist[v], 1);
+  // every thread walks the same (TK + 3) / 4 vectors, so the trip count is uniform and the reads pipeline
   int rank = 0;
-  for (int j = 0; j < s; j++) rank += (sm.sid[j] == v);
+  const v4i *sid4 = (const v4i *)sm.sid;
+#pragma unroll 8
+  for (int j4 = 0; j4 < (TK + 3) / 4; j4++) {
+    const v4i q = sid4[j4];
+    rank += ((uint32_t)q[0] - lo < own - lo) + ((uint32_t)q[1] - lo < own - lo) + ((uint32_t)q[2] - lo < own - lo) +
+            ((uint32_t)q[3] - lo < own - lo);
+  }
   __syncthreads();
   // exclusive scans of the counts and of the tile counts over the experts, kChunk experts per pass
   int carry = 0, tcarry = 0;

@@ -4,7 +4,9 @@
 // Thread e owns expert e.  Instead of K arg-max rounds in sequence, every thread counts the
 // experts that come before its own in "greater score, then lower index" order: that count is the
 // expert's position in the sorted row, so the K picks are the threads whose count is below K, and
-// they come out in descending order.  The group limit works the same way: position inside the
+// they come out in descending order.  The order is one unsigned 64-bit compare per pair: the
+// score mapped to an unsigned integer of the same order in the high half, "lower index first" in
+// the low half (compare masks combined on the scalar side cost several times as much).  The group limit works the same way: position inside the
 // group (0 and 1 make the group's score), then position of the group among the groups.  All reads
 // of the score table are LDS broadcasts.  Orders, sums and divisions are those of the
 // one-wavefront-per-token kernel, so both give the same ids and the same weights, bit for bit.
@@ -17,18 +19,21 @@ namespace moe {
 constexpr int kRouteBlock = 256;
 
 struct RouteBlockSmem {
-  float sel[kRouteBlock];      // selection score of every expert (-inf beyond E and in dropped groups)
+  uint64_t key[kRouteBlock];   // order key of every expert's selection score (0 beyond E: after everything)
   float raw[kRouteBlock];      // softmax numerators
   float gtop[64][2];           // best two selection scores of every group
-  float gscore[64];
+  uint64_t gkey[64];           // order key of every group's score
   float wmax[kRouteBlock / 64];
   float wsel[64];              // weight source of pick k
   int isel[64];                // expert of pick k
 };
 
-// a (score, index) comes before b
-__device__ __forceinline__ int comes_before(float av, int ai, float bv, int bi) {
-  return (av > bv) | ((av == bv) & (ai < bi));
+// (score a, index ai) comes before (b, bi) - greater score, then lower index - exactly when
+// order_key(a, ai) > order_key(b, bi).  Adding +0 first makes -0 and +0 the same key, as they compare equal.
+__device__ __forceinline__ uint64_t order_key(float v, int idx) {
+  uint32_t u = __float_as_uint(v + 0.0f);
+  u = (u >> 31) ? ~u : (u | 0x80000000u);
+  return ((uint64_t)u << 32) | (uint32_t)(0x7fffffff - idx);
 }
 
 __device__ __forceinline__ void route_block(RouteBlockSmem &sm, const void *logits_row, int logits_bf16,
@@ -64,37 +69,39 @@ __device__ __forceinline__ void route_block(RouteBlockSmem &sm, const void *logi
     denom_all = part;
     if (scores_row != nullptr && live) scores_row[e] = raw / denom_all;
   }
-  sm.sel[e] = v;
+  uint64_t key = live ? order_key(v, e) : 0;
+  sm.key[e] = key;
   __syncthreads();
 
   if (n_groups > 1) {
     const int per = E / n_groups, g = live ? e / per : 0;
     if (live) {
       int r = 0;
-      for (int j = g * per; j < g * per + per; j++) r += comes_before(sm.sel[j], j, v, e);
+#pragma unroll 8
+      for (int j = g * per; j < g * per + per; j++) r += sm.key[j] > key;
       if (r < 2) sm.gtop[g][r] = v;
     }
     __syncthreads();
-    if (e < n_groups) sm.gscore[e] = sm.gtop[e][0] + sm.gtop[e][1];
+    if (e < n_groups) sm.gkey[e] = order_key(sm.gtop[e][0] + sm.gtop[e][1], e);
     __syncthreads();
     if (live) {
-      const float gs = sm.gscore[g];
+      const uint64_t gk = sm.gkey[g];
       int r = 0;
-      for (int h = 0; h < n_groups; h++) r += comes_before(sm.gscore[h], h, gs, g);
-      if (r >= topk_groups) v = -INFINITY;     // dropped groups stay candidates with -inf, as a masked_fill would leave them
+#pragma unroll 8
+      for (int h = 0; h < n_groups; h++) r += sm.gkey[h] > gk;
+      if (r >= topk_groups) {     // dropped groups stay candidates with -inf, as a masked_fill would leave them
+        v = -INFINITY;
+        key = order_key(v, e);
+      }
     }
-    sm.sel[e] = v;          // every read of the unmasked table happened before the barrier above
+    sm.key[e] = key;        // every read of the unmasked table happened before the barrier above
     __syncthreads();
   }
 
   if (live) {
     int r = 0;
-    const v4f *tab = (const v4f *)sm.sel;
-    for (int j4 = 0; j4 < (E + 3) / 4; j4++) {            // entries beyond E hold -inf at a higher index: they never come first
-      const v4f s = tab[j4];
-      r += comes_before(s[0], 4 * j4, v, e) + comes_before(s[1], 4 * j4 + 1, v, e) +
-           comes_before(s[2], 4 * j4 + 2, v, e) + comes_before(s[3], 4 * j4 + 3, v, e);
-    }
+#pragma unroll 16
+    for (int j = 0; j < kRouteBlock; j++) r += sm.key[j] > key;     // the whole table, so that the reads pipeline
     if (r < K) { sm.isel[r] = e; sm.wsel[r] = raw; }
   }
   __syncthreads();
