@@ -230,15 +230,6 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   if (rows <= 0) return;
   const int mt_live = (rows + 15) >> 4;               // m-tiles that hold at least one row
 
-  for (int i = tid; i < BM; i += NT) {
-    const int p = row0 + min(i, rows - 1);
-    int src = p;
-    if (GATED && !direct) src = a.sorted_slot[p] / a.topk;
-    sm.arow[i] = min(max(src, 0), rows_a - 1);
-    if (!GATED) sm.oslot[i] = direct ? p : a.sorted_slot[p];      // output row (slot) of each tile row
-  }
-  __syncthreads();
-
   const int NKB = a.Kd >> 7;
   const int n_wblk = (a.n_rows_w + 127) >> 7;         // weight-scale rows per expert
 
@@ -260,16 +251,35 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   const uint32_t wdma_off = (uint32_t)(lane >> 3) * (uint32_t)a.Kd + (((lane & 7) ^ (lane >> 3)) << 4);
   // The strip's weight-block scales for all steps go to LDS once (two rows: gate/up blocks for
   // the gated GEMM, the strip's two 128-column blocks otherwise): uniform values re-read per
-  // step from LDS instead of through the vector-memory queue.
+  // step from LDS instead of through the vector-memory queue.  They are asked for together with
+  // the rows' sources, before either is waited for.
+  constexpr int NSB = (2 * kMaxKB + NT - 1) / NT;
+  float sbv[NSB];
   if constexpr (!BF16) {
     const int blk0 = GATED ? strip : min(strip * 2, n_wblk - 1);
     const int blk1 = GATED ? (a.N >> 7) + strip : min(strip * 2 + 1, n_wblk - 1);
-    for (int i = tid; i < 2 * NKB; i += NT) {
-      const int r = i >= NKB, kb = i - r * NKB;
-      sm.sb[r][kb] = ws[((size_t)e * n_wblk + (r ? blk1 : blk0)) * NKB + kb];
+#pragma unroll
+    for (int u = 0; u < NSB; u++) {
+      const int i = tid + u * NT, r = i >= NKB, kb = i - r * NKB;
+      sbv[u] = i < 2 * NKB ? ws[((size_t)e * n_wblk + (r ? blk1 : blk0)) * NKB + kb] : 0.f;
+    }
+  }
+  for (int i = tid; i < BM; i += NT) {
+    const int p = row0 + min(i, rows - 1);
+    int src = p;
+    if (GATED && !direct) src = a.sorted_slot[p] / a.topk;
+    sm.arow[i] = min(max(src, 0), rows_a - 1);
+    if (!GATED) sm.oslot[i] = direct ? p : a.sorted_slot[p];      // output row (slot) of each tile row
+  }
+  if constexpr (!BF16) {
+#pragma unroll
+    for (int u = 0; u < NSB; u++) {
+      const int i = tid + u * NT, r = i >= NKB, kb = i - r * NKB;
+      if (i < 2 * NKB) sm.sb[r][kb] = sbv[u];
     }
     if (tid < 8) sm.sb[tid >> 2][NKB + (tid & 3)] = 0.f;
   }
+  __syncthreads();
   const int sb_row0 = GATED ? 0 : (wave * WT) / 8;      // which of the two rows this wavefront's tiles use
   const int sb_row1 = GATED ? 1 : sb_row0;
   // Token tile -> LDS by direct loads: one instruction moves 64 x 16 bytes = 8 rows x 128 bytes to
@@ -348,13 +358,14 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(sac_src[u]), "s"(base) : "memory", "m0");
     }
   };
+  auto request_tok = [&](int kb, int stage, int u) {
+    const uint8_t *base = aq + (size_t)kb * 128;
+    const uint32_t m0 = tok_base + stage * kTokStage + tok_m0[u];
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(tok_src[u]), "s"(base) : "memory", "m0");
+  };
   auto request = [&](int kb, int stage) {
 #pragma unroll
-    for (int u = 0; u < NTOK; u++) {
-      const uint8_t *base = aq + (size_t)kb * 128;
-      const uint32_t m0 = tok_base + stage * kTokStage + tok_m0[u];
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(tok_src[u]), "s"(base) : "memory", "m0");
-    }
+    for (int u = 0; u < NTOK; u++) request_tok(kb, stage, u);
     // weight tiles through LDS: like the token tile, an instruction moves 8 whole rows x 128 bytes
     // (every cache line it touches is used completely) into swizzled [row][16-byte chunk] order
     if (!WREG)
@@ -491,7 +502,6 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
       arrived_weights(wlo[0], whi[0]);
       __syncthreads();
       if (n_chunks > 1) request_scales(1);
-      request(min(3, last), 3);
       // Scale products: what a lane multiplies a matrix-instruction result with is (activation scale
       // of its token and step) x (weight-block scale of its tile and step).  One thread per tile row
       // forms both products of a step once, two steps ahead, instead of every wavefront forming them
@@ -550,6 +560,14 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
               x[(g + PD) % XB] = read_x(kk, LIVE - 1 - qq);
               fb[(g + PD) % XB] = read_f(kk, LIVE - 1 - qq);
             }
+            // the token tile of step kb + 3 goes into the stage that step kb - 1 used, one piece with each of a few
+            // m-tiles: all wavefronts asking for everything at the step boundary queued up behind one another
+#pragma unroll
+            for (int u = 0; u < NTOK; u++)
+              if (u * LIVE / NTOK == q) request_tok(min(kb + 3, last), (kb + 3) & 3, u);
+            // the scale products of step kb + 3 take the slot step kb - 1 read from: formed in the middle of a step, where
+            // the matrix pipe has work, instead of at the boundary, where every wavefront stands still
+            if (q == LIVE / 2) produce_f(kb + 3);
             if constexpr (BF16) {                        // accumulates in place: nothing is pending afterwards
               mma_bf16<WT>(acc[LIVE - 1 - q], wc, x[g % XB]);
               __builtin_amdgcn_sched_barrier(0);
@@ -580,9 +598,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
           asm volatile("s_waitcnt vmcnt(%0)" ::"n"(L_WAIT) : "memory");
           arrived_weights(wlo[(h + 1) % R], whi[(h + 1) % R]);
           __syncthreads();
-          produce_f(kb + 3);
           if (((kb + 1) & 15) == 0 && ((kb + 1) >> 4) + 1 < n_chunks) request_scales(((kb + 1) >> 4) + 1);
-          request(min(kb + 4, last), kb & 3);
           __builtin_amdgcn_sched_barrier(0);
         }
       }
@@ -623,11 +639,11 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
 #pragma unroll
         for (int r = 0; r < 4; r++) {
           const float g = acc[mt][j][r], u = acc[mt][j + G][r];
-          v[r] = (g / (1.0f + expf(-g))) * u;
+          v[r] = silu_fast(g) * u;
         }
         v2i o;
-        o[0] = (int)((uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16));
-        o[1] = (int)((uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16));
+        o[0] = (int)pack2_bf16(v[0], v[1]);
+        o[1] = (int)pack2_bf16(v[2], v[3]);
         *(v2i *)(h + (size_t)(row0 + i) * a.N + strip * 128 + wave * (16 * G) + j * 16 + lg * 4) = o;
       }
     }
@@ -635,35 +651,40 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     constexpr int G = WT / 2;                          // gate tiles per wavefront
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
-      float m = 0.f;
+      if (mt < mt_live) {                              // m-tiles without a row have nothing to write
+        float m = 0.f;
 #pragma unroll
-      for (int j = 0; j < G; j++)
+        for (int j = 0; j < G; j++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-          const float g = acc[mt][j][r], u = acc[mt][j + G][r];
-          const float h = (g / (1.0f + expf(-g))) * u;
-          acc[mt][j][r] = h;
-          m = fmaxf(m, fabsf(h));
-        }
-      m = max_over_lane_groups(m);
-      if (lg == 0) sm.amax[wave][mt * 16 + li] = m;
+          for (int r = 0; r < 4; r++) {
+            const float g = acc[mt][j][r], u = acc[mt][j + G][r];
+            const float h = silu_fast(g) * u;
+            acc[mt][j][r] = h;
+            m = fmaxf(m, fabsf(h));
+          }
+        m = max_over_lane_groups(m);
+        if (lg == 0) sm.amax[wave][mt * 16 + li] = m;
+      }
     }
     __syncthreads();
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
       const int i = mt * 16 + li;
       const bool valid = i < rows;
-      float am = 0.f;
+      if (mt < mt_live) {
+        float am = 0.f;
 #pragma unroll
-      for (int w = 0; w < NW; w++) am = fmaxf(am, sm.amax[w][i]);
-      const float sc = group_scale(am);
-      const size_t orow = (size_t)(row0 + i);
+        for (int w = 0; w < NW; w++) am = fmaxf(am, sm.amax[w][i]);
+        const float sc = group_scale(am);
+        const float inv = 1.0f / sc;                   // one division per row; the elements are multiplied
+        const size_t orow = (size_t)(row0 + i);
 #pragma unroll
-      for (int j = 0; j < G; j++) {
-        const uint32_t packed = pack4_fp8(acc[mt][j][0] / sc, acc[mt][j][1] / sc, acc[mt][j][2] / sc, acc[mt][j][3] / sc);
-        if (valid) *(uint32_t *)((shared ? a.sh_hq : a.hq) + orow * a.N + strip * 128 + wave * (16 * G) + j * 16 + lg * 4) = packed;
+        for (int j = 0; j < G; j++) {
+          const uint32_t packed = pack4_fp8(acc[mt][j][0] * inv, acc[mt][j][1] * inv, acc[mt][j][2] * inv, acc[mt][j][3] * inv);
+          if (valid) *(uint32_t *)((shared ? a.sh_hq : a.hq) + orow * a.N + strip * 128 + wave * (16 * G) + j * 16 + lg * 4) = packed;
+        }
+        if (valid && wave == 0 && lg == 0) (shared ? a.sh_hs : a.hs)[orow * a.hs_pitch + strip] = sc;
       }
-      if (valid && wave == 0 && lg == 0) (shared ? a.sh_hs : a.hs)[orow * a.hs_pitch + strip] = sc;
     }
   } else {
 #pragma unroll
@@ -671,13 +692,14 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
       const int i = mt * 16 + li;
       const bool valid = i < rows;
       const int slot = sm.oslot[i];
+      if (mt < mt_live)
 #pragma unroll
       for (int j = 0; j < WT; j++) {
         const int col = strip * 256 + wave * (16 * WT) + j * 16 + lg * 4;
         if (valid && col < a.N) {
           v2i o;
-          o[0] = (int)((uint32_t)f32_to_bf16(acc[mt][j][0]) | ((uint32_t)f32_to_bf16(acc[mt][j][1]) << 16));
-          o[1] = (int)((uint32_t)f32_to_bf16(acc[mt][j][2]) | ((uint32_t)f32_to_bf16(acc[mt][j][3]) << 16));
+          o[0] = (int)pack2_bf16(acc[mt][j][0], acc[mt][j][1]);
+          o[1] = (int)pack2_bf16(acc[mt][j][2], acc[mt][j][3]);
           *(v2i *)((shared ? a.sh_y : a.y) + (size_t)slot * a.N + col) = o;
         }
       }

@@ -39,6 +39,16 @@ __device__ __forceinline__ float group_scale(float amax) { return fmaxf(amax, kA
 
 __device__ __forceinline__ float silu_f32(float g) { return g / (1.0f + __expf(-g)); }
 
+// silu on the hardware's exp2 and reciprocal (a few ulp; two instructions instead of a division sequence)
+__device__ __forceinline__ float silu_fast(float g) { return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)); }
+
+// two fp32 -> two bf16 (round to nearest even) in one instruction, first value in the low half
+typedef float v2f_t __attribute__((ext_vector_type(2)));
+typedef __bf16 v2bf_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector((v2f_t){lo, hi}, v2bf_t));
+}
+
 // max over the lanes that share (lane % 16): butterflies over lane bits 4 and 5
 __device__ __forceinline__ float max_over_lane_groups(float v) {
   v = fmaxf(v, __shfl_xor(v, 16, 64));
