@@ -279,7 +279,7 @@ extern "C" int moe_mm_fp8(void *stream, const void *x_bf16, int M, int K, const 
   if (M < 0 || K < 1 || N < 16 || K > 32768 || N > (1 << 20)) return MOE_E_SHAPE;
   if (K % kBlock || N % 16) return MOE_E_ALIGN;
   if ((double)M * K >= 2147483648.0 || (double)M * N >= 2147483648.0 || (double)N * K >= 4294967296.0) return MOE_E_SHAPE;
-  if (((uintptr_t)workspace % 256) || ((uintptr_t)x_bf16 % 16) || ((uintptr_t)out_bf16 % 8) || ((uintptr_t)w % 16))
+  if (((uintptr_t)workspace % 256) || ((uintptr_t)x_bf16 % 16) || ((uintptr_t)out_bf16 % 16) || ((uintptr_t)w % 16))
     return MOE_E_ALIGN;
   DenseWs d = dense_layout(workspace, M, K, 0, N);
   if (workspace_bytes < d.bytes) return MOE_E_WORKSPACE;
@@ -305,7 +305,7 @@ extern "C" int moe_mlp_fp8(void *stream, const void *x_bf16, int M, int H, const
   if (M < 0 || H < 1 || I < 1 || H > 32768 || I > 32768) return MOE_E_SHAPE;
   if (H % kBlock || I % kBlock) return MOE_E_ALIGN;
   if ((double)M * H >= 2147483648.0 || (double)M * I >= 2147483648.0) return MOE_E_SHAPE;
-  if (((uintptr_t)workspace % 256) || ((uintptr_t)x_bf16 % 16) || ((uintptr_t)out_bf16 % 8) || ((uintptr_t)w13 % 16) ||
+  if (((uintptr_t)workspace % 256) || ((uintptr_t)x_bf16 % 16) || ((uintptr_t)out_bf16 % 16) || ((uintptr_t)w13 % 16) ||
       ((uintptr_t)w2 % 16))
     return MOE_E_ALIGN;
   DenseWs d = dense_layout(workspace, M, H, I, H);

@@ -34,6 +34,7 @@
 //   butterflies -> LDS across the wavefronts), scale = max(amax, 1e-10) / 448, h / scale -> e4m3fn.
 // GATED = false (second GEMM): the strip is 256 output columns, wavefront w owns 32 of them;
 //   the bf16 result row is written at its slot (t*K + k), which undoes the permutation.
+#include <cstddef>
 #include <type_traits>
 #include "moe_common.h"
 #include "moe_layout.h"
@@ -626,25 +627,31 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   __syncthreads();
 
   // ---- epilogue -------------------------------------------------------------------------------
+  // A lane holds 4 neighbouring columns of a row: stored from the registers, one instruction would touch 16 rows with
+  // a few bytes each.  The tile is laid down in LDS instead (the operand stages are idle now: every load has landed
+  // and the barrier above has passed) and streamed out in whole rows, 16 bytes per lane.
+  constexpr int RB = GATED ? (BF16 ? 256 : 128) : 512;         // bytes of one output row inside this strip
+  constexpr int RS = RB + (RB == 128 ? 16 : 32);               // row pitch in LDS: the lanes of a write hit different banks
+  static_assert(offsetof(Smem, arow) >= (size_t)BM * RS, "the staged output tile overlays the operand stages only");
+  uint8_t *const stage = (uint8_t *)&sm;
   if (GATED && BF16) {
     constexpr int G = WT / 2;                          // gate tiles per wavefront
-    uint16_t *const h = (uint16_t *)(shared ? a.sh_hq : a.hq);
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
-      const int i = mt * 16 + li;
-      if (i >= rows) continue;
+      if (mt < mt_live) {
 #pragma unroll
-      for (int j = 0; j < G; j++) {
-        float v[4];
+        for (int j = 0; j < G; j++) {
+          float v[4];
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-          const float g = acc[mt][j][r], u = acc[mt][j + G][r];
-          v[r] = silu_fast(g) * u;
+          for (int r = 0; r < 4; r++) {
+            const float g = acc[mt][j][r], u = acc[mt][j + G][r];
+            v[r] = silu_fast(g) * u;
+          }
+          v2i o;
+          o[0] = (int)pack2_bf16(v[0], v[1]);
+          o[1] = (int)pack2_bf16(v[2], v[3]);
+          *(v2i *)(stage + (mt * 16 + li) * RS + (wave * (16 * G) + j * 16 + lg * 4) * 2) = o;
         }
-        v2i o;
-        o[0] = (int)pack2_bf16(v[0], v[1]);
-        o[1] = (int)pack2_bf16(v[2], v[3]);
-        *(v2i *)(h + (size_t)(row0 + i) * a.N + strip * 128 + wave * (16 * G) + j * 16 + lg * 4) = o;
       }
     }
   } else if (GATED) {
@@ -670,39 +677,46 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
       const int i = mt * 16 + li;
-      const bool valid = i < rows;
       if (mt < mt_live) {
         float am = 0.f;
 #pragma unroll
         for (int w = 0; w < NW; w++) am = fmaxf(am, sm.amax[w][i]);
         const float sc = group_scale(am);
         const float inv = 1.0f / sc;                   // one division per row; the elements are multiplied
-        const size_t orow = (size_t)(row0 + i);
 #pragma unroll
-        for (int j = 0; j < G; j++) {
-          const uint32_t packed = pack4_fp8(acc[mt][j][0] * inv, acc[mt][j][1] * inv, acc[mt][j][2] * inv, acc[mt][j][3] * inv);
-          if (valid) *(uint32_t *)((shared ? a.sh_hq : a.hq) + orow * a.N + strip * 128 + wave * (16 * G) + j * 16 + lg * 4) = packed;
-        }
-        if (valid && wave == 0 && lg == 0) (shared ? a.sh_hs : a.hs)[orow * a.hs_pitch + strip] = sc;
+        for (int j = 0; j < G; j++)
+          *(uint32_t *)(stage + i * RS + wave * (16 * G) + j * 16 + lg * 4) =
+              pack4_fp8(acc[mt][j][0] * inv, acc[mt][j][1] * inv, acc[mt][j][2] * inv, acc[mt][j][3] * inv);
+        if (i < rows && wave == 0 && lg == 0) (shared ? a.sh_hs : a.hs)[(size_t)(row0 + i) * a.hs_pitch + strip] = sc;
       }
     }
   } else {
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
-      const int i = mt * 16 + li;
-      const bool valid = i < rows;
-      const int slot = sm.oslot[i];
-      if (mt < mt_live)
+      if (mt < mt_live) {
 #pragma unroll
-      for (int j = 0; j < WT; j++) {
-        const int col = strip * 256 + wave * (16 * WT) + j * 16 + lg * 4;
-        if (valid && col < a.N) {
+        for (int j = 0; j < WT; j++) {
           v2i o;
           o[0] = (int)pack2_bf16(acc[mt][j][0], acc[mt][j][1]);
           o[1] = (int)pack2_bf16(acc[mt][j][2], acc[mt][j][3]);
-          *(v2i *)((shared ? a.sh_y : a.y) + (size_t)slot * a.N + col) = o;
+          *(v2i *)(stage + (mt * 16 + li) * RS + (wave * (16 * WT) + j * 16 + lg * 4) * 2) = o;
         }
       }
+    }
+  }
+  __syncthreads();
+  {
+    constexpr int PIECES = RB / 16;                    // 16-byte pieces of a row
+    constexpr int RPI = 64 / PIECES;                   // rows one instruction of a wavefront moves
+    const int piece = lane % PIECES;
+    uint8_t *const out = GATED ? (shared ? a.sh_hq : a.hq) : (uint8_t *)(shared ? a.sh_y : a.y);
+    const size_t row_bytes = (size_t)a.N * (GATED && !BF16 ? 1 : 2);
+    // second GEMM: a strip is 256 columns, the matrix may end inside it (its width is a multiple of 8 columns)
+    const bool in_width = GATED || strip * 256 + piece * 8 < a.N;
+    for (int r = wave * RPI + lane / PIECES; r < rows; r += NW * RPI) {
+      const v4i d = *(const v4i *)(stage + r * RS + piece * 16);
+      const size_t orow = GATED ? (size_t)(row0 + r) : (size_t)sm.oslot[r];
+      if (in_width) *(v4i *)(out + orow * row_bytes + (size_t)strip * RB + piece * 16) = d;
     }
   }
 }
@@ -791,7 +805,7 @@ extern "C" int moe_gemm1_swiglu(void *stream, const uint8_t *xq, const float *xs
     return MOE_E_NULL;
   int rc = check_dims(T, H, I, E, K);
   if (rc) return rc;
-  if (((uintptr_t)xq % 16) || ((uintptr_t)w13 % 16) || ((uintptr_t)hq % 4) || ((uintptr_t)xs % 64) || ((uintptr_t)hs % 64))
+  if (((uintptr_t)xq % 16) || ((uintptr_t)w13 % 16) || ((uintptr_t)hq % 16) || ((uintptr_t)xs % 64) || ((uintptr_t)hs % 64))
     return MOE_E_ALIGN;
   if (T == 0) return MOE_OK;
   PermuteWs pw = permute_ws_layout(const_cast<void *>(permute_workspace), T, K, E);
@@ -807,7 +821,7 @@ extern "C" int moe_gemm2(void *stream, const uint8_t *hq, const float *hs, int T
     return MOE_E_NULL;
   int rc = check_dims(T, H, I, E, K);
   if (rc) return rc;
-  if (((uintptr_t)hq % 16) || ((uintptr_t)w2 % 16) || ((uintptr_t)y_bf16 % 8) || ((uintptr_t)hs % 64)) return MOE_E_ALIGN;
+  if (((uintptr_t)hq % 16) || ((uintptr_t)w2 % 16) || ((uintptr_t)y_bf16 % 16) || ((uintptr_t)hs % 64)) return MOE_E_ALIGN;
   if (T == 0) return MOE_OK;
   PermuteWs pw = permute_ws_layout(const_cast<void *>(permute_workspace), T, K, E);
   return gemm2_launch((hipStream_t)stream, hq, hs, T * K, T, H, w2, w2_scale, I, E, K, sorted_slot, expert_offsets, &pw,
