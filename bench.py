@@ -30,16 +30,16 @@ PEAK_HBM_GBS = 8000.0         # MI355X HBM3E, GB/s
 MEASURED_TRAFFIC = {(4096, 7168, 2048, 256, 8): 7.830e9}
 
 WORKLOADS = {
-    # BASELINE.json configs[2]: DeepSeek-V3-shaped prefill layer
+    # the headline configuration: DeepSeek-V3-shaped prefill layer
     "c3_prefill": dict(H=7168, I=2048, E=256, K=8, I_sh=2048, T=4096, route="sigmoid", n_groups=8, topk_groups=4,
                        scale=2.5, desc="DeepSeek-V3-shaped FP8 MoE layer, T=4096, E=256+1 shared, top-8"),
-    # configs[1]: Mixtral-8x7B-shaped layer at its largest T
+    # Mixtral-8x7B-shaped layer at its largest T
     "c2_prefill": dict(H=4096, I=14336, E=8, K=2, I_sh=0, T=4096, route="softmax", n_groups=1, topk_groups=1,
                        scale=1.0, desc="Mixtral-8x7B-shaped FP8 MoE layer, T=4096, E=8, top-2"),
-    # configs[4]: Qwen3-30B-A3B-shaped layer, Zipf(1.2) expert popularity, ~10% empty experts
+    # Qwen3-30B-A3B-shaped layer, Zipf(1.2) expert popularity, ~10% empty experts
     "c5_skewed": dict(H=2048, I=768, E=128, K=8, I_sh=0, T=16384, route="softmax", n_groups=1, topk_groups=1,
                       scale=1.0, zipf=1.2, empty=13, desc="Qwen3-30B-A3B-shaped FP8 MoE layer, T=16384, Zipf load"),
-    # configs[0]: toy
+    # toy size (the one a CPU runs in seconds)
     "c1_toy": dict(H=256, I=512, E=8, K=2, I_sh=0, T=16, route="softmax", n_groups=1, topk_groups=1, scale=1.0,
                    desc="toy FP8 MoE layer, T=16"),
 }
