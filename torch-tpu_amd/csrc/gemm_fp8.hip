@@ -10,7 +10,7 @@
 // Operand roles: the WEIGHT tile is the MFMA "A" operand (its 16 rows become the rows of the
 // 16x16 result) and the TOKEN tile is the "B" operand (its 16 rows become the columns).  A
 // lane then holds 4 consecutive output columns of ONE token, which makes the activation scale
-// a single value per lane and instruction, and lets the epilogue pack 4 outputs per store.
+// a single value per lane and instruction, and lets the epilogue pack 4 outputs at a time.
 //   lane l of an operand: row (l % 16), reduction bytes 16g..16g+15 and 64+16g..64+16g+15 of the
 //                         128-step, g = l / 16 (the instruction only needs both operands to agree;
 //                         this split makes the 128-bit LDS reads of the token tile conflict-free)
@@ -31,9 +31,10 @@
 // GATED = true  (first GEMM): the strip is 128 gate columns plus the 128 matching up columns of
 //   W13; wavefront w owns gate columns 16w..16w+15 and the same up columns.  Epilogue:
 //   h = silu(gate) * up, per-token amax over the strip's 128 columns (registers -> lane
-//   butterflies -> LDS across the wavefronts), scale = max(amax, 1e-10) / 448, h / scale -> e4m3fn.
+//   butterflies -> LDS across the wavefronts), scale = max(amax, 1e-10) / 448, h * (1 / scale) -> e4m3fn.
 // GATED = false (second GEMM): the strip is 256 output columns, wavefront w owns 32 of them;
 //   the bf16 result row is written at its slot (t*K + k), which undoes the permutation.
+// Both epilogues lay the output tile down in LDS and store it in whole rows.
 #include <cstddef>
 #include <type_traits>
 #include "moe_common.h"
