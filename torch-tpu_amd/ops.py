@@ -145,6 +145,20 @@ def act_quant(x):
 
 
 # --------------------------------------------------------------------------- experts
+def _shared_args(shared, H: int):
+    """(four device pointers, intermediate size) of an optional shared expert
+    (w13 [1,2Is,H], w13_scale, w2 [1,H,Is], w2_scale); all None and 0 without one."""
+    if shared is None:
+        return [None, None, None, None], 0
+    s13, s13s, s2, s2s = shared
+    I_sh = s13.shape[1] // 2
+    _need(tuple(s13.shape) == (1, 2 * I_sh, H) and tuple(s2.shape) == (1, H, I_sh), "bad shared expert shapes")
+    _need(tuple(s13s.shape) == (1, 2 * I_sh // 128, H // 128) and tuple(s2s.shape) == (1, H // 128, I_sh // 128),
+          "bad shared expert scale shapes")
+    return [_dev(s13, "shared w13", _FP8), _dev(s13s, "shared w13 scale", torch.float32),
+            _dev(s2, "shared w2", _FP8), _dev(s2s, "shared w2 scale", torch.float32)], I_sh
+
+
 def fused_experts_workspace_bytes(T, H, I, E, K, I_shared=0) -> int:
     return lib.moe_fused_experts_workspace_bytes(T, H, I, E, K, I_shared)
 
@@ -179,16 +193,7 @@ def fused_experts_fp8(x, w13, w13_scale, w2, w2_scale, ids, routing_weights=None
         _need(tuple(routing_weights.shape) == (T, K), "routing_weights must be [T, K]")
         rw_ptr = _dev(routing_weights, "routing_weights", torch.float32)
     _need(mode == 0 or rw_ptr is not None, "routing_weights are required for a [T,H] output")
-    sh = [None, None, None, None]
-    I_sh = 0
-    if shared is not None:
-        s13, s13s, s2, s2s = shared
-        I_sh = s13.shape[1] // 2
-        _need(tuple(s13.shape) == (1, 2 * I_sh, H) and tuple(s2.shape) == (1, H, I_sh), "bad shared expert shapes")
-        _need(tuple(s13s.shape) == (1, 2 * I_sh // 128, H // 128) and tuple(s2s.shape) == (1, H // 128, I_sh // 128),
-              "bad shared expert scale shapes")
-        sh = [_dev(s13, "shared w13", _FP8), _dev(s13s, "shared w13 scale", torch.float32),
-              _dev(s2, "shared w2", _FP8), _dev(s2s, "shared w2 scale", torch.float32)]
+    sh, I_sh = _shared_args(shared, H)
     need = fused_experts_workspace_bytes(T, H, I, E, K, I_sh)
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
@@ -239,16 +244,7 @@ def decode_layer_fp8(x, router_weight, w13, w13_scale, w2, w2_scale, top_k: int,
     if bias is not None:
         _need(bias.numel() == E, "bias must hold one value per expert")
         bias_ptr = _dev(bias, "bias", torch.float32)
-    sh = [None, None, None, None]
-    I_sh = 0
-    if shared is not None:
-        s13, s13s, s2, s2s = shared
-        I_sh = s13.shape[1] // 2
-        _need(tuple(s13.shape) == (1, 2 * I_sh, H) and tuple(s2.shape) == (1, H, I_sh), "bad shared expert shapes")
-        _need(tuple(s13s.shape) == (1, 2 * I_sh // 128, H // 128) and tuple(s2s.shape) == (1, H // 128, I_sh // 128),
-              "bad shared expert scale shapes")
-        sh = [_dev(s13, "shared w13", _FP8), _dev(s13s, "shared w13 scale", torch.float32),
-              _dev(s2, "shared w2", _FP8), _dev(s2s, "shared w2 scale", torch.float32)]
+    sh, I_sh = _shared_args(shared, H)
     need = decode_layer_workspace_bytes(T, H, I, E, top_k, I_sh)
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
