@@ -80,23 +80,45 @@ __global__ __launch_bounds__(1024) void permute_scan_kernel(int32_t *__restrict_
                                                             int32_t *__restrict__ tile_expert,
                                                             int32_t *__restrict__ tile_desc) {
   __shared__ int wave_sums[16];
-  const int e = threadIdx.x;
-  int count = 0;
-  if (e < E) {
-    // sixteen independent loads at a time (a load-add-store chain per chunk would pay one memory
-    // round trip per chunk)
-    constexpr int B = 16;
-    for (int c0 = 0; c0 < n_chunks; c0 += B) {
+  __shared__ int partial[1024];                       // [part][expert]: slots of the expert in that part of the chunks
+  // The chunks are cut into P parts and thread (part, expert) walks one part: its sum first, then - once the sums of
+  // the parts before it are known - the running count that turns each chunk's histogram entry into the rank of the
+  // chunk's first slot inside the expert.  Sixteen independent loads at a time in both passes (a load-add-store chain
+  // per chunk would pay one memory round trip per chunk).
+  int epad = 1;
+  while (epad < E) epad <<= 1;
+  const int P = 1024 / epad, part = threadIdx.x / epad, pe = threadIdx.x % epad;
+  const int len = (n_chunks + P - 1) / P, c_lo = part * len, c_hi = min(n_chunks, c_lo + len);
+  constexpr int B = 16;
+  int sum = 0;
+  if (pe < E)
+    for (int c0 = c_lo; c0 < c_hi; c0 += B) {
       int x[B];
 #pragma unroll
-      for (int i = 0; i < B; i++) x[i] = c0 + i < n_chunks ? chunk_counts[(size_t)(c0 + i) * E + e] : 0;
+      for (int i = 0; i < B; i++) x[i] = c0 + i < c_hi ? chunk_counts[(size_t)(c0 + i) * E + pe] : 0;
+#pragma unroll
+      for (int i = 0; i < B; i++) sum += x[i];
+    }
+  partial[threadIdx.x] = sum;
+  __syncthreads();
+  if (pe < E) {
+    int run = 0;
+    for (int q = 0; q < part; q++) run += partial[q * epad + pe];
+    for (int c0 = c_lo; c0 < c_hi; c0 += B) {
+      int x[B];
+#pragma unroll
+      for (int i = 0; i < B; i++) x[i] = c0 + i < c_hi ? chunk_counts[(size_t)(c0 + i) * E + pe] : 0;
 #pragma unroll
       for (int i = 0; i < B; i++) {
-        if (c0 + i < n_chunks) chunk_counts[(size_t)(c0 + i) * E + e] = count;   // rank of the chunk's first slot inside expert e
-        count += x[i];
+        if (c0 + i < c_hi) chunk_counts[(size_t)(c0 + i) * E + pe] = run;   // rank of the chunk's first slot inside the expert
+        run += x[i];
       }
     }
   }
+  const int e = threadIdx.x;
+  int count = 0;
+  if (e < E)
+    for (int q = 0; q < P; q++) count += partial[q * epad + e];
   int total;
   int off = block_exclusive_scan(count, wave_sums, total);
   int tiles = (count + tile_m - 1) / tile_m;
