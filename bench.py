@@ -368,6 +368,20 @@ def main():
         result["decode"] = bench_decode(pkg, moe, cfg, dev, args.steps, args.warmup)
     if not args.no_decode and args.workload == "c3_prefill":
         result["dense"] = bench_dense(pkg, dev, args.steps, args.warmup)
+        # the two matrix-core-bound layer shapes of the same benchmark definition, same step, for the record
+        others = []
+        for name in ("c2_prefill", "c5_skewed"):
+            ocfg = WORKLOADS[name]
+            omoe = build_layer(pkg, ocfg, dev)
+            osec, oroof, _ = bench_prefill(pkg, omoe, ocfg, dev, args.steps, args.warmup)
+            oflops = gemm_flops(ocfg, ocfg["T"])
+            others.append(dict(workload=f"{name}: {ocfg['desc']}", ms_per_step=osec * 1e3, tflops=oflops / osec / 1e12,
+                               mfma_frac_of_peak=oflops / osec / 1e12 / PEAK_FP8_TFLOPS,
+                               tokens_per_s=ocfg["T"] / osec, first_gemm_ms=oroof["launch_ms"],
+                               first_gemm_tflops=oroof["mfma_tflops"], second_gemm_ms=oroof["second_gemm"]["launch_ms"],
+                               second_gemm_tflops=oroof["second_gemm"]["mfma_tflops"]))
+            del omoe
+        result["other_shapes"] = others
     if not args.no_cpu:
         base, parity = cpu_baseline(pkg, moe, cfg, x, min(args.cpu_sample, T))
         result["cpu_baseline"] = base
