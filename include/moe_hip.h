@@ -32,6 +32,9 @@
 extern "C" {
 #endif
 
+/* Pointers to per-token data (activations, ids, routing weights, outputs) may be NULL when the
+ * token count is 0: an empty batch is a valid call that does nothing (moe_permute still writes
+ * its all-zero expert_offsets). */
 #define MOE_OK                0
 #define MOE_E_NULL           -1   /* a required pointer is NULL                          */
 #define MOE_E_SHAPE          -2   /* a dimension is out of the supported range           */

@@ -141,3 +141,16 @@ def test_checkpoint_layout_conversion_is_pure_data_movement(pkg, oracle):
     sw13, sw13s, sw2, sw2s = out["shared"]
     assert sw13.shape == (1, 2 * I, H) and sw2.shape == (1, H, I) and sw13s.dtype == torch.float32
     assert torch.equal(out["bias"], state[pre + "gate.e_score_correction_bias"])
+
+
+def test_size_functions_accept_an_empty_batch(pkg):
+    """Workspace sizes are host arithmetic: they must not trip over a token count of zero."""
+    lib = pkg._lib.lib
+    assert lib.moe_permute_workspace_bytes(0, 2, 8) > 0
+    assert lib.moe_fused_experts_workspace_bytes(0, 256, 128, 8, 2, 0) > 0
+    assert lib.moe_fused_experts_workspace_bytes(0, 256, 128, 8, 2, 128) > 0
+    assert lib.moe_decode_layer_fp8_workspace_bytes(0, 256, 128, 8, 2, 0) > 0
+    assert lib.moe_fused_experts_bf16_workspace_bytes(0, 256, 128, 8, 2) > 0
+    assert lib.moe_mm_fp8_workspace_bytes(0, 256, 256) > 0
+    assert lib.moe_mlp_fp8_workspace_bytes(0, 256, 128) > 0
+    assert lib.moe_tile_rows(0, 2, 8) == 16

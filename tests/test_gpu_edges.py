@@ -1,0 +1,103 @@
+"""Edge cases of the HIP path through the C ABI: empty batches, ids outside [0, E), a workspace that
+is reused by calls of different sizes, and the largest expert / top-k counts."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def test_empty_batch_is_a_valid_call_everywhere(pkg, oracle, dev):
+    say("empty batch")
+    H, I, E, K = 256, 128, 8, 2
+    ld = tuple(t.to(dev) for t in oracle.make_layer(E, H, I, seed=3))
+    x = torch.empty(0, H, dtype=torch.bfloat16, device=dev)
+    ids = torch.empty(0, K, dtype=torch.int32, device=dev)
+    w = torch.empty(0, K, dtype=torch.float32, device=dev)
+    wr = torch.zeros(E, H, dtype=torch.bfloat16, device=dev)
+    # routing
+    wt, idx = pkg.moe_route(torch.empty(0, E, device=dev), K, "softmax")
+    assert wt.shape == (0, K) and idx.shape == (0, K)
+    v = torch.empty(0, K, device=dev)
+    i = torch.empty(0, K, dtype=torch.int32, device=dev)
+    pkg.noaux_tc_topk(v, i, torch.empty(0, E, device=dev), 1, 1, K)
+    # permutation: nothing to place, every expert starts and ends at row 0
+    ss, off, s2r = pkg.moe_permute(ids, E)
+    torch.cuda.synchronize()
+    assert ss.numel() == 0 and s2r.numel() == 0 and torch.equal(off.cpu(), torch.zeros(E + 1, dtype=torch.int32))
+    # quantiser, experts (both output forms), un-quantised experts, dense layers, the one-call layer
+    q, s = pkg.act_quant(x)
+    assert q.shape == (0, H)
+    assert pkg.fused_experts_fp8(x, *ld, ids).shape == (0, K, H)
+    assert pkg.fused_experts_fp8(x, *ld, ids, w).shape == (0, H)
+    w13b = torch.zeros(E, 2 * I, H, dtype=torch.bfloat16, device=dev)
+    w2b = torch.zeros(E, H, I, dtype=torch.bfloat16, device=dev)
+    assert pkg.fused_experts_bf16(x, w13b, w2b, ids, w).shape == (0, H)
+    assert pkg.mm_fp8(x, ld[0][0], ld[1][0]).shape == (0, 2 * I)
+    assert pkg.mlp_fp8(x, ld[0][0], ld[1][0], ld[2][0], ld[3][0]).shape == (0, H)
+    moe = pkg.FusedMoE(wr, *ld, top_k=K, mode="softmax")
+    assert moe(x).shape == (0, H)
+    torch.cuda.synchronize()
+
+
+def test_ids_outside_the_expert_range_are_dropped(pkg, oracle, dev):
+    say("ids out of range")
+    T, E, K = 37, 16, 4
+    g = torch.Generator().manual_seed(9)
+    ids = torch.argsort(torch.rand(T, E, generator=g), dim=-1)[:, :K].to(torch.int32)
+    bad = torch.rand(T, K, generator=g) < 0.2
+    ids[bad] = torch.where(torch.rand(int(bad.sum()), generator=g) < 0.5, torch.tensor(-1), torch.tensor(E + 3)).to(torch.int32)
+    ss, off, s2r = pkg.moe_permute(ids.to(dev), E)
+    torch.cuda.synchronize()
+    flat = ids.flatten()
+    valid = (flat >= 0) & (flat < E)
+    n_valid = int(valid.sum())
+    counts = torch.bincount(flat[valid].long(), minlength=E)
+    off_ref = torch.zeros(E + 1, dtype=torch.int64)
+    off_ref[1:] = torch.cumsum(counts, 0)
+    assert torch.equal(off.cpu().long(), off_ref)
+    # the valid slots in stable expert order, the dropped ones nowhere
+    order = torch.sort(torch.where(valid, flat, torch.tensor(E, dtype=torch.int32)).long(), stable=True).indices[:n_valid]
+    assert torch.equal(ss.cpu()[:n_valid].long(), order)
+    s2r = s2r.cpu()
+    assert bool((s2r[~valid] == -1).all())
+    inv = torch.full((T * K,), -1, dtype=torch.int64)
+    inv[order] = torch.arange(n_valid)
+    assert torch.equal(s2r.long(), inv)
+
+
+def test_one_workspace_serves_calls_of_different_sizes(pkg, oracle, dev):
+    say("workspace reuse")
+    H, I, E, K = 512, 256, 16, 4
+    ld = tuple(t.to(dev) for t in oracle.make_layer(E, H, I, seed=4))
+    sizes = [300, 3, 70, 1, 129]
+    ws = torch.empty(pkg.fused_experts_workspace_bytes(max(sizes), H, I, E, K), dtype=torch.uint8, device=dev)
+    ws.fill_(0xA5)
+    g = torch.Generator().manual_seed(4)
+    for T in sizes:
+        x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+        ids = torch.argsort(torch.rand(T, E, generator=g), dim=-1)[:, :K].to(torch.int32).to(dev)
+        w = torch.rand(T, K, generator=g).to(dev)
+        shared_ws = pkg.fused_experts_fp8(x, *ld, ids, w, workspace=ws)
+        fresh_ws = pkg.fused_experts_fp8(x, *ld, ids, w)
+        assert torch.equal(shared_ws.view(torch.int16), fresh_ws.view(torch.int16)), T
+
+
+def test_largest_expert_and_topk_counts(pkg, oracle, dev):
+    say("E=1024, K=32")
+    T, H, I, E, K = 40, 256, 128, 1024, 32
+    layer = oracle.make_layer(E, H, I, seed=6)
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    logits = torch.randn(T, E, generator=g)
+    w_ref, ids_ref = oracle.route_softmax_topk(logits, K)
+    w, ids = pkg.moe_route(logits.to(dev), K, "softmax")
+    assert torch.equal(ids.cpu(), ids_ref)
+    out = pkg.fused_experts_fp8(x.to(dev), *(t.to(dev) for t in layer), ids, w)
+    torch.cuda.synchronize()
+    ref = oracle.moe_w8a8_fp32(x, ids_ref, w_ref, *layer)
+    bad = (out.float().cpu() - ref).abs() > 1e-2 + 2e-2 * ref.abs()
+    assert bad.float().mean().item() <= 5e-3

@@ -154,9 +154,11 @@ extern "C" int moe_fused_experts_fp8(void *stream, const void *x_bf16, int T, in
                                      const uint8_t *shared_w2, const float *shared_w2_scale, int I_shared,
                                      void *out_bf16, int out_mode, void *workspace, size_t workspace_bytes) {
   using namespace moe;
-  if (!x_bf16 || !w13 || !w13_scale || !w2 || !w2_scale || !ids || !out_bf16 || !workspace) return MOE_E_NULL;
+  // per-token pointers may be NULL for an empty batch (T == 0): nothing is read or written through them
+  if (!w13 || !w13_scale || !w2 || !w2_scale || !workspace) return MOE_E_NULL;
+  if (T != 0 && (!x_bf16 || !ids || !out_bf16)) return MOE_E_NULL;
   if (out_mode != 0 && out_mode != 1) return MOE_E_MODE;
-  if (out_mode == 1 && !routing_weights) return MOE_E_NULL;
+  if (T != 0 && out_mode == 1 && !routing_weights) return MOE_E_NULL;
   if (T < 0 || H < 1 || I < 1 || E < 1 || E > MOE_MAX_EXPERTS || K < 1 || K > MOE_MAX_TOPK || K > E) return MOE_E_SHAPE;
   if ((long)T * K > (1l << 30)) return MOE_E_SHAPE;
   if (H % kBlock || I % kBlock) return MOE_E_ALIGN;
@@ -198,7 +200,8 @@ extern "C" int moe_decode_layer_fp8(void *stream, const void *x_bf16, int T, int
                                     const float *shared_w2_scale, int I_shared, void *out_bf16, void *logits_out_bf16,
                                     float *weights_out, int32_t *ids_out, void *workspace, size_t workspace_bytes) {
   using namespace moe;
-  if (!x_bf16 || !router_w_bf16 || !w13 || !w13_scale || !w2 || !w2_scale || !out_bf16 || !workspace) return MOE_E_NULL;
+  if (!router_w_bf16 || !w13 || !w13_scale || !w2 || !w2_scale || !workspace) return MOE_E_NULL;
+  if (T != 0 && (!x_bf16 || !out_bf16)) return MOE_E_NULL;
   if (T < 0 || H < 1 || I < 1 || E < 1 || E > 256 || K < 1 || K > MOE_MAX_TOPK || K > E) return MOE_E_SHAPE;
   if ((long)T * K > kChunk) return MOE_E_SHAPE;
   if (H % kBlock || I % kBlock) return MOE_E_ALIGN;
@@ -275,7 +278,8 @@ extern "C" size_t moe_mm_fp8_workspace_bytes(int M, int K, int N) {
 extern "C" int moe_mm_fp8(void *stream, const void *x_bf16, int M, int K, const uint8_t *w, const float *w_scale,
                           int N, void *out_bf16, void *workspace, size_t workspace_bytes) {
   using namespace moe;
-  if (!x_bf16 || !w || !w_scale || !out_bf16 || !workspace) return MOE_E_NULL;
+  if (!w || !w_scale || !workspace) return MOE_E_NULL;
+  if (M != 0 && (!x_bf16 || !out_bf16)) return MOE_E_NULL;
   if (M < 0 || K < 1 || N < 16 || K > 32768 || N > (1 << 20)) return MOE_E_SHAPE;
   if (K % kBlock || N % 16) return MOE_E_ALIGN;
   if ((double)M * K >= 2147483648.0 || (double)M * N >= 2147483648.0 || (double)N * K >= 4294967296.0) return MOE_E_SHAPE;
@@ -301,7 +305,8 @@ extern "C" int moe_mlp_fp8(void *stream, const void *x_bf16, int M, int H, const
                            const uint8_t *w2, const float *w2_scale, int I, void *out_bf16, void *workspace,
                            size_t workspace_bytes) {
   using namespace moe;
-  if (!x_bf16 || !w13 || !w13_scale || !w2 || !w2_scale || !out_bf16 || !workspace) return MOE_E_NULL;
+  if (!w13 || !w13_scale || !w2 || !w2_scale || !workspace) return MOE_E_NULL;
+  if (M != 0 && (!x_bf16 || !out_bf16)) return MOE_E_NULL;
   if (M < 0 || H < 1 || I < 1 || H > 32768 || I > 32768) return MOE_E_SHAPE;
   if (H % kBlock || I % kBlock) return MOE_E_ALIGN;
   if ((double)M * H >= 2147483648.0 || (double)M * I >= 2147483648.0) return MOE_E_SHAPE;
@@ -368,9 +373,10 @@ extern "C" int moe_fused_experts_bf16(void *stream, const void *x_bf16, int T, i
                                       const float *routing_weights, int K, void *out_bf16, int out_mode,
                                       void *workspace, size_t workspace_bytes) {
   using namespace moe;
-  if (!x_bf16 || !w13_bf16 || !w2_bf16 || !ids || !out_bf16 || !workspace) return MOE_E_NULL;
+  if (!w13_bf16 || !w2_bf16 || !workspace) return MOE_E_NULL;
+  if (T != 0 && (!x_bf16 || !ids || !out_bf16)) return MOE_E_NULL;
   if (out_mode != 0 && out_mode != 1) return MOE_E_MODE;
-  if (out_mode == 1 && !routing_weights) return MOE_E_NULL;
+  if (T != 0 && out_mode == 1 && !routing_weights) return MOE_E_NULL;
   if (T < 0 || H < 1 || I < 1 || E < 1 || E > MOE_MAX_EXPERTS || K < 1 || K > MOE_MAX_TOPK || K > E) return MOE_E_SHAPE;
   if ((long)T * K > (1l << 30) || H > 16384 || I > 16384) return MOE_E_SHAPE;
   if (H % kBlock || I % kBlock) return MOE_E_ALIGN;

@@ -184,7 +184,7 @@ void dense_small_plan(int M, int K, int N, int *n_splits, int *split_len, int *r
                       int *tiles_per_item) {
   const int NKB = K / kBlock;
   const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-  const int chunks = (M + 16 * mt - 1) / (16 * mt);
+  const int chunks = M > 0 ? (M + 16 * mt - 1) / (16 * mt) : 1;        // an empty batch plans like one row
   // four weight tiles per item when the layer is wide enough to still fill the chip with short slices
   const int ntw = (N % 64 == 0 && (long)(N / 64) * chunks * (NKB / 8) >= 1024) ? 4 : 1;
   *tiles_per_item = ntw;

@@ -802,8 +802,8 @@ extern "C" int moe_gemm1_swiglu(void *stream, const uint8_t *xq, const float *xs
                                 const float *w13_scale, int I, int E, int K, const int32_t *sorted_slot,
                                 const int32_t *expert_offsets, const void *permute_workspace, uint8_t *hq, float *hs) {
   using namespace moe;
-  if (!xq || !xs || !w13 || !w13_scale || !sorted_slot || !expert_offsets || !permute_workspace || !hq || !hs)
-    return MOE_E_NULL;
+  if (!w13 || !w13_scale || !expert_offsets || !permute_workspace) return MOE_E_NULL;
+  if (T != 0 && (!xq || !xs || !sorted_slot || !hq || !hs)) return MOE_E_NULL;
   int rc = check_dims(T, H, I, E, K);
   if (rc) return rc;
   if (((uintptr_t)xq % 16) || ((uintptr_t)w13 % 16) || ((uintptr_t)hq % 16) || ((uintptr_t)xs % 64) || ((uintptr_t)hs % 64))
@@ -818,8 +818,8 @@ extern "C" int moe_gemm2(void *stream, const uint8_t *hq, const float *hs, int T
                          const float *w2_scale, int I, int E, int K, const int32_t *sorted_slot,
                          const int32_t *expert_offsets, const void *permute_workspace, void *y_bf16) {
   using namespace moe;
-  if (!hq || !hs || !w2 || !w2_scale || !sorted_slot || !expert_offsets || !permute_workspace || !y_bf16)
-    return MOE_E_NULL;
+  if (!w2 || !w2_scale || !expert_offsets || !permute_workspace) return MOE_E_NULL;
+  if (T != 0 && (!hq || !hs || !sorted_slot || !y_bf16)) return MOE_E_NULL;
   int rc = check_dims(T, H, I, E, K);
   if (rc) return rc;
   if (((uintptr_t)hq % 16) || ((uintptr_t)w2 % 16) || ((uintptr_t)y_bf16 % 16) || ((uintptr_t)hs % 64)) return MOE_E_ALIGN;

@@ -211,7 +211,8 @@ extern "C" int moe_tile_rows(int T, int K, int E) { return moe::choose_tile_m(T,
 extern "C" int moe_permute(void *stream, const int32_t *ids, int T, int K, int E, int32_t *sorted_slot,
                            int32_t *expert_offsets, int32_t *slot_to_row, void *workspace, size_t workspace_bytes) {
   using namespace moe;
-  if (!ids || !sorted_slot || !expert_offsets || !slot_to_row || !workspace) return MOE_E_NULL;
+  if (!expert_offsets || !workspace) return MOE_E_NULL;
+  if (T != 0 && (!ids || !sorted_slot || !slot_to_row)) return MOE_E_NULL;   // an empty batch still gets its (all zero) offsets
   if (T < 0 || K < 1 || K > MOE_MAX_TOPK || E < 1 || E > MOE_MAX_EXPERTS) return MOE_E_SHAPE;
   if ((long)T * K > (1l << 30)) return MOE_E_SHAPE;
   if (workspace_bytes < permute_ws_bytes(T, K, E)) return MOE_E_WORKSPACE;

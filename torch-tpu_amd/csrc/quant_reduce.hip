@@ -59,7 +59,7 @@ extern "C" int moe_scale_pitch(int n_groups) { return n_groups < 0 ? 0 : moe::sc
 
 extern "C" int moe_act_quant(void *stream, const void *x_bf16, int R, int C, uint8_t *q, float *s) {
   using namespace moe;
-  if (!x_bf16 || !q || !s) return MOE_E_NULL;
+  if (R != 0 && (!x_bf16 || !q || !s)) return MOE_E_NULL;
   if (R < 0 || C < 1) return MOE_E_SHAPE;
   if (C % kBlock) return MOE_E_ALIGN;
   if (((uintptr_t)x_bf16 % 16) || ((uintptr_t)q % 8) || ((uintptr_t)s % 64)) return MOE_E_ALIGN;
@@ -75,7 +75,7 @@ extern "C" int moe_act_quant(void *stream, const void *x_bf16, int R, int C, uin
 extern "C" int moe_weighted_reduce(void *stream, const void *y_bf16, const float *routing_weights,
                                    const void *shared_y_bf16, int T, int K, int H, void *out_bf16) {
   using namespace moe;
-  if (!y_bf16 || !routing_weights || !out_bf16) return MOE_E_NULL;
+  if (T != 0 && (!y_bf16 || !routing_weights || !out_bf16)) return MOE_E_NULL;
   if (T < 0 || K < 1 || H < 1) return MOE_E_SHAPE;
   if (H % 8) return MOE_E_ALIGN;
   if (((uintptr_t)y_bf16 % 16) || ((uintptr_t)out_bf16 % 16) || (shared_y_bf16 && ((uintptr_t)shared_y_bf16 % 16)))

@@ -292,7 +292,7 @@ int check_route_shape(int T, int E, int K, int n_groups, int topk_groups) {
 extern "C" int moe_noaux_tc_topk(void *stream, const void *scores, int scores_dtype, int T, int E, int n_groups,
                                  int topk_groups, int top_k, void *values_out, int32_t *indices_out) {
   using namespace moe;
-  if (!scores || !values_out || !indices_out) return MOE_E_NULL;
+  if (T != 0 && (!scores || !values_out || !indices_out)) return MOE_E_NULL;
   if (scores_dtype != MOE_DTYPE_F32 && scores_dtype != MOE_DTYPE_BF16) return MOE_E_MODE;
   int rc = check_route_shape(T, E, top_k, n_groups, topk_groups);
   if (rc) return rc;
@@ -309,7 +309,7 @@ extern "C" int moe_route_topk(void *stream, const void *logits, int logits_dtype
                               int K, int mode, int n_groups, int topk_groups, int renorm, float scale,
                               float *weights_out, int32_t *ids_out, float *scores_out) {
   using namespace moe;
-  if (!logits || !weights_out || !ids_out) return MOE_E_NULL;
+  if (T != 0 && (!logits || !weights_out || !ids_out)) return MOE_E_NULL;
   if (logits_dtype != MOE_DTYPE_F32 && logits_dtype != MOE_DTYPE_BF16) return MOE_E_MODE;
   if (mode != MOE_ROUTE_SOFTMAX && mode != MOE_ROUTE_SIGMOID && mode != MOE_ROUTE_SCORES) return MOE_E_MODE;
   int rc = check_route_shape(T, E, K, n_groups, topk_groups);
