@@ -82,6 +82,7 @@ LAYER_CASES = [
     (19, 1280, 128, 100, 4, "sigmoid", 4, 2, True, 384),
     (32, 2304, 128, 256, 8, "sigmoid", 8, 4, False, 128),
     (3, 8192 + 1024, 128, 16, 3, "sigmoid", 1, 1, False, 0),
+    (8, 7168, 2048, 256, 8, "sigmoid", 8, 4, True, 2048),        # the DeepSeek-V3 layer at its real size
 ]
 
 
@@ -94,10 +95,16 @@ def test_decode_layer_entry_point(pkg, oracle, dev, T, H, I, E, K, mode, G, TG, 
         ld = tuple(t.to(dev) for t in layer)
     else:                                   # too large to make on the host: random weights made on the device
         gd = torch.Generator(device=dev).manual_seed(T + E)
-        w13 = (torch.randn(E, 2 * I, H, generator=gd, device=dev) * 0.02).to(torch.bfloat16)
-        w2 = (torch.randn(E, H, I, generator=gd, device=dev) * 0.02).to(torch.bfloat16)
-        ld = (*pkg.quant_weight_block128(w13), *pkg.quant_weight_block128(w2))
-        del w13, w2
+
+        def make(n, k):                      # in slices of experts: the fp32 intermediates of a whole layer are large
+            q = torch.empty(E, n, k, dtype=torch.float8_e4m3fn, device=dev)
+            sc = torch.empty(E, n // 128, k // 128, dtype=torch.float32, device=dev)
+            step = max(1, (1 << 27) // (n * k))
+            for e0 in range(0, E, step):
+                w = (torch.randn(min(step, E - e0), n, k, generator=gd, device=dev) * 0.02).to(torch.bfloat16)
+                q[e0:e0 + step], sc[e0:e0 + step] = pkg.quant_weight_block128(w)
+            return q, sc
+        ld = (*make(2 * I, H), *make(H, I))
     g = torch.Generator().manual_seed(7 * T + E)
     x = torch.randn(T, H, generator=g).to(torch.bfloat16)
     wr = (torch.randn(E, H, generator=g) * 0.05).to(torch.bfloat16)
