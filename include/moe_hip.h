@@ -202,23 +202,25 @@ int moe_mlp_fp8(void *stream, const void *x_bf16, int M, int H, const uint8_t *w
                 size_t workspace_bytes);
 
 /*
- * Router and experts of one layer in a single call, for decode-size batches: T * K <= 256 slots and
- * E <= 256 experts (MOE_E_SHAPE beyond that - route, then moe_fused_experts_fp8, cover every size).
- * Replaces, in one go, what the reference's callers chain on the host for every token batch
- * (python/regression/test_llm/test_torch_ops.py:441-456: logits = x Wr^T in bf16 -> sigmoid -> top-k ->
- * renormalise -> scale) and the expert op behind it (torch_tpu/csrc/ops/my_ops/fusedMoE.cpp:117-236).
- * Two launches stand in front of the grouped GEMMs instead of five: the router logits (fp32 sums rounded
- * to bf16) together with the activation quantisation, then routing and permutation.
+ * Router and experts of one layer in a single call, E <= 256 experts (MOE_E_SHAPE beyond that: the staged
+ * calls cover every size).  Replaces, in one go, what the reference's callers chain on the host for every
+ * token batch (python/regression/test_llm/test_torch_ops.py:440-456: logits = x Wr^T in bf16 -> sigmoid ->
+ * top-k -> renormalise -> scale) and the expert op behind it
+ * (torch_tpu/csrc/ops/my_ops/fusedMoE.cpp:117-236).
+ * Decode-size batches (T * K <= 256 slots): two launches stand in front of the grouped GEMMs - the router
+ * logits together with the activation quantisation, then routing and permutation.  Larger batches: the
+ * router product runs on the matrix cores with its reduction cut into slices, and the routing kernel adds
+ * the slices.  Either way the logits are fp32 sums rounded once to bf16.
  * router_w_bf16 [E, H] bf16; router_bias [E] fp32 or NULL (selection only, as in moe_route_topk);
  * mode MOE_ROUTE_SOFTMAX or MOE_ROUTE_SIGMOID; the other routing arguments as in moe_route_topk.
  * out bf16 [T, H] (the weighted sum, shared expert added when its pointers are non-NULL).
  * logits_out_bf16 [T, E], weights_out [T, K], ids_out [T, K]: optional copies of what the router
  * produced (NULL to skip).  Given the same logits, ids and weights equal moe_route_topk's, and given the
  * same ids and weights the output equals moe_fused_experts_fp8's, bit for bit.
- * workspace: moe_decode_layer_fp8_workspace_bytes(...) bytes, 256-byte aligned.
+ * workspace: moe_layer_fp8_workspace_bytes(...) bytes, 256-byte aligned.
  */
-size_t moe_decode_layer_fp8_workspace_bytes(int T, int H, int I, int E, int K, int I_shared);
-int moe_decode_layer_fp8(void *stream, const void *x_bf16, int T, int H,
+size_t moe_layer_fp8_workspace_bytes(int T, int H, int I, int E, int K, int I_shared);
+int moe_layer_fp8(void *stream, const void *x_bf16, int T, int H,
                          const void *router_w_bf16, const float *router_bias, int E, int K, int mode,
                          int n_groups, int topk_groups, int renorm, float scale,
                          const uint8_t *w13, const float *w13_scale,
@@ -227,6 +229,16 @@ int moe_decode_layer_fp8(void *stream, const void *x_bf16, int T, int H,
                          const uint8_t *shared_w2, const float *shared_w2_scale, int I_shared,
                          void *out_bf16, void *logits_out_bf16, float *weights_out, int32_t *ids_out,
                          void *workspace, size_t workspace_bytes);
+
+/*
+ * The router product on its own (any T, E <= 256): logits [T, E] bf16 = x [T, H] . router_w [E, H]^T, the
+ * first step of the routing recipe (test_torch_ops.py:440).  The kernel moe_layer_fp8 uses for batches
+ * beyond the decode size, followed by the sum over its slices.
+ * workspace: moe_router_logits_workspace_bytes(T, H, E) bytes, 256-byte aligned.
+ */
+size_t moe_router_logits_workspace_bytes(int T, int H, int E);
+int moe_router_logits(void *stream, const void *x_bf16, int T, int H, const void *router_w_bf16, int E,
+                      void *logits_bf16, void *workspace, size_t workspace_bytes);
 
 #ifdef __cplusplus
 }

@@ -149,7 +149,7 @@ def test_size_functions_accept_an_empty_batch(pkg):
     assert lib.moe_permute_workspace_bytes(0, 2, 8) > 0
     assert lib.moe_fused_experts_workspace_bytes(0, 256, 128, 8, 2, 0) > 0
     assert lib.moe_fused_experts_workspace_bytes(0, 256, 128, 8, 2, 128) > 0
-    assert lib.moe_decode_layer_fp8_workspace_bytes(0, 256, 128, 8, 2, 0) > 0
+    assert lib.moe_layer_fp8_workspace_bytes(0, 256, 128, 8, 2, 0) > 0
     assert lib.moe_fused_experts_bf16_workspace_bytes(0, 256, 128, 8, 2) > 0
     assert lib.moe_mm_fp8_workspace_bytes(0, 256, 256) > 0
     assert lib.moe_mlp_fp8_workspace_bytes(0, 256, 128) > 0

@@ -1,5 +1,5 @@
-"""Decode-size batches: the workgroup-per-token routing kernel and the one-call layer entry point
-(moe_decode_layer_fp8), through the C ABI, on a real MI355X.
+"""The one-call layer entry point (moe_layer_fp8: router and experts) at decode sizes and beyond, and the
+workgroup-per-token routing kernel, through the C ABI, on a real MI355X.
 
 What must hold, bit for bit: the routing of a small batch equals the routing of the same rows inside
 a large batch (two different kernels) and the oracle's ids; given the logits the entry point produced, its
@@ -83,6 +83,11 @@ LAYER_CASES = [
     (32, 2304, 128, 256, 8, "sigmoid", 8, 4, False, 128),
     (3, 8192 + 1024, 128, 16, 3, "sigmoid", 1, 1, False, 0),
     (8, 7168, 2048, 256, 8, "sigmoid", 8, 4, True, 2048),        # the DeepSeek-V3 layer at its real size
+    # beyond the decode size: the router product on the matrix cores, reduction in slices
+    (300, 1024, 256, 64, 6, "softmax", 1, 1, False, 0),
+    (77, 512, 128, 8, 4, "sigmoid", 1, 1, True, 128),
+    (1000, 7168, 256, 256, 8, "sigmoid", 8, 4, True, 256),
+    (4096, 2048, 128, 250, 5, "sigmoid", 1, 1, False, 0),
 ]
 
 
@@ -114,7 +119,7 @@ def test_decode_layer_entry_point(pkg, oracle, dev, T, H, I, E, K, mode, G, TG, 
     shared = _shared(pkg, oracle, H, I_sh, 99, dev) if I_sh else None
     kw = dict(bias=biasd, n_groups=G, topk_groups=TG, renorm=True, scale=2.5 if mode == "sigmoid" else 1.0)
 
-    out, logits, w, ids = pkg.decode_layer_fp8(xd, wrd, *ld, K, mode, shared=shared, return_routing=True, **kw)
+    out, logits, w, ids = pkg.layer_fp8(xd, wrd, *ld, K, mode, shared=shared, return_routing=True, **kw)
     torch.cuda.synchronize()
     # logits: bf16 rounding of the exact product
     exact = x.double() @ wr.double().t()
@@ -128,9 +133,9 @@ def test_decode_layer_entry_point(pkg, oracle, dev, T, H, I, E, K, mode, G, TG, 
     ref_out = pkg.fused_experts_fp8(xd, *ld, ids, w, shared=shared)
     assert torch.equal(out.view(torch.int16), ref_out.view(torch.int16))
     # a second call into the same workspace (the arrival counter starts over), without the optional outputs
-    ws = torch.empty(pkg.decode_layer_workspace_bytes(T, H, I, E, K, I_sh), dtype=torch.uint8, device=dev)
+    ws = torch.empty(pkg.layer_workspace_bytes(T, H, I, E, K, I_sh), dtype=torch.uint8, device=dev)
     for _ in range(2):
-        again = pkg.decode_layer_fp8(xd, wrd, *ld, K, mode, shared=shared, workspace=ws, **kw)
+        again = pkg.layer_fp8(xd, wrd, *ld, K, mode, shared=shared, workspace=ws, **kw)
         assert torch.equal(again.view(torch.int16), out.view(torch.int16))
     # the module takes this road by itself for such a batch
     moe = pkg.FusedMoE(wrd, *ld, top_k=K, mode=mode, bias=biasd, n_groups=G, topk_groups=TG, renorm=True,
@@ -153,6 +158,23 @@ def test_decode_layer_entry_point(pkg, oracle, dev, T, H, I, E, K, mode, G, TG, 
         assert bad.float().mean().item() <= 2e-3
     else:
         assert mode == "sigmoid"
+
+
+@pytest.mark.parametrize("T,H,E", [(1, 128, 1), (5, 7168, 256), (64, 256, 16), (65, 384, 100), (700, 7168, 256),
+                                   (4096, 2048, 128), (130, 9216, 37)])
+def test_router_logits_kernel(pkg, dev, T, H, E):
+    say("router logits", T, H, E)
+    g = torch.Generator().manual_seed(T + H + E)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    wr = (torch.randn(E, H, generator=g) * 0.05).to(torch.bfloat16)
+    got = pkg.router_logits(x.to(dev), wr.to(dev))
+    again = pkg.router_logits(x.to(dev), wr.to(dev))
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), again.view(torch.int16))           # fixed summation order
+    exact = x.double() @ wr.double().t()
+    err = (got.double().cpu() - exact).abs()
+    bound = exact.abs() * 2.0 ** -8 + 1e-4 * x.double().norm(dim=1, keepdim=True) * wr.double().norm(dim=1)[None]
+    assert bool((err <= bound).all()), float((err - bound).max())
 
 
 def test_decode_layer_in_a_hip_graph(pkg, oracle, dev):
@@ -183,26 +205,25 @@ def test_decode_layer_in_a_hip_graph(pkg, oracle, dev):
             assert torch.equal(moe(x).view(torch.int16), ref.view(torch.int16))     # eager work between replays
 
 
-def test_decode_layer_rejects_what_it_does_not_cover(pkg, oracle, dev):
-    say("decode layer errors")
+def test_layer_entry_point_rejects_what_it_does_not_cover(pkg, oracle, dev):
+    say("layer entry errors")
     H, I = 256, 128
     g = torch.Generator().manual_seed(1)
-
-    def call(T, E, K):
-        ld = tuple(t.to(dev) for t in oracle.make_layer(E, H, I, seed=1))
-        wr = (torch.randn(E, H, generator=g) * 0.05).to(torch.bfloat16).to(dev)
-        x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
-        return pkg.decode_layer_fp8(x, wr, *ld, K, "softmax")
-
-    with pytest.raises(RuntimeError):
-        call(33, 16, 8)             # 264 slots
-    assert not pkg.decode_layer_eligible(33, 16, 8) and pkg.decode_layer_eligible(32, 16, 8)
-    assert not pkg.decode_layer_eligible(1, 257, 8)
+    assert pkg.layer_eligible(33, 16, 8) and pkg.layer_eligible(4096, 256, 8)
+    assert not pkg.layer_eligible(1, 257, 8) and not pkg.layer_eligible(1, 4, 8)
     lib = pkg._lib.lib
-    assert lib.moe_decode_layer_fp8(None, 1, 33, H, 1, None, 16, 8, 0, 1, 1, 1, 1.0, 1, 1, 1, 1, I, None, None, None, None,
-                                    0, 1, None, None, None, 256, 1 << 30) == -2
-    assert lib.moe_decode_layer_fp8(None, 1, 1, H, 1, None, 300, 8, 0, 1, 1, 1, 1.0, 1, 1, 1, 1, I, None, None, None, None,
-                                    0, 1, None, None, None, 256, 1 << 30) == -2
-    out = call(2, 16, 8)
+    # more than 256 experts: refused on the shape alone, before anything is launched (the pointers are never used)
+    assert lib.moe_layer_fp8(None, 1, 1, H, 1, None, 300, 8, 0, 1, 1, 1, 1.0, 1, 1, 1, 1, I, None, None, None, None,
+                             0, 1, None, None, None, 256, 1 << 30) == -2
+    assert lib.moe_layer_fp8_workspace_bytes(1, H, I, 300, 8, 0) == 0
+    E, K = 16, 8
+    ld = tuple(t.to(dev) for t in oracle.make_layer(E, H, I, seed=1))
+    wr = (torch.randn(E, H, generator=g) * 0.05).to(torch.bfloat16).to(dev)
+    x = torch.randn(2, H, generator=g).to(torch.bfloat16).to(dev)
+    with pytest.raises(RuntimeError):
+        pkg.layer_fp8(x, wr, *ld, K, "scores")                       # not a routing mode of this entry point
+    with pytest.raises(RuntimeError):
+        pkg.layer_fp8(x, wr, *ld, K, "softmax", workspace=torch.empty(256, dtype=torch.uint8, device=dev))
+    out = pkg.layer_fp8(x, wr, *ld, K, "softmax")
     torch.cuda.synchronize()
     assert torch.isfinite(out.float()).all()

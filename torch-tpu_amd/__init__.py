@@ -8,11 +8,11 @@ from . import _lib                      # noqa: F401  (raises if the library is 
 from . import my_ops as _my_ops         # noqa: F401  (registers torch.ops.my_ops.*)
 from .my_ops import set_expert_numerics
 from .layer import FusedMoE, convert_hf_moe_layer, pack_expert_weights, quant_weight_block128
-from .ops import (MoeHipError, act_quant, decode_layer_eligible, decode_layer_fp8, decode_layer_workspace_bytes,
+from .ops import (MoeHipError, act_quant, layer_eligible, layer_fp8, layer_workspace_bytes,
                   fused_experts_bf16, fused_experts_fp8, fused_experts_workspace_bytes, gemm1_swiglu, gemm2, mlp_fp8, mm_fp8,
-                  moe_permute, moe_route, noaux_tc_topk, scale_pitch, tile_rows, weighted_reduce)
+                  moe_permute, moe_route, noaux_tc_topk, router_logits, scale_pitch, tile_rows, weighted_reduce)
 
 __all__ = ["FusedMoE", "set_expert_numerics", "convert_hf_moe_layer", "pack_expert_weights", "quant_weight_block128", "MoeHipError", "act_quant",
-           "decode_layer_eligible", "decode_layer_fp8", "decode_layer_workspace_bytes", "fused_experts_bf16", "fused_experts_fp8",
-           "fused_experts_workspace_bytes", "gemm1_swiglu", "gemm2", "mlp_fp8", "mm_fp8", "moe_permute", "moe_route", "noaux_tc_topk",
+           "layer_eligible", "layer_fp8", "layer_workspace_bytes", "fused_experts_bf16", "fused_experts_fp8",
+           "fused_experts_workspace_bytes", "gemm1_swiglu", "gemm2", "mlp_fp8", "mm_fp8", "moe_permute", "moe_route", "noaux_tc_topk", "router_logits",
            "scale_pitch", "tile_rows", "weighted_reduce"]

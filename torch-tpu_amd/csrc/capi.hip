@@ -21,6 +21,13 @@ int decode_prep_launch(hipStream_t st, const uint16_t *x, int T, int H, const ui
                        int32_t *ids, int *arrivals, uint8_t *xq, float *xs, int tile_m, int32_t *sorted_slot,
                        int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &pw);
 
+size_t router_front_partial_bytes(int T, int H, int E);
+int router_front_launch(hipStream_t st, const void *x, int T, int H, const void *wr, int E, float *partial, int *n_slices_out);
+int sum_slices_launch(hipStream_t st, const float *partial, int n_slices, int T, int E, uint16_t *logits);
+int route_from_partials_launch(hipStream_t st, const float *partial, int n_slices, const float *bias, int T, int E, int K,
+                               int mode, int n_groups, int topk_groups, int renorm, float scale, float *weights_out,
+                               int32_t *ids_out);
+
 size_t dense_small_partial_bytes(int M, int K, int N, bool keep_partial);
 int dense_small_launch(hipStream_t st, const uint8_t *xq, const float *xs, int M, int K, const uint8_t *w, const float *ws,
                        int N, uint16_t *out, float *partial, int *n_splits_out);
@@ -98,18 +105,22 @@ static int run_experts(void *stream, const FusedWs &w, const PermuteWs &pw, int 
   return moe_weighted_reduce(stream, y, routing_weights, has_shared ? w.sh_y : nullptr, T, K, H, out_bf16);
 }
 
-// moe_decode_layer_fp8: the fused-experts workspace followed by the router's own pieces
-struct DecodeWs {
+// moe_layer_fp8: the fused-experts workspace followed by the router's own pieces
+struct LayerWs {
   FusedWs fused;
   uint16_t *logits;
   float *weights;
   int32_t *ids;
   int *arrivals;
+  float *partial;      // batches beyond the decode size: partial sums of the router product
   size_t bytes;
 };
 
-static DecodeWs decode_layout(void *base, int T, int H, int I, int E, int K, int I_sh) {
-  DecodeWs d{};
+// up to this many slots (T * K) one workgroup can permute, and the two-launch decode front end applies
+static bool decode_size(int T, int K) { return (long)T * K <= kChunk; }
+
+static LayerWs layer_layout(void *base, int T, int H, int I, int E, int K, int I_sh) {
+  LayerWs d{};
   d.fused = fused_layout(base, T, H, I, E, K, I_sh);
   size_t off = d.fused.bytes;
   auto take = [&](size_t n) {
@@ -121,6 +132,7 @@ static DecodeWs decode_layout(void *base, int T, int H, int I, int E, int K, int
   d.weights = (float *)take((size_t)T * K * 4);
   d.ids = (int32_t *)take((size_t)T * K * 4);
   d.arrivals = (int *)take(4);
+  if (!decode_size(T, K)) d.partial = (float *)take(router_front_partial_bytes(T, H, E));
   d.bytes = off;
   return d;
 }
@@ -187,23 +199,24 @@ extern "C" int moe_fused_experts_fp8(void *stream, const void *x_bf16, int T, in
                      shared_w13_scale, shared_w2, shared_w2_scale, I_sh, out_bf16, out_mode);
 }
 
-extern "C" size_t moe_decode_layer_fp8_workspace_bytes(int T, int H, int I, int E, int K, int I_shared) {
-  if (T < 0 || H < 1 || I < 1 || E < 1 || K < 1 || I_shared < 0) return 0;
-  return moe::decode_layout(nullptr, T, H, I, E, K, I_shared).bytes;
+extern "C" size_t moe_layer_fp8_workspace_bytes(int T, int H, int I, int E, int K, int I_shared) {
+  if (T < 0 || H < 1 || I < 1 || E < 1 || E > 256 || K < 1 || I_shared < 0 || H % moe::kBlock) return 0;
+  return moe::layer_layout(nullptr, T, H, I, E, K, I_shared).bytes;
 }
 
-extern "C" int moe_decode_layer_fp8(void *stream, const void *x_bf16, int T, int H, const void *router_w_bf16,
-                                    const float *router_bias, int E, int K, int mode, int n_groups, int topk_groups,
-                                    int renorm, float scale, const uint8_t *w13, const float *w13_scale,
-                                    const uint8_t *w2, const float *w2_scale, int I, const uint8_t *shared_w13,
-                                    const float *shared_w13_scale, const uint8_t *shared_w2,
-                                    const float *shared_w2_scale, int I_shared, void *out_bf16, void *logits_out_bf16,
-                                    float *weights_out, int32_t *ids_out, void *workspace, size_t workspace_bytes) {
+extern "C" int moe_layer_fp8(void *stream, const void *x_bf16, int T, int H, const void *router_w_bf16,
+                             const float *router_bias, int E, int K, int mode, int n_groups, int topk_groups,
+                             int renorm, float scale, const uint8_t *w13, const float *w13_scale, const uint8_t *w2,
+                             const float *w2_scale, int I, const uint8_t *shared_w13, const float *shared_w13_scale,
+                             const uint8_t *shared_w2, const float *shared_w2_scale, int I_shared, void *out_bf16,
+                             void *logits_out_bf16, float *weights_out, int32_t *ids_out, void *workspace,
+                             size_t workspace_bytes) {
   using namespace moe;
   if (!router_w_bf16 || !w13 || !w13_scale || !w2 || !w2_scale || !workspace) return MOE_E_NULL;
   if (T != 0 && (!x_bf16 || !out_bf16)) return MOE_E_NULL;
   if (T < 0 || H < 1 || I < 1 || E < 1 || E > 256 || K < 1 || K > MOE_MAX_TOPK || K > E) return MOE_E_SHAPE;
-  if ((long)T * K > kChunk) return MOE_E_SHAPE;
+  if ((long)T * K > (1l << 30)) return MOE_E_SHAPE;
+  if (mode != MOE_ROUTE_SOFTMAX && mode != MOE_ROUTE_SIGMOID) return MOE_E_MODE;
   if (H % kBlock || I % kBlock) return MOE_E_ALIGN;
   const bool has_shared = shared_w13 != nullptr;
   if (has_shared) {
@@ -215,20 +228,63 @@ extern "C" int moe_decode_layer_fp8(void *stream, const void *x_bf16, int T, int
   if (((uintptr_t)workspace % 256) || ((uintptr_t)x_bf16 % 16) || ((uintptr_t)out_bf16 % 16) ||
       ((uintptr_t)router_w_bf16 % 16) || ((uintptr_t)w13 % 16) || ((uintptr_t)w2 % 16))
     return MOE_E_ALIGN;
-  DecodeWs d = decode_layout(workspace, T, H, I, E, K, I_sh);
+  LayerWs d = layer_layout(workspace, T, H, I, E, K, I_sh);
   if (workspace_bytes < d.bytes) return MOE_E_WORKSPACE;
   if (T == 0) return MOE_OK;
+  hipStream_t st = (hipStream_t)stream;
   const FusedWs &w = d.fused;
   PermuteWs pw = permute_ws_layout(w.permute, T, K, E);
   float *weights = weights_out ? weights_out : d.weights;
-  int rc = decode_prep_launch((hipStream_t)stream, (const uint16_t *)x_bf16, T, H, (const uint16_t *)router_w_bf16,
-                              router_bias, E, K, mode, n_groups, topk_groups, renorm, scale,
-                              logits_out_bf16 ? (uint16_t *)logits_out_bf16 : d.logits, weights,
-                              ids_out ? ids_out : d.ids, d.arrivals, w.xq, w.xs, choose_tile_m(T, K, E), w.sorted_slot,
-                              w.expert_offsets, w.slot_to_row, pw);
-  if (rc) return rc;
+  int32_t *ids = ids_out ? ids_out : d.ids;
+  int rc;
+  if (decode_size(T, K)) {
+    // two launches: router logits + activation quantisation, then routing + permutation
+    rc = decode_prep_launch(st, (const uint16_t *)x_bf16, T, H, (const uint16_t *)router_w_bf16, router_bias, E, K, mode,
+                            n_groups, topk_groups, renorm, scale, logits_out_bf16 ? (uint16_t *)logits_out_bf16 : d.logits,
+                            weights, ids, d.arrivals, w.xq, w.xs, choose_tile_m(T, K, E), w.sorted_slot, w.expert_offsets,
+                            w.slot_to_row, pw);
+    if (rc) return rc;
+  } else {
+    // the router product on the matrix cores, its reduction cut into slices; the routing kernel adds the slices
+    int n_slices = 0;
+    rc = router_front_launch(st, x_bf16, T, H, router_w_bf16, E, d.partial, &n_slices);
+    if (rc) return rc;
+    if (logits_out_bf16) {
+      rc = sum_slices_launch(st, d.partial, n_slices, T, E, (uint16_t *)logits_out_bf16);
+      if (rc) return rc;
+    }
+    rc = route_from_partials_launch(st, d.partial, n_slices, router_bias, T, E, K, mode, n_groups, topk_groups, renorm,
+                                    scale, weights, ids);
+    if (rc) return rc;
+    rc = permute_launch(st, ids, T, K, E, choose_tile_m(T, K, E), w.sorted_slot, w.expert_offsets, w.slot_to_row, pw);
+    if (rc) return rc;
+    rc = moe_act_quant(stream, x_bf16, T, H, w.xq, w.xs);
+    if (rc) return rc;
+  }
   return run_experts(stream, w, pw, T, H, w13, w13_scale, w2, w2_scale, I, E, K, weights, shared_w13, shared_w13_scale,
                      shared_w2, shared_w2_scale, I_sh, out_bf16, 1);
+}
+
+// The router product on its own: logits [T, E] bf16 = x [T, H] . Wr [E, H]^T (fp32 sums, rounded once).
+extern "C" size_t moe_router_logits_workspace_bytes(int T, int H, int E) {
+  if (T < 0 || H < 1 || E < 1 || E > 256 || H % moe::kBlock) return 0;
+  return moe::align_up(moe::router_front_partial_bytes(T, H, E) + 1, 256);
+}
+
+extern "C" int moe_router_logits(void *stream, const void *x_bf16, int T, int H, const void *router_w_bf16, int E,
+                                 void *logits_bf16, void *workspace, size_t workspace_bytes) {
+  using namespace moe;
+  if (!router_w_bf16 || !workspace) return MOE_E_NULL;
+  if (T != 0 && (!x_bf16 || !logits_bf16)) return MOE_E_NULL;
+  if (T < 0 || H < 1 || E < 1 || E > 256) return MOE_E_SHAPE;
+  if (H % kBlock) return MOE_E_ALIGN;
+  if (((uintptr_t)workspace % 256) || ((uintptr_t)x_bf16 % 16) || ((uintptr_t)router_w_bf16 % 16)) return MOE_E_ALIGN;
+  if (workspace_bytes < moe_router_logits_workspace_bytes(T, H, E)) return MOE_E_WORKSPACE;
+  if (T == 0) return MOE_OK;
+  int n_slices = 0;
+  int rc = router_front_launch((hipStream_t)stream, x_bf16, T, H, router_w_bf16, E, (float *)workspace, &n_slices);
+  if (rc) return rc;
+  return sum_slices_launch((hipStream_t)stream, (const float *)workspace, n_slices, T, E, (uint16_t *)logits_bf16);
 }
 
 // ---- dense block-scaled FP8 linear layers: the grouped kernels with one "expert" that owns every row ----

@@ -65,6 +65,18 @@ __device__ __forceinline__ Best half_argmax(Best b, int lane) {
 
 __device__ __forceinline__ float round_to_bf16(float f) { return bf16_to_f32(f32_to_bf16(f)); }
 
+// p[0] + p[stride] + ... (n terms, n <= 8) added in that order; all terms are asked for before the first is used
+__device__ __forceinline__ float sum_slices_in_order(const float *__restrict__ p, size_t stride, int n) {
+  float v[8];
+#pragma unroll
+  for (int k = 0; k < 8; k++) v[k] = k < n ? p[(size_t)k * stride] : 0.f;
+  float acc = v[0];
+#pragma unroll
+  for (int k = 1; k < 8; k++)
+    if (k < n) acc += v[k];
+  return acc;
+}
+
 // Select top_k of one row.  v[j] holds element lane + 64*j (only j < per_lane are used,
 // elements >= E must be pre-marked dead).  dead bit j set = element is not a candidate.
 // Group limiting (n_groups > 1): group score = top1 + top2 of the group (fp32 add, rounded to
@@ -184,7 +196,7 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const void *__restrict_
                                                           const float *__restrict__ bias, int T, int E, int K, int mode,
                                                           int n_groups, int topk_groups, int renorm, float scale,
                                                           float *__restrict__ weights_out, int32_t *__restrict__ ids_out,
-                                                          float *__restrict__ scores_out) {
+                                                          float *__restrict__ scores_out, int n_slices = 0) {
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (t >= T) return;
@@ -196,7 +208,11 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const void *__restrict_
     int e = lane + 64 * j;
     float x = -INFINITY;
     if (e < E) {
-      if (logits_bf16) x = bf16_to_f32(((const uint16_t *)logits)[(size_t)t * E + e]);
+      if (n_slices > 0) {
+        // the logits arrive as fp32 partial sums over slices of the reduction [n_slices][T][E]: added in slice
+        // order and rounded to bf16, which is what a bf16 matrix product would have left
+        x = round_to_bf16(sum_slices_in_order((const float *)logits + (size_t)t * E + e, (size_t)T * E, n_slices));
+      } else if (logits_bf16) x = bf16_to_f32(((const uint16_t *)logits)[(size_t)t * E + e]);
       else x = ((const float *)logits)[(size_t)t * E + e];
     }
     if (mode == MOE_ROUTE_SIGMOID && e < E) x = 1.0f / (1.0f + expf(-x));
@@ -285,6 +301,38 @@ int check_route_shape(int T, int E, int K, int n_groups, int topk_groups) {
     if ((long)topk_groups * (E / n_groups) < K) return MOE_E_SHAPE;
   }
   return MOE_OK;
+}
+
+// partial sums [n_slices][T][E] -> bf16 logits [T][E], slices added in order (the same sum the routing kernel forms)
+__global__ __launch_bounds__(256) void sum_slices_kernel(const float *__restrict__ partial, int n_slices, size_t n,
+                                                         uint16_t *__restrict__ logits) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  logits[i] = f32_to_bf16(sum_slices_in_order(partial + i, n, n_slices));
+}
+
+int sum_slices_launch(hipStream_t st, const float *partial, int n_slices, int T, int E, uint16_t *logits) {
+  const size_t n = (size_t)T * E;
+  sum_slices_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(partial, n_slices, n, logits);
+  return (int)hipGetLastError();
+}
+
+// routing straight from the partial sums of the router product (E <= 256: four scores per lane)
+int route_from_partials_launch(hipStream_t st, const float *partial, int n_slices, const float *bias, int T, int E, int K,
+                               int mode, int n_groups, int topk_groups, int renorm, float scale, float *weights_out,
+                               int32_t *ids_out) {
+  if (E > 256 || n_slices < 1) return MOE_E_SHAPE;
+  if (mode != MOE_ROUTE_SOFTMAX && mode != MOE_ROUTE_SIGMOID) return MOE_E_MODE;
+  const int rc = check_route_shape(T, E, K, n_groups, topk_groups);
+  if (rc) return rc;
+  dim3 grid((T + 3) / 4), block(256);
+  if (E <= 64)
+    route_topk_kernel<1><<<grid, block, 0, st>>>(partial, 0, bias, T, E, K, mode, n_groups, topk_groups, renorm, scale, weights_out, ids_out, nullptr, n_slices);
+  else if (E <= 128)
+    route_topk_kernel<2><<<grid, block, 0, st>>>(partial, 0, bias, T, E, K, mode, n_groups, topk_groups, renorm, scale, weights_out, ids_out, nullptr, n_slices);
+  else
+    route_topk_kernel<4><<<grid, block, 0, st>>>(partial, 0, bias, T, E, K, mode, n_groups, topk_groups, renorm, scale, weights_out, ids_out, nullptr, n_slices);
+  return (int)hipGetLastError();
 }
 
 }  // namespace moe

@@ -1,0 +1,156 @@
+// Router logits for batches beyond the decode size: logits[T, E] = x[T, H] . Wr[E, H]^T in bf16 on the matrix
+// cores, E <= 256.
+//
+// The product is short and wide (a few thousand tokens by at most 256 experts over a long reduction), so the
+// reduction is cut into slices: workgroup (block of 128 tokens, slice) leaves its fp32 partial sums, and the routing
+// kernel that follows adds the slices in a fixed order, rounds to bf16 (what a bf16 matmul leaves) and routes.
+// Four wavefronts; wavefront w owns experts 64w .. 64w+63 for all 128 tokens (8 x 4 tiles of 16 x 16: with fewer
+// tokens per workgroup the router rows, re-read by every token block, saturate the L2 -> LDS path before the matrix
+// pipe).  A step is 64 reduction elements = 128 bytes of a row = two v_mfma_f32_16x16x32_bf16 per tile pair.  Both
+// operands travel L2 -> LDS with direct loads, two steps ahead, through three stages: the token tile (shared, one
+// barrier per step) and each wavefront's own 64 router rows (loaded and read by the same wavefront).
+#include "moe_common.h"
+#include "moe_layout.h"
+#include "../../include/moe_hip.h"
+
+namespace moe {
+
+typedef __bf16 v8bf_t __attribute__((ext_vector_type(8)));
+
+constexpr int kRfTokens = 128;                // tokens per workgroup
+constexpr int kRfMT = kRfTokens / 16;
+constexpr int kRfXStages = 3, kRfWStages = 3;
+
+struct RfSmem {
+  alignas(1024) uint8_t x[kRfXStages][kRfTokens * 128];   // [row][16-byte chunk, XOR-swizzled by row % 8]
+  alignas(1024) uint8_t w[kRfWStages][256 * 128];
+};
+
+typedef __attribute__((address_space(3))) uint8_t rf_lds_byte;
+__device__ __forceinline__ uint32_t rf_lds_offset(const void *p) { return (uint32_t)(uintptr_t)(rf_lds_byte *)p; }
+
+__global__ __launch_bounds__(256) void router_logits_splitk_kernel(const uint8_t *__restrict__ x,
+                                                                   const uint8_t *__restrict__ wr, int T, int H, int E,
+                                                                   int n_slices, int blocks_per_slice,
+                                                                   float *__restrict__ partial) {
+  __shared__ RfSmem sm;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int li = lane & 15, lg = lane >> 4;
+  const int slice = blockIdx.x % n_slices, m0 = (blockIdx.x / n_slices) * kRfTokens;
+  const int nblk = H >> 7;
+  const int b0 = slice * blocks_per_slice, b1 = min(nblk, b0 + blocks_per_slice);
+  const int n_steps = 2 * (b1 - b0);                      // steps of 64 elements
+  if (n_steps <= 0) return;
+  const size_t row_bytes = (size_t)H * 2;
+  const uint8_t *const xbase = x + (size_t)b0 * 256;      // first byte of the slice in a row
+  const uint8_t *const wbase = wr + (size_t)b0 * 256;
+
+  // direct-to-LDS loads: one instruction moves 8 rows x 128 bytes; lane l fetches row l/8 and the chunk that
+  // belongs at position l%8 of the swizzled row
+  const int sub = lane >> 3, chunk = (lane & 7) ^ sub;
+  constexpr int NX = kRfTokens / 32;              // token-tile instructions per wavefront and step
+  uint32_t x_src[NX], w_src[8];
+#pragma unroll
+  for (int u = 0; u < NX; u++) x_src[u] = (uint32_t)min(m0 + 8 * (NX * wave + u) + sub, T - 1) * (uint32_t)row_bytes + chunk * 16;
+#pragma unroll
+  for (int u = 0; u < 8; u++) w_src[u] = (uint32_t)min(64 * wave + 8 * u + sub, E - 1) * (uint32_t)row_bytes + chunk * 16;
+  const uint32_t x_lds = __builtin_amdgcn_readfirstlane(rf_lds_offset(&sm.x[0][0])) + (NX * wave) * 1024;
+  const uint32_t w_lds = __builtin_amdgcn_readfirstlane(rf_lds_offset(&sm.w[0][0])) + (8 * wave) * 1024;
+  auto request = [&](int step) {
+    const uint8_t *xb = xbase + (size_t)step * 128, *wb = wbase + (size_t)step * 128;
+    const uint32_t xm = x_lds + (step % kRfXStages) * (kRfTokens * 128), wm = w_lds + (step % kRfWStages) * (256 * 128);
+#pragma unroll
+    for (int u = 0; u < NX; u++)
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(xm + u * 1024), "v"(x_src[u]), "s"(xb) : "memory", "m0");
+#pragma unroll
+    for (int u = 0; u < 8; u++)
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(wm + u * 1024), "v"(w_src[u]), "s"(wb) : "memory", "m0");
+  };
+  constexpr int kLoadsPerStep = NX + 8;
+
+  v4f acc[kRfMT][4];
+#pragma unroll
+  for (int i = 0; i < kRfMT; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+  const int last = n_steps - 1;
+  request(0);
+  request(min(1, last));
+  const int o0 = (lg ^ (li & 7)) << 4, o1 = ((lg + 4) ^ (li & 7)) << 4;
+  for (int t = 0; t < n_steps; t++) {
+    // step t has landed (step t + 1 may still be in flight); everybody has left step t - 1, whose token stage the
+    // request below overwrites
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoadsPerStep) : "memory");
+    __syncthreads();
+    request(min(t + 2, last));          // past the end: the last step again, so that the count in flight stays the same
+    const uint8_t *xs = sm.x[t % kRfXStages] + li * 128;
+    const uint8_t *ws = sm.w[t % kRfWStages] + (64 * wave + li) * 128;
+    v4i xa[kRfMT][2], wb[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      wb[i][0] = *(const v4i *)(ws + i * 2048 + o0);
+      wb[i][1] = *(const v4i *)(ws + i * 2048 + o1);
+    }
+#pragma unroll
+    for (int i = 0; i < kRfMT; i++) {
+      xa[i][0] = *(const v4i *)(xs + i * 2048 + o0);
+      xa[i][1] = *(const v4i *)(xs + i * 2048 + o1);
+    }
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+      for (int i = 0; i < kRfMT; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf_t, xa[i][h]),
+                                                              __builtin_bit_cast(v8bf_t, wb[j][h]), acc[i][j], 0, 0, 0);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // c[r] of tile (i, j): token m0 + 16 i + 4 (l / 16) + r, expert 64 w + 16 j + l % 16
+  float *const out = partial + (size_t)slice * T * E;
+#pragma unroll
+  for (int i = 0; i < kRfMT; i++)
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int tok = m0 + 16 * i + 4 * lg + r;
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const int e = 64 * wave + 16 * j + li;
+        if (tok < T && e < E) out[(size_t)tok * E + e] = acc[i][j][r];
+      }
+    }
+}
+
+// how the reduction is cut: enough workgroups for every compute unit, slices of whole 128-column blocks
+void router_front_plan(int T, int H, int *n_slices, int *blocks_per_slice) {
+  const int mblocks = (T + kRfTokens - 1) / kRfTokens, nblk = H / kBlock;
+  int s = (512 + mblocks - 1) / mblocks;
+  if (s < 1) s = 1;
+  if (s > 8) s = 8;
+  if (s > nblk) s = nblk;
+  const int per = (nblk + s - 1) / s;
+  *blocks_per_slice = per;
+  *n_slices = (nblk + per - 1) / per;
+}
+
+size_t router_front_partial_bytes(int T, int H, int E) {
+  int s, per;
+  if (T < 1) return 0;
+  router_front_plan(T, H, &s, &per);
+  return (size_t)s * T * E * 4;
+}
+
+// x [T, H] bf16, wr [E, H] bf16 -> partial [n_slices][T][E] fp32.  The caller has checked pointers and alignment.
+int router_front_launch(hipStream_t st, const void *x, int T, int H, const void *wr, int E, float *partial, int *n_slices_out) {
+  if (T < 1 || E < 1 || E > 256 || H % kBlock) return MOE_E_SHAPE;
+  if ((double)T * H * 2 >= 2147483648.0) return MOE_E_SHAPE;       // per-lane source offsets are 32-bit
+  int s, per;
+  router_front_plan(T, H, &s, &per);
+  const long blocks = (long)((T + kRfTokens - 1) / kRfTokens) * s;
+  router_logits_splitk_kernel<<<(unsigned)blocks, 256, 0, st>>>((const uint8_t *)x, (const uint8_t *)wr, T, H, E, s, per, partial);
+  *n_slices_out = s;
+  return (int)hipGetLastError();
+}
+
+}  // namespace moe

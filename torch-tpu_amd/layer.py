@@ -96,7 +96,7 @@ class FusedMoE:
     def _workspace(self, T, decode=False):
         E, I2, H = self.w13.shape
         I_sh = self.shared[0].shape[1] // 2 if self.shared is not None else 0
-        size = ops.decode_layer_workspace_bytes if decode else ops.fused_experts_workspace_bytes
+        size = ops.layer_workspace_bytes if decode else ops.fused_experts_workspace_bytes
         need = size(T, H, I2 // 2, E, self.top_k, I_sh)
         if self._ws is None or self._ws.numel() < need:
             self._ws = torch.empty(need, dtype=torch.uint8, device=self.w13.device)
@@ -116,14 +116,14 @@ class FusedMoE:
 
     def _one_call(self, T):
         # a softmax router's bias belongs to the logits, which the one-call entry point computes itself
-        return (ops.decode_layer_eligible(T, self.w13.shape[0], self.top_k)
+        return (ops.layer_eligible(T, self.w13.shape[0], self.top_k)
                 and not (self.mode == "softmax" and self.bias is not None)
                 and self.router_weight.dtype == torch.bfloat16)
 
     def __call__(self, x, out=None):
         T = x.shape[0]
-        if self._one_call(T):      # decode-size batch: router and experts behind one entry point
-            return ops.decode_layer_fp8(x, self.router_weight, self.w13, self.w13_scale, self.w2, self.w2_scale,
+        if self._one_call(T):      # router and experts behind one entry point
+            return ops.layer_fp8(x, self.router_weight, self.w13, self.w13_scale, self.w2, self.w2_scale,
                                         self.top_k, self.mode, self.bias, self.n_groups, self.topk_groups, self.renorm,
                                         self.scale, shared=self.shared, out=out, workspace=self._workspace(T, True))
         weights, ids = self.route(x)

@@ -210,19 +210,39 @@ def fused_experts_fp8(x, w13, w13_scale, w2, w2_scale, ids, routing_weights=None
     return out
 
 
-def decode_layer_eligible(T: int, E: int, K: int) -> bool:
-    """Shapes the one-call decode entry point takes (decode_layer_fp8)."""
-    return 1 <= T and T * K <= 256 and E <= 256
+def layer_eligible(T: int, E: int, K: int) -> bool:
+    """Shapes the one-call entry point takes (layer_fp8): any batch, up to 256 experts."""
+    return T >= 0 and 1 <= K <= E <= 256
 
 
-def decode_layer_workspace_bytes(T, H, I, E, K, I_shared=0) -> int:
-    return lib.moe_decode_layer_fp8_workspace_bytes(T, H, I, E, K, I_shared)
+def router_logits(x, router_weight, out=None, workspace=None):
+    """logits [T,E] bf16 = x [T,H] bf16 . router_weight [E,H]^T bf16 (fp32 sums, rounded once), E <= 256."""
+    _need(x.dim() == 2 and router_weight.dim() == 2 and x.shape[1] == router_weight.shape[1], "x must be [T,H], router_weight [E,H]")
+    T, H = x.shape
+    E = router_weight.shape[0]
+    _need(E <= 256 and H % 128 == 0, "router_logits takes E <= 256 and H a multiple of 128")
+    if out is None:
+        out = torch.empty(T, E, dtype=torch.bfloat16, device=x.device)
+    _need(tuple(out.shape) == (T, E), "out must be [T, E]")
+    need = lib.moe_router_logits_workspace_bytes(T, H, E)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+    _need(workspace.numel() * workspace.element_size() >= need, "workspace too small")
+    rc = lib.moe_router_logits(_stream(), _dev(x, "x", torch.bfloat16), T, H, _dev(router_weight, "router_weight", torch.bfloat16),
+                               E, _dev(out, "out", torch.bfloat16), _dev(workspace, "workspace"),
+                               workspace.numel() * workspace.element_size())
+    check(rc, "router_logits")
+    return out
 
 
-def decode_layer_fp8(x, router_weight, w13, w13_scale, w2, w2_scale, top_k: int, mode: str = "softmax", bias=None,
+def layer_workspace_bytes(T, H, I, E, K, I_shared=0) -> int:
+    return lib.moe_layer_fp8_workspace_bytes(T, H, I, E, K, I_shared)
+
+
+def layer_fp8(x, router_weight, w13, w13_scale, w2, w2_scale, top_k: int, mode: str = "softmax", bias=None,
                      n_groups: int = 1, topk_groups: int = 1, renorm: bool = True, scale: float = 1.0, shared=None,
                      out=None, workspace=None, return_routing: bool = False):
-    """Router and experts of one layer in one call, for decode-size batches (T*top_k <= 256, E <= 256).
+    """Router and experts of one layer in one call (E <= 256).
 
     x [T,H] bf16, router_weight [E,H] bf16, the expert weights as in fused_experts_fp8.  Returns out [T,H] bf16,
     or (out, logits bf16 [T,E], weights fp32 [T,k], ids int32 [T,k]) with return_routing."""
@@ -232,7 +252,7 @@ def decode_layer_fp8(x, router_weight, w13, w13_scale, w2, w2_scale, top_k: int,
     T, H = x.shape
     E, I2, H2 = w13.shape
     I = I2 // 2
-    _need(decode_layer_eligible(T, E, top_k), "decode_layer_fp8 takes T*top_k <= 256 and E <= 256")
+    _need(layer_eligible(T, E, top_k), "layer_fp8 takes E <= 256 and top_k <= E")
     _need(H2 == H and tuple(w2.shape) == (E, H, I) and tuple(router_weight.shape) == (E, H), "weight shapes do not match x")
     _need(H % 128 == 0 and I % 128 == 0, "H and I must be multiples of 128")
     _need(tuple(w13_scale.shape) == (E, I2 // 128, H // 128), "w13_scale must be [E, 2I/128, H/128]")
@@ -245,7 +265,7 @@ def decode_layer_fp8(x, router_weight, w13, w13_scale, w2, w2_scale, top_k: int,
         _need(bias.numel() == E, "bias must hold one value per expert")
         bias_ptr = _dev(bias, "bias", torch.float32)
     sh, I_sh = _shared_args(shared, H)
-    need = decode_layer_workspace_bytes(T, H, I, E, top_k, I_sh)
+    need = layer_workspace_bytes(T, H, I, E, top_k, I_sh)
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
     _need(workspace.numel() * workspace.element_size() >= need, "workspace too small")
@@ -254,7 +274,7 @@ def decode_layer_fp8(x, router_weight, w13, w13_scale, w2, w2_scale, top_k: int,
         logits = torch.empty(T, E, dtype=torch.bfloat16, device=x.device)
         weights = torch.empty(T, top_k, dtype=torch.float32, device=x.device)
         ids = torch.empty(T, top_k, dtype=torch.int32, device=x.device)
-    rc = lib.moe_decode_layer_fp8(
+    rc = lib.moe_layer_fp8(
         _stream(), _dev(x, "x", torch.bfloat16), T, H, _dev(router_weight, "router_weight", torch.bfloat16), bias_ptr,
         E, top_k, modes[mode], n_groups, topk_groups, int(renorm), float(scale),
         _dev(w13, "w13", _FP8), _dev(w13_scale, "w13_scale", torch.float32),
@@ -263,7 +283,7 @@ def decode_layer_fp8(x, router_weight, w13, w13_scale, w2, w2_scale, top_k: int,
         logits.data_ptr() if return_routing else None, weights.data_ptr() if return_routing else None,
         ids.data_ptr() if return_routing else None,
         _dev(workspace, "workspace"), workspace.numel() * workspace.element_size())
-    check(rc, "decode_layer_fp8")
+    check(rc, "layer_fp8")
     return (out, logits, weights, ids) if return_routing else out
 
 
