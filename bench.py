@@ -282,7 +282,14 @@ def cpu_baseline(pkg, moe, cfg, x, sample_tokens):
     torch.set_num_threads(threads)
     n = sample_tokens
     # device side of the comparison: scores the device routed on, its picks and its output
-    logits_dev = torch.matmul(x[:n], moe.router_weight.t()).float()
+    one_call = moe._one_call(n)
+    if one_call:
+        # the entry point the timed step goes through, asked for what its router produced
+        out_dev, logits_dev, w_one, ids_one = pkg.layer_fp8(
+            x[:n].contiguous(), moe.router_weight, moe.w13, moe.w13_scale, moe.w2, moe.w2_scale, cfg["K"], cfg["route"],
+            moe.bias, cfg["n_groups"], cfg["topk_groups"], True, cfg["scale"], shared=moe.shared, return_routing=True)
+    else:
+        logits_dev = torch.matmul(x[:n], moe.router_weight.t()).float()
     if cfg["route"] == "sigmoid":
         w_dev, ids_dev, scores_dev = pkg.moe_route(logits_dev, cfg["K"], "sigmoid", moe.bias, cfg["n_groups"],
                                                    cfg["topk_groups"], True, cfg["scale"], return_scores=True)
@@ -290,7 +297,10 @@ def cpu_baseline(pkg, moe, cfg, x, sample_tokens):
         lg = logits_dev if moe.bias is None else logits_dev + moe.bias
         w_dev, ids_dev = pkg.moe_route(lg, cfg["K"], "softmax")
         scores_dev = lg
-    out_dev = moe.experts(x[:n].contiguous(), w_dev, ids_dev)
+    if one_call:
+        same_routing = bool(torch.equal(ids_one, ids_dev) and torch.equal(w_one, w_dev))
+    else:
+        out_dev = moe.experts(x[:n].contiguous(), w_dev, ids_dev)
     torch.cuda.synchronize()
     xs = x[:n].cpu()
     wr = moe.router_weight.float().cpu()
@@ -314,6 +324,8 @@ def cpu_baseline(pkg, moe, cfg, x, sample_tokens):
               "routing_weights_max_abs_diff": (w_dev.cpu() - w_ref).abs().max().item(),
               "outputs_outside_rtol2e-2_atol1e-2": ((got - ref).abs() > 1e-2 + 2e-2 * ref.abs()).float().mean().item(),
               "cos_diff": orc.cal_diff(ref, got)[0], "tokens_checked": n}
+    if one_call:
+        parity["one_call_routing_equals_staged_routing"] = same_routing
     base = dict(value=gemm_flops(cfg, n) / sec / 1e12, unit="TFLOP/s", cores=threads, kind="port",
                 sample=f"first {n} tokens of the same batch through the CPU oracle (routing twice, per-expert "
                        f"dequantise + fp32 matmul, weighted reduce): {sec:.1f} s, {n / sec:.2f} tokens/s",
