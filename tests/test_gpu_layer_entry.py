@@ -92,7 +92,7 @@ LAYER_CASES = [
 
 
 @pytest.mark.parametrize("T,H,I,E,K,mode,G,TG,with_bias,I_sh", LAYER_CASES)
-def test_decode_layer_entry_point(pkg, oracle, dev, T, H, I, E, K, mode, G, TG, with_bias, I_sh):
+def test_layer_entry_point(pkg, oracle, dev, T, H, I, E, K, mode, G, TG, with_bias, I_sh):
     say("decode layer", T, H, I, E, K, mode, G, TG, with_bias, I_sh)
     small = 3 * E * H * I <= (1 << 26)
     if small:
@@ -177,7 +177,7 @@ def test_router_logits_kernel(pkg, dev, T, H, E):
     assert bool((err <= bound).all()), float((err - bound).max())
 
 
-def test_decode_layer_in_a_hip_graph(pkg, oracle, dev):
+def test_layer_entry_point_in_a_hip_graph(pkg, oracle, dev):
     say("decode layer graph")
     T, H, I, E, K = 4, 1024, 256, 64, 4
     ld = tuple(t.to(dev) for t in oracle.make_layer(E, H, I, seed=5))
