@@ -382,6 +382,20 @@ def main():
         result["decode"] = bench_decode(pkg, moe, cfg, dev, args.steps, args.warmup)
     if not args.no_decode and args.workload == "c3_prefill":
         result["dense"] = bench_dense(pkg, dev, args.steps, args.warmup)
+        # the same layer between decode and the headline batch: the step alone, with the bytes of the experts it touched
+        sweep = []
+        for Ts in (128, 512, 2048):
+            g = torch.Generator(device=dev).manual_seed(200 + Ts)
+            xs_ = torch.randn(Ts, cfg["H"], generator=g, device=dev).to(torch.bfloat16)
+            outs_ = torch.empty(Ts, cfg["H"], dtype=torch.bfloat16, device=dev)
+            ssec = time_steps(lambda: moe(xs_, out=outs_), args.steps, args.warmup)
+            _, ids_ = moe.route(xs_)
+            touched = int(torch.unique(ids_).numel())
+            byts = touched * expert_bytes(cfg["H"], cfg["I"]) + (expert_bytes(cfg["H"], cfg["I_sh"]) if cfg["I_sh"] else 0)
+            sweep.append(dict(T=Ts, ms_per_step=ssec * 1e3, tflops=gemm_flops(cfg, Ts) / ssec / 1e12,
+                              weight_gbs=byts / ssec / 1e9, experts_touched=touched,
+                              tile_rows=pkg.tile_rows(Ts, cfg["K"], cfg["E"])))
+        result["batch_sweep"] = sweep
         # the two matrix-core-bound layer shapes of the same benchmark definition, same step, for the record
         others = []
         for name in ("c2_prefill", "c5_skewed"):
