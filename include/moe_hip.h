@@ -196,6 +196,15 @@ int moe_fused_experts_bf16(void *stream, const void *x_bf16, int T, int H, const
 size_t moe_mm_fp8_workspace_bytes(int M, int K, int N);
 int moe_mm_fp8(void *stream, const void *x_bf16, int M, int K, const uint8_t *w, const float *w_scale, int N,
                void *out_bf16, void *workspace, size_t workspace_bytes);
+/*
+ * The reference's own arithmetic for the same dense layer (MmW8A16Dq.cpp:185-228 multiplies bf16
+ * activations with weights de-quantised to bf16): out [M, N] bf16 = x [M, K] bf16 times the transpose of
+ * w [N, K] bf16, bf16 matrix instructions with fp32 accumulation.  The caller de-quantises once; this is
+ * also the route for block sizes that do not divide into 128-blocks (the reference's tests use 64:
+ * python/regression/test_llm/test_deepseek_mm.py:225).  K a multiple of 64 and at most 16384, N a multiple
+ * of 16.  No workspace.
+ */
+int moe_mm_bf16(void *stream, const void *x_bf16, int M, int K, const void *w_bf16, int N, void *out_bf16);
 size_t moe_mlp_fp8_workspace_bytes(int M, int H, int I);
 int moe_mlp_fp8(void *stream, const void *x_bf16, int M, int H, const uint8_t *w13, const float *w13_scale,
                 const uint8_t *w2, const float *w2_scale, int I, void *out_bf16, void *workspace,

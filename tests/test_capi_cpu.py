@@ -57,6 +57,10 @@ def test_argument_errors_are_codes_not_crashes(pkg):
     assert lib.moe_mm_fp8(None, fake, 4, 200, fake, fake, 64, fake, fake, 1 << 20) == E_ALIGN    # K % 128
     assert lib.moe_mm_fp8(None, fake, 4, 256, fake, fake, 8, fake, fake, 1 << 20) == E_SHAPE     # N < 16
     assert lib.moe_mlp_fp8(None, fake, 4, 256, fake, fake, fake, fake, 128, fake, fake, 16) == E_WS
+    assert lib.moe_mm_bf16(None, fake, 4, 200, fake, 64, fake) == E_ALIGN                        # K % 64
+    assert lib.moe_mm_bf16(None, fake, 4, 32768, fake, 64, fake) == E_SHAPE                      # K > 16384
+    assert lib.moe_mm_bf16(None, fake, 4, 256, None, 64, fake) == E_NULL
+    assert lib.moe_mm_bf16(None, None, 0, 256, fake, 64, None) == 0                              # no rows: nothing to do
     assert lib.moe_permute(None, fake, 4, 2, 5000, fake, fake, fake, fake, 1 << 20) == E_SHAPE
     ws = lib.moe_fused_experts_workspace_bytes(4, 256, 512, 8, 2, 0)
     assert ws > 0 and ws % 256 == 0

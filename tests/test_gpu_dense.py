@@ -71,12 +71,69 @@ def test_mlp_w8a16_dq_forward(pkg, oracle, dev, M, H, I):
     assert oracle.cal_diff(ref, got)[0] < 1e-4
 
 
+@pytest.mark.parametrize("block", [64, 256])
+@pytest.mark.parametrize("M,K,N", [(32, 2048, 512), (16, 2048, 512), (200, 1024, 272)])
+def test_mm_block_sizes(pkg, oracle, dev, M, K, N, block):
+    """The reference's block-size grid (python/regression/test_llm/test_deepseek_mm.py:225-248: 64, 128, 256 on
+    32 x 2048 -> 512).  256: the FP8 kernels on scales expanded to 128-blocks; 64: the reference's bf16 arithmetic."""
+    say("mm block", block, M, K, N)
+    g = torch.Generator().manual_seed(3000 + block + M)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = torch.randn(N, K, generator=g).to(torch.float8_e4m3fn)
+    s = torch.rand((N + block - 1) // block, (K + block - 1) // block, generator=g).to(torch.bfloat16)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    torch.ops.my_ops.mm_w8a16_dq_forward(x.to(dev), w.to(dev), s.to(dev), out, block)
+    torch.cuda.synchronize()
+    got = out.float().cpu()
+    assert torch.isfinite(got).all()
+    ref16 = oracle.mm_w8a16_dq_ref(x, w, s, block).float()
+    assert oracle.cos_sim(ref16.flatten(), got.flatten()) >= 0.99
+    if block == 64:
+        # same arithmetic as the reference: bf16 operands, fp32 accumulation, one rounding
+        ref = x.float() @ oracle.weight_dequant_literal(w, s, block).float().T
+        assert normalised_outside(got, ref) == 0.0
+        assert oracle.cal_diff(ref16, got)[0] < 1e-4
+    else:
+        xq, xs = oracle.act_quant_group128(x)
+        ref = oracle.act_dequant_group128(xq, xs) @ oracle.dequant_block(w, s.float(), block).T
+        assert normalised_outside(got, ref) == 0.0
+
+
+@pytest.mark.parametrize("block", [64, 256])
+def test_mlp_block_sizes(pkg, oracle, dev, block):
+    say("mlp block", block)
+    M, H, I = 48, 512, 256
+    g = torch.Generator().manual_seed(4000 + block)
+    x = torch.randn(M, H, generator=g).to(torch.bfloat16)
+    wg, wu = (torch.randn(I, H, generator=g).to(torch.float8_e4m3fn) for _ in range(2))
+    wd = torch.randn(H, I, generator=g).to(torch.float8_e4m3fn)
+    sg, su = (torch.rand(I // block, H // block, generator=g).mul(0.1).to(torch.bfloat16) for _ in range(2))
+    sd = torch.rand(H // block, I // block, generator=g).mul(0.1).to(torch.bfloat16)
+    out = torch.empty(M, H, dtype=torch.bfloat16, device=dev)
+    torch.ops.my_ops.mlp_w8a16_dq_forward(x.to(dev), wg.to(dev), wu.to(dev), wd.T.to(dev), sg.to(dev), su.to(dev),
+                                          sd.T.to(dev), out, block)
+    torch.cuda.synchronize()
+    got = out.float().cpu()
+    assert torch.isfinite(got).all()
+    ref16 = oracle.mlp_w8a16_dq_ref(x, wg, wu, wd, sg, su, sd, block).float()
+    assert oracle.cos_sim(ref16.flatten(), got.flatten()) >= 0.99
+    if block == 64:
+        assert oracle.cal_diff(ref16, got)[0] < 1e-4
+        assert normalised_outside(got, ref16) <= MAX_OUTSIDE
+    else:
+        w13q = torch.cat([wg, wu], 0)
+        w13s = torch.cat([sg, su], 0).float().repeat_interleave(2, 0).repeat_interleave(2, 1)
+        ref = oracle.mlp_w8a8_fp32(x, w13q, w13s, wd, sd.float().repeat_interleave(2, 0).repeat_interleave(2, 1))
+        assert normalised_outside(got, ref) <= MAX_OUTSIDE
+        assert oracle.cal_diff(ref, got)[0] < 1e-4
+
+
 def test_dense_ops_reject_what_they_do_not_support(pkg, dev):
     x = torch.zeros(4, 256, dtype=torch.bfloat16, device=dev)
     w = torch.zeros(128, 256, dtype=torch.float8_e4m3fn, device=dev)
     s = torch.ones(1, 2, dtype=torch.bfloat16, device=dev)
     out = torch.empty(4, 128, dtype=torch.bfloat16, device=dev)
     with pytest.raises(RuntimeError):
-        torch.ops.my_ops.mm_w8a16_dq_forward(x, w, s, out, 64)
+        torch.ops.my_ops.mm_w8a16_dq_forward(x, w, s, out, 0)
     with pytest.raises(RuntimeError):
         torch.ops.my_ops.mm_w8a16_dq_forward(x, w.view(torch.uint8), s, out, 128)

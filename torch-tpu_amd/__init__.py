@@ -9,10 +9,10 @@ from . import my_ops as _my_ops         # noqa: F401  (registers torch.ops.my_op
 from .my_ops import set_expert_numerics
 from .layer import FusedMoE, convert_hf_moe_layer, pack_expert_weights, quant_weight_block128
 from .ops import (MoeHipError, act_quant, layer_eligible, layer_fp8, layer_workspace_bytes,
-                  fused_experts_bf16, fused_experts_fp8, fused_experts_workspace_bytes, gemm1_swiglu, gemm2, mlp_fp8, mm_fp8,
+                  fused_experts_bf16, fused_experts_fp8, fused_experts_workspace_bytes, gemm1_swiglu, gemm2, mlp_fp8, mm_bf16, mm_fp8,
                   moe_permute, moe_route, noaux_tc_topk, router_logits, scale_pitch, tile_rows, weighted_reduce)
 
 __all__ = ["FusedMoE", "set_expert_numerics", "convert_hf_moe_layer", "pack_expert_weights", "quant_weight_block128", "MoeHipError", "act_quant",
            "layer_eligible", "layer_fp8", "layer_workspace_bytes", "fused_experts_bf16", "fused_experts_fp8",
-           "fused_experts_workspace_bytes", "gemm1_swiglu", "gemm2", "mlp_fp8", "mm_fp8", "moe_permute", "moe_route", "noaux_tc_topk", "router_logits",
+           "fused_experts_workspace_bytes", "gemm1_swiglu", "gemm2", "mlp_fp8", "mm_bf16", "mm_fp8", "moe_permute", "moe_route", "noaux_tc_topk", "router_logits",
            "scale_pitch", "tile_rows", "weighted_reduce"]

@@ -157,31 +157,67 @@ def _grouped_topk(*args):
 
 
 def _check_dense(blocksize, *fp8):
-    if blocksize != 128:
-        raise RuntimeError("only blocksize 128 is supported")
+    if blocksize < 1:
+        raise RuntimeError("blocksize must be positive")
     for t in fp8:
         if t.dtype != torch.float8_e4m3fn:
             raise RuntimeError("weights must be float8_e4m3fn")
 
 
+def _scales_128(s, blocksize, rows, cols):
+    """Block scales of a [rows, cols] matrix at a block size that is a multiple of 128, as fp32 scales of
+    128 x 128 blocks: every 128-block takes the scale of the block it lies in (the same products, exactly)."""
+    m = blocksize // 128
+    s = s.to(torch.float32).repeat_interleave(m, dim=-2).repeat_interleave(m, dim=-1)
+    return s[..., :(rows + 127) // 128, :(cols + 127) // 128].contiguous()
+
+
+def _dequant_any(w, s, blocksize):
+    """[N, K] fp8 with [ceil(N/bs), ceil(K/bs)] scales -> bf16(fp8) * bf16 scale in bf16, the reference's
+    weight_dequant (python/regression/test_llm/test_mm_w8a16_dq.py:10-49) for any block size."""
+    N, K = w.shape
+    full = s.to(torch.bfloat16).repeat_interleave(blocksize, dim=0)[:N].repeat_interleave(blocksize, dim=1)[:, :K]
+    return (w.to(torch.bfloat16) * full).contiguous()
+
+
 def _mlp_w8a16_dq_forward(input, gate_weight, up_weight, down_weight, gate_scale, up_scale, down_scale, output,
                           blocksize):
     """torch_tpu/csrc/ops/my_ops/MlpW8A16Dq.cpp:189-241: gate/up [I,H], down passed transposed as
-    [I,H] (python/regression/test_llm/test_mlp_w8a16_dq.py:106-109), scales likewise; output [M,H]."""
+    [I,H] (python/regression/test_llm/test_mlp_w8a16_dq.py:106-109), scales likewise; output [M,H].
+    Block sizes that are multiples of 128 run the FP8 kernels on the expanded scales; others run the
+    reference's own bf16 arithmetic on weights de-quantised once."""
     _check_dense(blocksize, gate_weight, up_weight, down_weight)
+    I, H = gate_weight.shape
+    if blocksize % 128:
+        w13, w2 = _dense_packed(
+            (gate_weight, up_weight, down_weight, gate_scale, up_scale, down_scale),
+            lambda: (torch.cat([_dequant_any(gate_weight, gate_scale, blocksize),
+                                _dequant_any(up_weight, up_scale, blocksize)], 0).unsqueeze(0).contiguous(),
+                     _dequant_any(down_weight, down_scale, blocksize).t().unsqueeze(0).contiguous()))
+        # one expert that every row selects; its per-slot result [M, 1, H] is the output itself
+        M = input.shape[0]
+        ids = torch.zeros(M, 1, dtype=torch.int32, device=input.device)
+        ops.fused_experts_bf16(input.contiguous(), w13, w2, ids, None, out=output.view(M, 1, H))
+        return output
     w13, w13s, w2, w2s = _dense_packed(
         (gate_weight, up_weight, down_weight, gate_scale, up_scale, down_scale),
         lambda: (torch.cat([gate_weight, up_weight], 0).contiguous(),
-                 torch.cat([gate_scale, up_scale], 0).to(torch.float32).contiguous(),
-                 down_weight.t().contiguous(), down_scale.t().to(torch.float32).contiguous()))
+                 torch.cat([_scales_128(gate_scale, blocksize, I, H), _scales_128(up_scale, blocksize, I, H)], 0).contiguous(),
+                 down_weight.t().contiguous(), _scales_128(down_scale, blocksize, I, H).t().contiguous()))
     ops.mlp_fp8(input.contiguous(), w13, w13s, w2, w2s, out=output)
     return output
 
 
 def _mm_w8a16_dq_forward(input, weight, scale, output, blocksize):
-    """torch_tpu/csrc/ops/my_ops/MmW8A16Dq.cpp:185-228: weight [N,K], scale [ceil(N/bs), K/bs], output [M,N]."""
+    """torch_tpu/csrc/ops/my_ops/MmW8A16Dq.cpp:185-228: weight [N,K], scale [ceil(N/bs), ceil(K/bs)], output [M,N].
+    Block sizes as in mlp_w8a16_dq_forward."""
     _check_dense(blocksize, weight)
-    w, ws = _dense_packed((weight, scale), lambda: (weight.contiguous(), scale.to(torch.float32).contiguous()))
+    N, K = weight.shape
+    if blocksize % 128:
+        (w,) = _dense_packed((weight, scale), lambda: (_dequant_any(weight, scale, blocksize),))
+        ops.mm_bf16(input.contiguous(), w, out=output)
+        return output
+    w, ws = _dense_packed((weight, scale), lambda: (weight.contiguous(), _scales_128(scale, blocksize, N, K)))
     ops.mm_fp8(input.contiguous(), w, ws, out=output)
     return output
 

@@ -340,6 +340,20 @@ def mm_fp8(x, w, w_scale, out=None, workspace=None):
     return out
 
 
+def mm_bf16(x, w, out=None):
+    """Dense linear layer on un-quantised operands: x [M,K] bf16, w [N,K] bf16 -> out [M,N] bf16."""
+    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], "x must be [M,K] and w [N,K]")
+    M, K = x.shape
+    N = w.shape[0]
+    if out is None:
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=x.device)
+    _need(tuple(out.shape) == (M, N), "out must be [M,N]")
+    rc = lib.moe_mm_bf16(_stream(), _dev(x, "x", torch.bfloat16), M, K, _dev(w, "w", torch.bfloat16), N,
+                         _dev(out, "out", torch.bfloat16))
+    check(rc, "mm_bf16")
+    return out
+
+
 def mlp_fp8(x, w13, w13_scale, w2, w2_scale, out=None, workspace=None):
     """Dense gated MLP: x [M,H] bf16, w13 [2I,H] (gate rows then up rows), w2 [H,I], fp32 128x128
     block scales -> out [M,H] bf16 = (silu(x Wg^T) * (x Wu^T)) Wd^T, FP8 matrix products."""
