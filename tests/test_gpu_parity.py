@@ -345,6 +345,39 @@ def test_my_ops_drop_in_reference_layout(pkg, oracle, dev):
     assert oracle.cal_diff(ref_bf16, got16)[0] < 1e-4
 
 
+@pytest.mark.parametrize("block", [64, 256])
+def test_my_ops_other_block_sizes(pkg, oracle, dev, block):
+    """Block sizes next to 128 (the reference's dense tests use 64 and 256): 256 runs the FP8 kernels on scales
+    expanded to 128-blocks, 64 the reference's bf16 arithmetic on weights de-quantised once."""
+    say("my_ops block", block)
+    T, H, I, E, K = 12, 512, 256, 8, 2
+    g = torch.Generator().manual_seed(block)
+    sel = torch.argsort(torch.rand(T, E, generator=g), dim=-1)[:, :K].to(torch.int32)
+    w0, w1 = ((torch.randn(E, I, H, generator=g) * 0.1).to(torch.float8_e4m3fn) for _ in range(2))
+    w2 = (torch.randn(E, H, I, generator=g) * 0.1).to(torch.float8_e4m3fn)
+    s0, s1 = ((torch.rand(E, I // block, H // block, generator=g) * 0.1 + 0.01).to(torch.bfloat16) for _ in range(2))
+    s2 = (torch.rand(E, H // block, I // block, generator=g) * 0.1 + 0.01).to(torch.bfloat16)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    rw = torch.rand(T, K, generator=g).to(torch.bfloat16)
+    ref_bf16 = oracle.experts_ref_bf16(x, sel, w0, w1, w2, s0, s1, s2, block).float()
+    out = torch.empty(T, K, H, dtype=torch.bfloat16, device=dev)
+    torch.ops.my_ops.fused_moe_fused_experts(
+        out, x.to(dev), None, None, w0.to(dev), w1.to(dev), w2.transpose(1, 2).contiguous().to(dev), s0.to(dev),
+        s1.to(dev), s2.transpose(1, 2).contiguous().to(dev), sel.to(dev), rw.to(dev), None, None, None, block, E, K,
+        True, 8, 4, None, None, None, False)
+    torch.cuda.synchronize()
+    got = out.float().cpu()
+    assert torch.isfinite(got).all()
+    assert oracle.cos_sim(ref_bf16.numpy(), got.numpy()) > 0.99
+    if block == 64:
+        assert oracle.cal_diff(ref_bf16, got)[0] < 1e-4
+    else:
+        up = lambda t: t.float().repeat_interleave(2, 1).repeat_interleave(2, 2)
+        ref = oracle.experts_w8a8_fp32(x, sel, torch.cat([w0, w1], 1), torch.cat([up(s0), up(s1)], 1), w2, up(s2))
+        scale = ref.abs().max().item()
+        assert outside_fraction(got / scale, ref / scale) <= MAX_OUTSIDE
+
+
 def test_layer_module_end_to_end_toy_config(pkg, oracle, dev):
     say("toy config end to end")
     T, H, I, E, K = 16, 256, 512, 8, 2

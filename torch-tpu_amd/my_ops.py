@@ -53,10 +53,10 @@ def set_expert_numerics(mode: str) -> None:
     _numerics = mode
 
 
-def _dequant_bf16(w, s):
-    """[E, N, K] fp8 with [E, ceil(N/128), ceil(K/128)] scales -> bf16, as the reference's weight_dequant does."""
+def _dequant_bf16(w, s, blocksize=128):
+    """[E, N, K] fp8 with [E, ceil(N/bs), ceil(K/bs)] scales -> bf16, as the reference's weight_dequant does."""
     E, N, K = w.shape
-    full = s.to(torch.bfloat16).repeat_interleave(128, dim=1)[:, :N].repeat_interleave(128, dim=2)[:, :, :K]
+    full = s.to(torch.bfloat16).repeat_interleave(blocksize, dim=1)[:, :N].repeat_interleave(blocksize, dim=2)[:, :, :K]
     return (w.to(torch.float32) * full.to(torch.float32)).to(torch.bfloat16)
 
 
@@ -119,16 +119,24 @@ def _fused_experts(output, input, output_sample, input_sample, gate_weights, up_
         return output
     if gate_scales is None or up_scales is None or down_scales is None:
         raise RuntimeError("either all three weight tensors carry block scales or none does")
-    if blocksize != 128:
-        raise RuntimeError("blocksize must be 128")
-    if _numerics == "w8a16":
+    if blocksize < 1:
+        raise RuntimeError("blocksize must be positive")
+    # block sizes that 128 does not divide cannot share a 128-long FP8 dot product: the reference's arithmetic then
+    if _numerics == "w8a16" or blocksize % 128:
         w13, w2 = _dense_packed(
             (gate_weights, up_weights, down_weights, gate_scales, up_scales, down_scales),
-            lambda: (torch.cat([_dequant_bf16(gate_weights, gate_scales), _dequant_bf16(up_weights, up_scales)], 1).contiguous(),
-                     _dequant_bf16(down_weights, down_scales).transpose(1, 2).contiguous()))
+            lambda: (torch.cat([_dequant_bf16(gate_weights, gate_scales, blocksize),
+                                _dequant_bf16(up_weights, up_scales, blocksize)], 1).contiguous(),
+                     _dequant_bf16(down_weights, down_scales, blocksize).transpose(1, 2).contiguous()))
         rw = routing_weights.to(torch.float32) if output.dim() == 2 else None
         ops.fused_experts_bf16(input, w13, w2, select_experts, rw, out=output)
         return output
+    if blocksize != 128:
+        # a multiple of 128: every 128-block takes the scale of the block it lies in (the same products, exactly)
+        I, H = gate_weights.shape[1:]
+        gate_scales, up_scales, down_scales = _dense_packed(
+            (gate_scales, up_scales, down_scales),
+            lambda: tuple(_scales_128(t, blocksize, I, H) for t in (gate_scales, up_scales, down_scales)))
     w13, w13s, w2, w2s = _packed(gate_weights, up_weights, down_weights, gate_scales, up_scales, down_scales)
     if w13.shape[0] != num_experts or select_experts.shape[1] != num_experts_per_tok:
         raise RuntimeError("num_experts / num_experts_per_tok do not match the tensors")
