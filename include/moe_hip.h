@@ -218,8 +218,9 @@ int moe_mlp_fp8(void *stream, const void *x_bf16, int M, int H, const uint8_t *w
  * (torch_tpu/csrc/ops/my_ops/fusedMoE.cpp:117-236).
  * Decode-size batches (T * K <= 256 slots): two launches stand in front of the grouped GEMMs - the router
  * logits together with the activation quantisation, then routing and permutation.  Larger batches: the
- * router product runs on the matrix cores with its reduction cut into slices, and the routing kernel adds
- * the slices.  Either way the logits are fp32 sums rounded once to bf16.
+ * router product runs on the matrix cores with its reduction cut into slices, the routing kernel adds
+ * the slices, and the activations are quantised by extra workgroups of that launch.  Either way the logits
+ * are fp32 sums rounded once to bf16.
  * router_w_bf16 [E, H] bf16; router_bias [E] fp32 or NULL (selection only, as in moe_route_topk);
  * mode MOE_ROUTE_SOFTMAX or MOE_ROUTE_SIGMOID; the other routing arguments as in moe_route_topk.
  * out bf16 [T, H] (the weighted sum, shared expert added when its pointers are non-NULL).

@@ -270,7 +270,9 @@ def check_experts(pkg, oracle, dev, x, layer, ids, w, shared=None):
 
 @pytest.mark.parametrize("T,H,I,E,K", [
     (16, 256, 512, 8, 2),        # the toy configuration
-    (1, 256, 128, 1, 1), (1, 7168, 256, 2, 2), (1, 7168, 256, 16, 8), (8, 7168, 256, 256, 8),   # reference grid
+    (1, 256, 128, 1, 1),
+    # the reference's grid (python/regression/test_llm/test_moe.py:219-227, 310-316)
+    (1, 7168, 256, 1, 1), (1, 7168, 256, 2, 2), (1, 7168, 256, 16, 8), (1, 7168, 256, 256, 8), (8, 7168, 256, 256, 8),
     (17, 512, 384, 8, 2), (33, 512, 256, 4, 2), (64, 1024, 256, 16, 4), (65, 256, 256, 8, 2),
     (200, 512, 256, 8, 2), (300, 256, 128, 3, 2), (256, 7168, 256, 256, 8),
 ])

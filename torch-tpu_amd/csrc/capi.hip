@@ -26,7 +26,7 @@ int router_front_launch(hipStream_t st, const void *x, int T, int H, const void 
 int sum_slices_launch(hipStream_t st, const float *partial, int n_slices, int T, int E, uint16_t *logits);
 int route_from_partials_launch(hipStream_t st, const float *partial, int n_slices, const float *bias, int T, int E, int K,
                                int mode, int n_groups, int topk_groups, int renorm, float scale, float *weights_out,
-                               int32_t *ids_out);
+                               int32_t *ids_out, const uint16_t *x, int H, uint8_t *xq, float *xs);
 
 size_t dense_small_partial_bytes(int M, int K, int N, bool keep_partial);
 int dense_small_launch(hipStream_t st, const uint8_t *xq, const float *xs, int M, int K, const uint8_t *w, const float *ws,
@@ -253,12 +253,11 @@ extern "C" int moe_layer_fp8(void *stream, const void *x_bf16, int T, int H, con
       rc = sum_slices_launch(st, d.partial, n_slices, T, E, (uint16_t *)logits_out_bf16);
       if (rc) return rc;
     }
+    // the activations are quantised by extra workgroups of the routing launch
     rc = route_from_partials_launch(st, d.partial, n_slices, router_bias, T, E, K, mode, n_groups, topk_groups, renorm,
-                                    scale, weights, ids);
+                                    scale, weights, ids, (const uint16_t *)x_bf16, H, w.xq, w.xs);
     if (rc) return rc;
     rc = permute_launch(st, ids, T, K, E, choose_tile_m(T, K, E), w.sorted_slot, w.expert_offsets, w.slot_to_row, pw);
-    if (rc) return rc;
-    rc = moe_act_quant(stream, x_bf16, T, H, w.xq, w.xs);
     if (rc) return rc;
   }
   return run_experts(stream, w, pw, T, H, w13, w13_scale, w2, w2_scale, I, E, K, weights, shared_w13, shared_w13_scale,

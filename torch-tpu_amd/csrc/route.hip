@@ -5,6 +5,8 @@
 // "greater value, then lower index" as the order, so equal scores resolve to the lower index
 // on every lane identically and the K picks come out in descending order.
 #include "moe_common.h"
+#include "moe_layout.h"
+#include "act_quant.h"
 #include "route_block.h"
 #include "../../include/moe_hip.h"
 
@@ -191,12 +193,31 @@ __global__ __launch_bounds__(256) void noaux_tc_topk_kernel(const void *__restri
   }
 }
 
+// Activation quantisation riding in the routing launch: the workgroups from `first_block` on quantise x (16 lanes
+// per 128-column group) instead of routing.  Routing is a chain of cross-lane steps per token and leaves the memory
+// system idle; the quantiser is pure streaming, so the two share the chip instead of following one another.
+struct QuantRide {
+  const uint16_t *x;      // null: nobody rides
+  uint8_t *q;
+  float *s;
+  size_t n_groups;
+  int groups_per_row;
+  int pitch;
+  int first_block;
+};
+
 template <int PER_LANE>
 __global__ __launch_bounds__(256) void route_topk_kernel(const void *__restrict__ logits, int logits_bf16,
                                                           const float *__restrict__ bias, int T, int E, int K, int mode,
                                                           int n_groups, int topk_groups, int renorm, float scale,
                                                           float *__restrict__ weights_out, int32_t *__restrict__ ids_out,
-                                                          float *__restrict__ scores_out, int n_slices = 0) {
+                                                          float *__restrict__ scores_out, int n_slices = 0,
+                                                          const QuantRide ride = QuantRide{}) {
+  if (ride.x != nullptr && (int)blockIdx.x >= ride.first_block) {
+    act_quant_thread(ride.x, ride.n_groups, ride.groups_per_row, ride.pitch, ride.q, ride.s,
+                     (size_t)(blockIdx.x - ride.first_block) * 256 + threadIdx.x);
+    return;
+  }
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (t >= T) return;
@@ -318,20 +339,35 @@ int sum_slices_launch(hipStream_t st, const float *partial, int n_slices, int T,
 }
 
 // routing straight from the partial sums of the router product (E <= 256: four scores per lane)
+// x / H / xq / xs: the activations [T, H] bf16 are quantised in the same launch (xq e4m3fn [T, H], xs fp32 with
+// pitch scale_pitch(H / 128)); x null: routing only.
 int route_from_partials_launch(hipStream_t st, const float *partial, int n_slices, const float *bias, int T, int E, int K,
                                int mode, int n_groups, int topk_groups, int renorm, float scale, float *weights_out,
-                               int32_t *ids_out) {
+                               int32_t *ids_out, const uint16_t *x, int H, uint8_t *xq, float *xs) {
   if (E > 256 || n_slices < 1) return MOE_E_SHAPE;
   if (mode != MOE_ROUTE_SOFTMAX && mode != MOE_ROUTE_SIGMOID) return MOE_E_MODE;
   const int rc = check_route_shape(T, E, K, n_groups, topk_groups);
   if (rc) return rc;
-  dim3 grid((T + 3) / 4), block(256);
+  const int route_blocks = (T + 3) / 4;
+  QuantRide ride{};
+  long blocks = route_blocks;
+  if (x != nullptr) {
+    if (H % kBlock) return MOE_E_ALIGN;
+    ride.x = x; ride.q = xq; ride.s = xs;
+    ride.n_groups = (size_t)T * (H / kBlock);
+    ride.groups_per_row = H / kBlock;
+    ride.pitch = scale_pitch(H / kBlock);
+    ride.first_block = route_blocks;
+    blocks += (long)((ride.n_groups * 16 + 255) / 256);
+  }
+  if (blocks > 0x7fffffffl) return MOE_E_SHAPE;
+  dim3 grid((unsigned)blocks), block(256);
   if (E <= 64)
-    route_topk_kernel<1><<<grid, block, 0, st>>>(partial, 0, bias, T, E, K, mode, n_groups, topk_groups, renorm, scale, weights_out, ids_out, nullptr, n_slices);
+    route_topk_kernel<1><<<grid, block, 0, st>>>(partial, 0, bias, T, E, K, mode, n_groups, topk_groups, renorm, scale, weights_out, ids_out, nullptr, n_slices, ride);
   else if (E <= 128)
-    route_topk_kernel<2><<<grid, block, 0, st>>>(partial, 0, bias, T, E, K, mode, n_groups, topk_groups, renorm, scale, weights_out, ids_out, nullptr, n_slices);
+    route_topk_kernel<2><<<grid, block, 0, st>>>(partial, 0, bias, T, E, K, mode, n_groups, topk_groups, renorm, scale, weights_out, ids_out, nullptr, n_slices, ride);
   else
-    route_topk_kernel<4><<<grid, block, 0, st>>>(partial, 0, bias, T, E, K, mode, n_groups, topk_groups, renorm, scale, weights_out, ids_out, nullptr, n_slices);
+    route_topk_kernel<4><<<grid, block, 0, st>>>(partial, 0, bias, T, E, K, mode, n_groups, topk_groups, renorm, scale, weights_out, ids_out, nullptr, n_slices, ride);
   return (int)hipGetLastError();
 }
 
