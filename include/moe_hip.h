@@ -131,6 +131,8 @@ int moe_act_quant(void *stream, const void *x_bf16, int R, int C, uint8_t *q, fl
  * out_mode 1: out is bf16 [T, H] = sum_k routing_weights[t,k] * slot result (fp32 sum).
  *             If the shared_* pointers are non-NULL a shared expert (W13 [1,2*I_sh,H],
  *             W2 [1,H,I_sh]) is applied to every token and added with weight 1.
+ * A slot whose id lies outside [0, E) has no expert (how a rank of an expert-parallel group marks the
+ * experts it does not hold): its row in the [T, K, H] form is zero and it adds nothing to the sum.
  * workspace: moe_fused_experts_workspace_bytes(...) bytes, 256-byte aligned.
  */
 size_t moe_fused_experts_workspace_bytes(int T, int H, int I, int E, int K, int I_shared);

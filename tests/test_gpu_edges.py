@@ -69,6 +69,55 @@ def test_ids_outside_the_expert_range_are_dropped(pkg, oracle, dev):
     assert torch.equal(s2r.long(), inv)
 
 
+@pytest.mark.parametrize("T", [5, 37, 300])
+def test_slots_without_an_expert_add_nothing(pkg, oracle, dev, T):
+    """Ids outside [0, E) (how an expert-parallel rank marks the experts it does not hold): zero rows in the
+    [T, K, H] form, no term in the weighted sum, everything else as if the slot were not there."""
+    say("dropped slots in the expert computation", T)
+    H, I, E, K = 256, 128, 8, 3
+    layer = oracle.make_layer(E, H, I, seed=12)
+    g = torch.Generator().manual_seed(12 + T)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    ids = torch.argsort(torch.rand(T, E, generator=g), dim=-1)[:, :K].to(torch.int32)
+    w = torch.rand(T, K, generator=g)
+    bad = torch.rand(T, K, generator=g) < 0.3
+    bad[0] = True                                            # a token none of whose slots has an expert
+    ids_bad = ids.clone()
+    ids_bad[bad] = torch.where(torch.rand(int(bad.sum()), generator=g) < 0.5, torch.tensor(-1), torch.tensor(E)).to(torch.int32)
+    ref_slots = oracle.experts_w8a8_fp32(x, ids, *layer)
+    ref_slots[bad] = 0.0
+    dl = tuple(t.to(dev) for t in layer)
+    # poisoned outputs and workspace: whatever the call does not write would show
+    out3 = torch.full((T, K, H), float("nan"), dtype=torch.bfloat16, device=dev)
+    pkg.fused_experts_fp8(x.to(dev), *dl, ids_bad.to(dev), out=out3)
+    torch.cuda.synchronize()
+    got3 = out3.float().cpu()
+    assert torch.isfinite(got3).all()
+    assert bool((got3[bad] == 0).all())
+    scale = ref_slots.abs().max().item()
+    frac = ((got3 - ref_slots).abs() > (1e-2 + 2e-2 * ref_slots.abs() / scale) * scale).float().mean().item()
+    assert frac <= 5e-3
+    ws = torch.empty(pkg.fused_experts_workspace_bytes(T, H, I, E, K), dtype=torch.uint8, device=dev)
+    ws.view(torch.int16)[: ws.numel() // 2].fill_(0x7FC0)       # bf16 NaN everywhere
+    out2 = pkg.fused_experts_fp8(x.to(dev), *dl, ids_bad.to(dev), w.to(dev), workspace=ws)
+    torch.cuda.synchronize()
+    got2 = out2.float().cpu()
+    assert torch.isfinite(got2).all()
+    assert bool((got2[0] == 0).all())
+    ref2 = torch.einsum("tk,tkh->th", w, got3)                  # the device's own slot results, summed on the host
+    torch.testing.assert_close(got2, ref2, rtol=2e-2, atol=1e-2 * scale)
+    # un-quantised experts take the same route
+    w13b = oracle.dequant_block(layer[0], layer[1]).to(torch.bfloat16).to(dev)
+    w2b = oracle.dequant_block(layer[2], layer[3]).to(torch.bfloat16).to(dev)
+    outb = torch.full((T, K, H), float("nan"), dtype=torch.bfloat16, device=dev)
+    pkg.fused_experts_bf16(x.to(dev), w13b, w2b, ids_bad.to(dev), out=outb)
+    torch.cuda.synchronize()
+    assert torch.isfinite(outb.float()).all() and bool((outb.float().cpu()[bad] == 0).all())
+    outb2 = pkg.fused_experts_bf16(x.to(dev), w13b, w2b, ids_bad.to(dev), w.to(dev))
+    torch.cuda.synchronize()
+    assert torch.isfinite(outb2.float()).all() and bool((outb2.float().cpu()[0] == 0).all())
+
+
 def test_one_workspace_serves_calls_of_different_sizes(pkg, oracle, dev):
     say("workspace reuse")
     H, I, E, K = 512, 256, 16, 4

@@ -21,6 +21,9 @@ int decode_prep_launch(hipStream_t st, const uint16_t *x, int T, int H, const ui
                        int32_t *ids, int *arrivals, uint8_t *xq, float *xs, int tile_m, int32_t *sorted_slot,
                        int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &pw);
 
+int zero_dropped_rows_launch(hipStream_t st, const int32_t *slot_to_row, int TK, int H, uint16_t *y);
+int weighted_reduce_launch(hipStream_t st, const uint16_t *y, const float *w, const uint16_t *shared_y,
+                           const int32_t *slot_to_row, int T, int K, int H, uint16_t *out);
 size_t router_front_partial_bytes(int T, int H, int E);
 int router_front_launch(hipStream_t st, const void *x, int T, int H, const void *wr, int E, float *partial, int *n_slices_out);
 int sum_slices_launch(hipStream_t st, const float *partial, int n_slices, int T, int E, uint16_t *logits);
@@ -93,7 +96,8 @@ static int run_experts(void *stream, const FusedWs &w, const PermuteWs &pw, int 
   rc = gemm2_launch(st, w.hq, w.hs, T * K, T, H, w2, w2_scale, I, E, K, w.sorted_slot, w.expert_offsets, &pw, -1, y,
                     w.sh_hq, w.sh_hs, T, fuse_shared ? shared_w2 : nullptr, shared_w2_scale, w.sh_y);
   if (rc) return rc;
-  if (out_mode == 0) return MOE_OK;
+  // slots whose expert id lies outside [0, E) have no row: zero rows in the per-slot form, no term in the sum
+  if (out_mode == 0) return zero_dropped_rows_launch(st, w.slot_to_row, T * K, H, y);
   if (has_shared && !fuse_shared) {
     rc = gemm1_launch(st, w.xq, w.xs, T, H, shared_w13, shared_w13_scale, I_sh, 1, 1, nullptr, nullptr, nullptr, 0,
                       w.sh_hq, w.sh_hs, nullptr, nullptr, nullptr, nullptr);
@@ -102,7 +106,8 @@ static int run_experts(void *stream, const FusedWs &w, const PermuteWs &pw, int 
                       0, w.sh_y, nullptr, nullptr, 0, nullptr, nullptr, nullptr);
     if (rc) return rc;
   }
-  return moe_weighted_reduce(stream, y, routing_weights, has_shared ? w.sh_y : nullptr, T, K, H, out_bf16);
+  return weighted_reduce_launch(st, y, routing_weights, has_shared ? w.sh_y : nullptr, w.slot_to_row, T, K, H,
+                                (uint16_t *)out_bf16);
 }
 
 // moe_layer_fp8: the fused-experts workspace followed by the router's own pieces
@@ -468,6 +473,6 @@ extern "C" int moe_fused_experts_bf16(void *stream, const void *x_bf16, int T, i
   rc = gemm2_launch(st, (const uint8_t *)w.h, nullptr, T * K, T, H, (const uint8_t *)w2_bf16, nullptr, I, E, K,
                     w.sorted_slot, w.expert_offsets, &pw, -1, y, nullptr, nullptr, 0, nullptr, nullptr, nullptr, true);
   if (rc) return rc;
-  if (out_mode == 0) return MOE_OK;
-  return moe_weighted_reduce(stream, y, routing_weights, nullptr, T, K, H, out_bf16);
+  if (out_mode == 0) return zero_dropped_rows_launch(st, w.slot_to_row, T * K, H, y);
+  return weighted_reduce_launch(st, y, routing_weights, nullptr, w.slot_to_row, T, K, H, (uint16_t *)out_bf16);
 }

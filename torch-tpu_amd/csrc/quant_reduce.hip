@@ -18,7 +18,8 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t *__restri
 // One lane produces 8 consecutive columns of one token.
 __global__ __launch_bounds__(256) void weighted_reduce_kernel(const uint16_t *__restrict__ y,
                                                               const float *__restrict__ w,
-                                                              const uint16_t *__restrict__ shared_y, int T, int K,
+                                                              const uint16_t *__restrict__ shared_y,
+                                                              const int32_t *__restrict__ slot_to_row, int T, int K,
                                                               int H, uint16_t *__restrict__ out) {
   const int hv = H >> 3;   // 16-byte vectors per row
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -28,6 +29,8 @@ __global__ __launch_bounds__(256) void weighted_reduce_kernel(const uint16_t *__
 #pragma unroll
   for (int i = 0; i < 8; i++) acc[i] = 0.f;
   for (int k = 0; k < K; k++) {
+    // a slot whose expert id was outside [0, E) has no row: nothing was computed for it and it adds nothing
+    if (slot_to_row != nullptr && slot_to_row[(size_t)t * K + k] < 0) continue;
     const float wk = w[(size_t)t * K + k];
     v4i raw = *(const v4i *)(y + ((size_t)t * K + k) * H + c);
 #pragma unroll
@@ -51,6 +54,33 @@ __global__ __launch_bounds__(256) void weighted_reduce_kernel(const uint16_t *__
   for (int i = 0; i < 4; i++)
     o[i] = (int)((uint32_t)f32_to_bf16(acc[2 * i]) | ((uint32_t)f32_to_bf16(acc[2 * i + 1]) << 16));
   *(v4i *)(out + (size_t)t * H + c) = o;
+}
+
+// [T, K, H] output form: the rows of slots without an expert (id outside [0, E)) are zero.  One thread per slot; the
+// rare thread that finds such a slot clears its row.
+__global__ __launch_bounds__(256) void zero_dropped_rows_kernel(const int32_t *__restrict__ slot_to_row, int TK, int H,
+                                                                uint16_t *__restrict__ y) {
+  const int s = blockIdx.x * 256 + threadIdx.x;
+  if (s >= TK || slot_to_row[s] >= 0) return;
+  v4i *row = (v4i *)(y + (size_t)s * H);
+  for (int i = 0; i < H / 8; i++) row[i] = (v4i){0, 0, 0, 0};
+}
+
+int zero_dropped_rows_launch(hipStream_t st, const int32_t *slot_to_row, int TK, int H, uint16_t *y) {
+  if (TK < 1) return MOE_OK;
+  zero_dropped_rows_kernel<<<(TK + 255) / 256, 256, 0, st>>>(slot_to_row, TK, H, y);
+  return (int)hipGetLastError();
+}
+
+// slot_to_row (may be null): slots with a negative entry are left out of the sum
+int weighted_reduce_launch(hipStream_t st, const uint16_t *y, const float *w, const uint16_t *shared_y,
+                           const int32_t *slot_to_row, int T, int K, int H, uint16_t *out) {
+  const size_t n = (size_t)T * (H / 8);
+  if (n == 0) return MOE_OK;
+  const size_t blocks = (n + 255) / 256;
+  if (blocks > 0x7fffffffull) return MOE_E_SHAPE;
+  weighted_reduce_kernel<<<(unsigned)blocks, 256, 0, st>>>(y, w, shared_y, slot_to_row, T, K, H, out);
+  return (int)hipGetLastError();
 }
 
 }  // namespace moe
@@ -80,11 +110,6 @@ extern "C" int moe_weighted_reduce(void *stream, const void *y_bf16, const float
   if (H % 8) return MOE_E_ALIGN;
   if (((uintptr_t)y_bf16 % 16) || ((uintptr_t)out_bf16 % 16) || (shared_y_bf16 && ((uintptr_t)shared_y_bf16 % 16)))
     return MOE_E_ALIGN;
-  const size_t n = (size_t)T * (H / 8);
-  if (n == 0) return MOE_OK;
-  const size_t blocks = (n + 255) / 256;
-  if (blocks > 0x7fffffffull) return MOE_E_SHAPE;
-  weighted_reduce_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>(
-      (const uint16_t *)y_bf16, routing_weights, (const uint16_t *)shared_y_bf16, T, K, H, (uint16_t *)out_bf16);
-  return (int)hipGetLastError();
+  return weighted_reduce_launch((hipStream_t)stream, (const uint16_t *)y_bf16, routing_weights,
+                                (const uint16_t *)shared_y_bf16, nullptr, T, K, H, (uint16_t *)out_bf16);
 }
