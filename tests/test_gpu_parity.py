@@ -546,6 +546,18 @@ def test_full_size_properties_mixtral_shape(pkg, oracle, dev):
     ss_ref, off_ref, s2r_ref = oracle.permute_counting_sort(ids_ref, E)
     assert torch.equal(ss.cpu(), ss_ref) and torch.equal(off.cpu(), off_ref) and torch.equal(s2r.cpu(), s2r_ref)
     _full_size_checks(pkg, oracle, dev, x, layer, ids, w, torch.tensor([7, 1900, 4095]))
+    # the other batch sizes of the same workload (1, 8, 64, 512 tokens: row tiles of 16, 16, 64 and 64/128 rows):
+    # the first tokens of the big batch on their own give the same bits, in both output forms
+    y = pkg.fused_experts_fp8(x, *layer, ids)
+    out = pkg.fused_experts_fp8(x, *layer, ids, w)
+    for Ts in (1, 8, 64, 512):
+        say("   C2 at T =", Ts)
+        xs, ids_s, w_s = x[:Ts].contiguous(), ids[:Ts].contiguous(), w[:Ts].contiguous()
+        y_s = pkg.fused_experts_fp8(xs, *layer, ids_s)
+        out_s = pkg.fused_experts_fp8(xs, *layer, ids_s, w_s)
+        torch.cuda.synchronize()
+        assert torch.equal(y_s.view(torch.int16), y[:Ts].view(torch.int16))
+        assert torch.equal(out_s.view(torch.int16), out[:Ts].view(torch.int16))
 
 
 def test_full_size_properties_skewed_load(pkg, oracle, dev):
