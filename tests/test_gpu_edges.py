@@ -150,3 +150,31 @@ def test_largest_expert_and_topk_counts(pkg, oracle, dev):
     ref = oracle.moe_w8a8_fp32(x, ids_ref, w_ref, *layer)
     bad = (out.float().cpu() - ref).abs() > 1e-2 + 2e-2 * ref.abs()
     assert bad.float().mean().item() <= 5e-3
+
+
+def test_large_batch_addresses(pkg, oracle, dev):
+    """A batch whose per-slot output is larger than 4 GB (and whose quantised intermediate is close to 1 GB): row
+    addresses must be formed in 64 bits.  Tokens from both ends of the batch equal the same tokens run on their own."""
+    say("large batch")
+    T, H, I, E, K = 150000, 2048, 768, 32, 8
+    gg = torch.Generator(device=dev).manual_seed(77)
+    w13 = (torch.randn(E, 2 * I, H, generator=gg, device=dev) * 0.02).to(torch.bfloat16)
+    w2 = (torch.randn(E, H, I, generator=gg, device=dev) * 0.02).to(torch.bfloat16)
+    w13q, w13s = pkg.quant_weight_block128(w13)
+    w2q, w2s = pkg.quant_weight_block128(w2)
+    del w13, w2
+    x = torch.randn(T, H, generator=gg, device=dev).to(torch.bfloat16)
+    logits = torch.randn(T, E, generator=gg, device=dev)
+    w, ids = pkg.moe_route(logits, K, "softmax")
+    assert T * K * H * 2 > (1 << 32) and T * K * I > (1 << 29)
+    y = pkg.fused_experts_fp8(x, w13q, w13s, w2q, w2s, ids)
+    out = pkg.fused_experts_fp8(x, w13q, w13s, w2q, w2s, ids, w)
+    torch.cuda.synchronize()
+    pick = torch.cat([torch.arange(0, 40), torch.arange(T // 2, T // 2 + 40), torch.arange(T - 40, T)]).to(dev)
+    y_s = pkg.fused_experts_fp8(x[pick].contiguous(), w13q, w13s, w2q, w2s, ids[pick].contiguous())
+    out_s = pkg.fused_experts_fp8(x[pick].contiguous(), w13q, w13s, w2q, w2s, ids[pick].contiguous(), w[pick].contiguous())
+    torch.cuda.synchronize()
+    assert torch.isfinite(y_s.float()).all() and float(y_s.float().abs().max()) > 0
+    assert torch.equal(y[pick].view(torch.int16), y_s.view(torch.int16))
+    assert torch.equal(out[pick].view(torch.int16), out_s.view(torch.int16))
+
