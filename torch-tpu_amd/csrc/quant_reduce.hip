@@ -28,16 +28,27 @@ __global__ __launch_bounds__(256) void weighted_reduce_kernel(const uint16_t *__
   float acc[8];
 #pragma unroll
   for (int i = 0; i < 8; i++) acc[i] = 0.f;
-  for (int k = 0; k < K; k++) {
-    // a slot whose expert id was outside [0, E) has no row: nothing was computed for it and it adds nothing
-    if (slot_to_row != nullptr && slot_to_row[(size_t)t * K + k] < 0) continue;
-    const float wk = w[(size_t)t * K + k];
-    v4i raw = *(const v4i *)(y + ((size_t)t * K + k) * H + c);
+  // eight slots at a time, every load of a group asked for before the first is used.  A slot whose expert id was
+  // outside [0, E) has no row (slot_to_row < 0): nothing was computed for it and it adds nothing.
+  for (int k0 = 0; k0 < K; k0 += 8) {
+    v4i raw[8];
+    float wk[8];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      uint32_t u = (uint32_t)raw[i];
-      acc[2 * i] += wk * bf16_to_f32((uint16_t)(u & 0xffff));
-      acc[2 * i + 1] += wk * bf16_to_f32((uint16_t)(u >> 16));
+    for (int i = 0; i < 8; i++) {
+      const size_t slot = (size_t)t * K + min(k0 + i, K - 1);
+      const bool live = k0 + i < K && (slot_to_row == nullptr || slot_to_row[slot] >= 0);
+      wk[i] = live ? w[slot] : 0.f;
+      raw[i] = *(const v4i *)(y + slot * H + c);
+      if (!live) raw[i] = (v4i){0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const uint32_t u = (uint32_t)raw[i][j];
+        acc[2 * j] += wk[i] * bf16_to_f32((uint16_t)(u & 0xffff));
+        acc[2 * j + 1] += wk[i] * bf16_to_f32((uint16_t)(u >> 16));
+      }
     }
   }
   if (shared_y != nullptr) {
