@@ -57,6 +57,11 @@ def test_argument_errors_are_codes_not_crashes(pkg):
     assert lib.moe_mm_fp8(None, fake, 4, 200, fake, fake, 64, fake, fake, 1 << 20) == E_ALIGN    # K % 128
     assert lib.moe_mm_fp8(None, fake, 4, 256, fake, fake, 8, fake, fake, 1 << 20) == E_SHAPE     # N < 16
     assert lib.moe_mlp_fp8(None, fake, 4, 256, fake, fake, fake, fake, 128, fake, fake, 16) == E_WS
+    # reduction lengths beyond 32768 and activation tensors of 2 GiB or more are refused before anything is launched
+    big = [None, fake, 4, 65536, fake, fake, fake, fake, 128, 8, fake, fake, 2, None, None, None, None, 0, fake, 1, fake, 1 << 40]
+    assert lib.moe_fused_experts_fp8(*big) == E_SHAPE
+    big[2], big[3] = 400000, 7168
+    assert lib.moe_fused_experts_fp8(*big) == E_SHAPE
     assert lib.moe_mm_bf16(None, fake, 4, 200, fake, 64, fake) == E_ALIGN                        # K % 64
     assert lib.moe_mm_bf16(None, fake, 4, 32768, fake, 64, fake) == E_SHAPE                      # K > 16384
     assert lib.moe_mm_bf16(None, fake, 4, 256, None, 64, fake) == E_NULL

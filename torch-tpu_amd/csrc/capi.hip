@@ -142,6 +142,13 @@ static LayerWs layer_layout(void *base, int T, int H, int I, int E, int K, int I
   return d;
 }
 
+// The grouped GEMMs keep one weight-block scale per 128 columns of the reduction in LDS (at most 256 of them) and
+// address their operands with 32-bit per-lane offsets: reduction lengths up to 32768, activation tensors below 2 GiB.
+static bool dims_in_range(int T, int H, int I, int K) {
+  if (H > 32768 || I > 32768) return false;
+  return (double)T * H < 2147483648.0 && (double)T * K * I < 2147483648.0;
+}
+
 }  // namespace moe
 
 extern "C" int moe_hip_version(void) { return 100; }
@@ -178,12 +185,13 @@ extern "C" int moe_fused_experts_fp8(void *stream, const void *x_bf16, int T, in
   if (T != 0 && out_mode == 1 && !routing_weights) return MOE_E_NULL;
   if (T < 0 || H < 1 || I < 1 || E < 1 || E > MOE_MAX_EXPERTS || K < 1 || K > MOE_MAX_TOPK || K > E) return MOE_E_SHAPE;
   if ((long)T * K > (1l << 30)) return MOE_E_SHAPE;
+  if (!dims_in_range(T, H, I, K)) return MOE_E_SHAPE;
   if (H % kBlock || I % kBlock) return MOE_E_ALIGN;
   const bool has_shared = shared_w13 != nullptr;
   if (has_shared) {
     if (out_mode != 1) return MOE_E_MODE;
     if (!shared_w13_scale || !shared_w2 || !shared_w2_scale) return MOE_E_NULL;
-    if (I_shared < 1) return MOE_E_SHAPE;
+    if (I_shared < 1 || !dims_in_range(T, H, I_shared, 1)) return MOE_E_SHAPE;
     if (I_shared % kBlock) return MOE_E_ALIGN;
   }
   const int I_sh = has_shared ? I_shared : 0;
@@ -221,12 +229,13 @@ extern "C" int moe_layer_fp8(void *stream, const void *x_bf16, int T, int H, con
   if (T != 0 && (!x_bf16 || !out_bf16)) return MOE_E_NULL;
   if (T < 0 || H < 1 || I < 1 || E < 1 || E > 256 || K < 1 || K > MOE_MAX_TOPK || K > E) return MOE_E_SHAPE;
   if ((long)T * K > (1l << 30)) return MOE_E_SHAPE;
+  if (!dims_in_range(T, H, I, K)) return MOE_E_SHAPE;
   if (mode != MOE_ROUTE_SOFTMAX && mode != MOE_ROUTE_SIGMOID) return MOE_E_MODE;
   if (H % kBlock || I % kBlock) return MOE_E_ALIGN;
   const bool has_shared = shared_w13 != nullptr;
   if (has_shared) {
     if (!shared_w13_scale || !shared_w2 || !shared_w2_scale) return MOE_E_NULL;
-    if (I_shared < 1) return MOE_E_SHAPE;
+    if (I_shared < 1 || !dims_in_range(T, H, I_shared, 1)) return MOE_E_SHAPE;
     if (I_shared % kBlock) return MOE_E_ALIGN;
   }
   const int I_sh = has_shared ? I_shared : 0;

@@ -726,6 +726,9 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
 // more loads in flight for the bandwidth-bound shapes.
 template <bool GATED, bool BF16 = false>
 static int launch_gemm(hipStream_t st, GemmArgs &a, int tile_m, int max_mtiles) {
+  // the kernel keeps one weight-block scale per 128-step in LDS and forms per-lane operand offsets in 32 bits
+  if (a.Kd < 128 || a.Kd % 128 || (a.Kd >> 7) > kMaxKB) return MOE_E_SHAPE;
+  if ((double)a.rows_a * a.Kd >= 2147483648.0 || (double)a.sh_rows * a.Kd >= 2147483648.0) return MOE_E_SHAPE;
   a.n_strips = GATED ? a.N / 128 : (a.N + 255) / 256;
   a.max_mtiles = max_mtiles - (a.sh_rows + tile_m - 1) / tile_m;
   long total = (long)max_mtiles * a.n_strips;
