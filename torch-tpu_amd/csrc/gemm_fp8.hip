@@ -82,10 +82,10 @@ struct GemmArgs {
 
 constexpr int kMaxKB = 256;                 // reduction length limit: 256 * 128 = 32768
 
-template <int MT, int NW, int STAGES, int WSTAGES, int WTILE = 2048>
+template <int MT, int NW, int STAGES, int WSTAGES, int WTILE = 2048, int TPS = 16>
 struct GemmSmem {
   static constexpr int BM = 16 * MT;
-  alignas(1024) uint8_t wt[WSTAGES][16 * WTILE];   // weight tiles: [tile][row][swizzled 16-byte chunk], read by their owner
+  alignas(1024) uint8_t wt[WSTAGES][TPS * WTILE];   // weight tiles: [tile][row][swizzled 16-byte chunk], read by their owner
   alignas(1024) uint8_t tok[STAGES][BM * 128];   // token tiles, XOR-swizzled 16-byte chunks
   alignas(1024) float sac[2][MT * 256];          // activation scales, 16 steps at a time: [m-tile][4-step part][row][4]
   int arow[BM];                                  // source row in aq / as for each tile row
@@ -136,17 +136,20 @@ __device__ __forceinline__ void mma_bf16(v4f (&acc)[WT], const v8i (&w)[WT], con
 }
 
 // MT     token m-tiles (of 16 rows) per workgroup
-// NW     wavefronts per workgroup (4 or 8); each owns WT = 16 / NW of the strip's 16 weight tiles
+// NW     wavefronts per workgroup (4 or 8); each owns WT = TPS / NW of the strip's weight tiles
+// TPS    weight tiles (of 16 rows) per strip: 16, or 4 for the second GEMM of a batch that would leave most
+//        of the chip without a strip (narrow strips of 64 output columns; every sum keeps its order)
 // DEPTH  128-steps of weights kept in flight per wavefront (register ring)
 // BF16   un-quantised mode: both operands are bf16 (a 128-byte step is 64 elements = two
 //        v_mfma_f32_16x16x32_bf16 accumulating in place), no scales, bf16 intermediate
-template <int MT, int NW, int DEPTH, bool GATED, bool WREG, bool BF16 = false>
+template <int MT, int NW, int DEPTH, bool GATED, bool WREG, bool BF16 = false, int TPS = 16>
 __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a) {
+  static_assert(TPS % NW == 0 && (TPS == 16 || (!GATED && !WREG && TPS <= 8)), "narrow strips: second GEMM, operands through LDS");
   constexpr int BM = 16 * MT;
   constexpr int NT = 64 * NW;                         // threads
-  constexpr int WT = 16 / NW;                         // weight tiles per wavefront
+  constexpr int WT = TPS / NW;                        // weight tiles per wavefront
   constexpr int STAGES = WREG ? 4 : DEPTH + 1;        // token tiles staged in LDS
-  using Smem = GemmSmem<MT, NW, STAGES, WREG ? 1 : STAGES, WREG ? 64 : 2048>;
+  using Smem = GemmSmem<MT, NW, STAGES, WREG ? 1 : STAGES, WREG ? 64 : 2048, TPS>;
   static_assert(sizeof(Smem) <= 160 * 1024, "one workgroup's LDS");
   __shared__ Smem sm;
 
@@ -244,7 +247,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   for (int j = 0; j < WT; j++) {
     int wrow;
     if (GATED) wrow = (j < WT / 2 ? 0 : a.N) + strip * 128 + wave * (8 * WT) + (j % (WT / 2)) * 16;
-    else wrow = strip * 256 + wave * (16 * WT) + j * 16;
+    else wrow = strip * (16 * TPS) + wave * (16 * WT) + j * 16;
     wrow = min(wrow, a.n_rows_w - 16);                 // tiles past the matrix re-read its last rows
     wtile[j] = wq + ((size_t)e * a.n_rows_w + wrow) * a.Kd;
   }
@@ -258,8 +261,9 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   constexpr int NSB = (2 * kMaxKB + NT - 1) / NT;
   float sbv[NSB];
   if constexpr (!BF16) {
-    const int blk0 = GATED ? strip : min(strip * 2, n_wblk - 1);
-    const int blk1 = GATED ? (a.N >> 7) + strip : min(strip * 2 + 1, n_wblk - 1);
+    // second GEMM: the 128-row blocks the strip's first and ninth tile lie in (a narrow strip lies in one)
+    const int blk0 = GATED ? strip : min(strip * TPS / 8, n_wblk - 1);
+    const int blk1 = GATED ? (a.N >> 7) + strip : min(strip * TPS / 8 + 1, n_wblk - 1);
 #pragma unroll
     for (int u = 0; u < NSB; u++) {
       const int i = tid + u * NT, r = i >= NKB, kb = i - r * NKB;
@@ -316,7 +320,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     sac_m0[u] = mt * 1024;
   }
   const uint32_t wt_base = __builtin_amdgcn_readfirstlane(lds_offset(&sm.wt[0][0])) + wave * (WT * 2048);
-  constexpr uint32_t kWtStage = 16 * 2048;
+  constexpr uint32_t kWtStage = TPS * 2048;
   const uint32_t tok_base = __builtin_amdgcn_readfirstlane(lds_offset(&sm.tok[0][0]));
   const uint32_t sac_base = __builtin_amdgcn_readfirstlane(lds_offset(&sm.sac[0][0]));
   constexpr uint32_t kTokStage = BM * 128, kSacBuf = MT * 1024;
@@ -631,7 +635,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   // A lane holds 4 neighbouring columns of a row: stored from the registers, one instruction would touch 16 rows with
   // a few bytes each.  The tile is laid down in LDS instead (the operand stages are idle now: every load has landed
   // and the barrier above has passed) and streamed out in whole rows, 16 bytes per lane.
-  constexpr int RB = GATED ? (BF16 ? 256 : 128) : 512;         // bytes of one output row inside this strip
+  constexpr int RB = GATED ? (BF16 ? 256 : 128) : 32 * TPS;    // bytes of one output row inside this strip
   constexpr int RS = RB + (RB == 128 ? 16 : 32);               // row pitch in LDS: the lanes of a write hit different banks
   static_assert(offsetof(Smem, arow) >= (size_t)BM * RS, "the staged output tile overlays the operand stages only");
   uint8_t *const stage = (uint8_t *)&sm;
@@ -713,7 +717,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     uint8_t *const out = GATED ? (shared ? a.sh_hq : a.hq) : (uint8_t *)(shared ? a.sh_y : a.y);
     const size_t row_bytes = (size_t)a.N * (GATED && !BF16 ? 1 : 2);
     // second GEMM: a strip is 256 columns, the matrix may end inside it (its width is a multiple of 8 columns)
-    const bool in_width = GATED || strip * 256 + piece * 8 < a.N;
+    const bool in_width = GATED || strip * (16 * TPS) + piece * 8 < a.N;
     for (int r = wave * RPI + lane / PIECES; r < rows; r += NW * RPI) {
       const v4i d = *(const v4i *)(stage + r * RS + piece * 16);
       const size_t orow = GATED ? (size_t)(row0 + r) : (size_t)sm.oslot[r];
@@ -729,7 +733,12 @@ static int launch_gemm(hipStream_t st, GemmArgs &a, int tile_m, int max_mtiles) 
   // the kernel keeps one weight-block scale per 128-step in LDS and forms per-lane operand offsets in 32 bits
   if (a.Kd < 128 || a.Kd % 128 || (a.Kd >> 7) > kMaxKB) return MOE_E_SHAPE;
   if ((double)a.rows_a * a.Kd >= 2147483648.0 || (double)a.sh_rows * a.Kd >= 2147483648.0) return MOE_E_SHAPE;
-  a.n_strips = GATED ? a.N / 128 : (a.N + 255) / 256;
+  // Second GEMM with small row tiles: strips of 64 output columns instead of 256 - four times the workgroups,
+  // three of them resident per compute unit, so that one's start and end hide behind the others' streams (and a
+  // batch with few experts still reaches every compute unit: a workgroup alone streams at most ~37 GB/s).  The
+  // order of every sum is the same.  With 64-row tiles it only pays while the wide strips would leave units idle.
+  const bool narrow = !GATED && (tile_m <= 32 || (tile_m == 64 && (long)max_mtiles * ((a.N + 255) / 256) < 192));
+  a.n_strips = GATED ? a.N / 128 : narrow ? (a.N + 63) / 64 : (a.N + 255) / 256;
   a.max_mtiles = max_mtiles - (a.sh_rows + tile_m - 1) / tile_m;
   long total = (long)max_mtiles * a.n_strips;
   total = (total + 7) / 8 * 8 + 16;                  // the per-XCD split rounds two shares up
@@ -739,6 +748,18 @@ static int launch_gemm(hipStream_t st, GemmArgs &a, int tile_m, int max_mtiles) 
 #define MOE_GEMM(MT, NW, D, WREG) grouped_gemm_kernel<MT, NW, D, GATED, WREG, BF16><<<grid, dim3(64 * NW), 0, st>>>(a)
   // small tiles: both operands through LDS (few registers, deeper pipeline); large tiles: weights in
   // a register ring so that LDS holds three stages of the bigger token tile
+  if constexpr (!GATED) {
+    if (narrow) {
+#define MOE_GEMM_NARROW(MT, D) grouped_gemm_kernel<MT, 4, D, false, false, BF16, 4><<<grid, dim3(256), 0, st>>>(a)
+      switch (tile_m) {
+        case 16: MOE_GEMM_NARROW(1, 3); break;
+        case 32: MOE_GEMM_NARROW(2, 3); break;
+        default: MOE_GEMM_NARROW(4, 2); break;
+      }
+#undef MOE_GEMM_NARROW
+      return (int)hipGetLastError();
+    }
+  }
   switch (tile_m) {
     case 16: MOE_GEMM(1, 8, 3, false); break;
     case 32: MOE_GEMM(2, 8, 3, false); break;
