@@ -32,7 +32,8 @@
 //   W13; wavefront w owns gate columns 16w..16w+15 and the same up columns.  Epilogue:
 //   h = silu(gate) * up, per-token amax over the strip's 128 columns (registers -> lane
 //   butterflies -> LDS across the wavefronts), scale = max(amax, 1e-10) / 448, h * (1 / scale) -> e4m3fn.
-// GATED = false (second GEMM): the strip is 256 output columns, wavefront w owns 32 of them;
+// GATED = false (second GEMM): the strip is 256 output columns, wavefront w owns 32 of them (with small
+//   row tiles: 64 output columns, four wavefronts with 16 each - more, smaller workgroups, same sums);
 //   the bf16 result row is written at its slot (t*K + k), which undoes the permutation.
 // Both epilogues lay the output tile down in LDS and store it in whole rows.
 #include <cstddef>
