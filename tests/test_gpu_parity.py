@@ -189,7 +189,7 @@ def test_permutation_skewed_with_empty_experts(pkg, oracle, dev):
 # checks below therefore prove parity in two strict steps plus one end-to-end figure:
 #   (1) first GEMM + SwiGLU + re-quantisation: every device code is within one e4m3 step of
 #       the oracle's (plus the sums' absolute error for near-zero elements), and all but a sliver
-#       are identical; scales agree to 1e-4;
+#       are identical; scales agree to 5e-4;
 #   (2) second GEMM + un-permute (+ weighted reduce): strict rtol 2e-2 / atol 1e-2, ALL
 #       elements, against the oracle run on the very codes the device produced;
 #   (3) end to end against the oracle's own codes: the share of elements outside
@@ -226,7 +226,9 @@ def check_experts(pkg, oracle, dev, x, layer, ids, w, shared=None):
     hq_dev[slot] = hq.cpu().view(torch.uint8)
     hs_dev[slot] = hs.cpu()
     hq_r, hs_r = hq_ref.reshape(T * K, I), hs_ref.reshape(T * K, -1)
-    assert torch.allclose(hs_dev, hs_r, rtol=1e-4, atol=0)
+    # a scale is the largest |h| of 128 columns / 448: it carries the matrix instruction's summation error of that one
+    # element (up to 2^-11.8 = 2.8e-4 of the largest product, measured), most visibly where the reduction is short
+    assert torch.allclose(hs_dev, hs_r, rtol=5e-4, atol=0)
     v_dev = hq_dev.view(torch.float8_e4m3fn).float()
     v_ref = hq_r.view(torch.float8_e4m3fn).float()
     # one grid step, or (for elements far below the group maximum, where the grid is finer than the
