@@ -497,6 +497,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
       constexpr int LIVE = decltype(live_c)::value;
       static_assert(LIVE % 2 == 0 && LIVE >= 2 && LIVE <= MT, "live m-tiles come in pairs");
       constexpr int PD = 2;                              // m-tiles between an LDS read and its use
+      const bool top_empty = mt_live < LIVE;             // uniform: the top m-tile of the top pair holds no row
       // the first requests go out inside the instantiation: no branch may sit between a register
       // load's request and its wait (the compiler would copy the registers while the load is in flight)
       request(0, 0);
@@ -564,8 +565,10 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
             {
               const int qq = q + PD < LIVE ? q + PD : q + PD - LIVE;
               const int kk = q + PD < LIVE ? kb : kb + 1;
-              x[(g + PD) % XB] = read_x(kk, LIVE - 1 - qq);
-              fb[(g + PD) % XB] = read_f(kk, LIVE - 1 - qq);
+              if (qq != 0 || !top_empty) {               // nothing to read for a top m-tile without a row
+                x[(g + PD) % XB] = read_x(kk, LIVE - 1 - qq);
+                fb[(g + PD) % XB] = read_f(kk, LIVE - 1 - qq);
+              }
             }
             // the token tile of step kb + 3 goes into the stage that step kb - 1 used, one piece with each of a few
             // m-tiles: all wavefronts asking for everything at the step boundary queued up behind one another
@@ -576,24 +579,31 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
             // the matrix pipe has work, instead of at the boundary, where every wavefront stands still
             if (q == LIVE / 2) produce_f(kb + 3);
             if constexpr (BF16) {                        // accumulates in place: nothing is pending afterwards
-              mma_bf16<WT>(acc[LIVE - 1 - q], wc, x[g % XB]);
+              if (q != 0 || !top_empty) mma_bf16<WT>(acc[LIVE - 1 - q], wc, x[g % XB]);
               __builtin_amdgcn_sched_barrier(0);
               return;
             }
+            // Live m-tiles come in pairs; when the rows end in the lower one of the top pair, the top m-tile (the
+            // first of the walk) has no row: its matrix instructions are left out, like its operand reads and the
+            // multiply-adds that would fold its products in; the epilogue never looks at its accumulator.
+            if (q != 0 || !top_empty) {
 #pragma unroll
-            for (int j = 0; j < WT; j++) {
-              const v4f zero = {0.f, 0.f, 0.f, 0.f};
-              p[g & 1][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wc[j], x[g % XB], zero, 0, 0, 0, 0, 0, 0);
+              for (int j = 0; j < WT; j++) {
+                const v4f zero = {0.f, 0.f, 0.f, 0.f};
+                p[g & 1][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wc[j], x[g % XB], zero, 0, 0, 0, 0, 0, 0);
+              }
             }
             __builtin_amdgcn_sched_barrier(0);
+            if (q != 1 || !top_empty) {                  // the m-tile before this one was the empty top one: no products
 #pragma unroll
-            for (int j = 0; j < WT; j++) {
-              const float f = (GATED && j >= WT / 2) ? fb[(g + XB - 1) % XB].y : fb[(g + XB - 1) % XB].x;
+              for (int j = 0; j < WT; j++) {
+                const float f = (GATED && j >= WT / 2) ? fb[(g + XB - 1) % XB].y : fb[(g + XB - 1) % XB].x;
 #pragma unroll
-              for (int r = 0; r < 4; r++) acc[tp][j][r] = fmaf(p[(g + 1) & 1][j][r], f, acc[tp][j][r]);
-              // pins the multiply-adds here: without it they are sunk below the whole step's matrix
-              // instructions, whose results then all stay live
-              asm volatile("" : "+v"(acc[tp][j]));
+                for (int r = 0; r < 4; r++) acc[tp][j][r] = fmaf(p[(g + 1) & 1][j][r], f, acc[tp][j][r]);
+                // pins the multiply-adds here: without it they are sunk below the whole step's matrix
+                // instructions, whose results then all stay live
+                asm volatile("" : "+v"(acc[tp][j]));
+              }
             }
             __builtin_amdgcn_sched_barrier(0);
           };
