@@ -410,37 +410,45 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
       if (mg == 0 || mg * MG < mt_live) {
         v8i x[MG];
         float sa_[MG];
+        // m-tiles of the group that hold no row (the first of a group always does) are left out one by one
 #pragma unroll
         for (int mi = 0; mi < MG; mi++) {
           const int mt = mg * MG + mi;
-          x[mi] = concat8(*(const v4i *)(tbase + mt * 2048 + o0), *(const v4i *)(tbase + mt * 2048 + o1));
-          sa_[mi] = BF16 ? 0.f : sap[mt * 256];
+          if (mi == 0 || mt < mt_live) {
+            x[mi] = concat8(*(const v4i *)(tbase + mt * 2048 + o0), *(const v4i *)(tbase + mt * 2048 + o1));
+            sa_[mi] = BF16 ? 0.f : sap[mt * 256];
+          }
         }
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (BF16) {
 #pragma unroll
-          for (int mi = 0; mi < MG; mi++) mma_bf16<WT>(acc[mg * MG + mi], wc, x[mi]);
+          for (int mi = 0; mi < MG; mi++)
+            if (mi == 0 || mg * MG + mi < mt_live) mma_bf16<WT>(acc[mg * MG + mi], wc, x[mi]);
           __builtin_amdgcn_sched_barrier(0);
           continue;
         }
         v4f p[MG][WT];
 #pragma unroll
         for (int mi = 0; mi < MG; mi++) {
+          if (mi == 0 || mg * MG + mi < mt_live) {
 #pragma unroll
-          for (int j = 0; j < WT; j++) {
-            const v4f zero = {0.f, 0.f, 0.f, 0.f};
-            p[mi][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wc[j], x[mi], zero, 0, 0, 0, 0, 0, 0);
+            for (int j = 0; j < WT; j++) {
+              const v4f zero = {0.f, 0.f, 0.f, 0.f};
+              p[mi][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wc[j], x[mi], zero, 0, 0, 0, 0, 0, 0);
+            }
           }
         }
 #pragma unroll
         for (int mi = 0; mi < MG; mi++) {
           const int mt = mg * MG + mi;
-          const float f0 = sa_[mi] * s0, f1 = sa_[mi] * s1;
+          if (mi == 0 || mt < mt_live) {
+            const float f0 = sa_[mi] * s0, f1 = sa_[mi] * s1;
 #pragma unroll
-          for (int j = 0; j < WT; j++) {
-            const float f = (GATED && j >= WT / 2) ? f1 : f0;
+            for (int j = 0; j < WT; j++) {
+              const float f = (GATED && j >= WT / 2) ? f1 : f0;
 #pragma unroll
-            for (int r = 0; r < 4; r++) acc[mt][j][r] = fmaf(p[mi][j][r], f, acc[mt][j][r]);
+              for (int r = 0; r < 4; r++) acc[mt][j][r] = fmaf(p[mi][j][r], f, acc[mt][j][r]);
+            }
           }
         }
         __builtin_amdgcn_sched_barrier(0);
