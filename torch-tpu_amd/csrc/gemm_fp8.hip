@@ -655,7 +655,10 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   // a few bytes each.  The tile is laid down in LDS instead (the operand stages are idle now: every load has landed
   // and the barrier above has passed) and streamed out in whole rows, 16 bytes per lane.
   constexpr int RB = GATED ? (BF16 ? 256 : 128) : 32 * TPS;    // bytes of one output row inside this strip
-  constexpr int RS = RB + (RB == 128 ? 16 : 32);               // row pitch in LDS: the lanes of a write hit different banks
+  // row pitch in LDS: the lanes of a write hit different banks.  16 rows x 4 dwords (RB = 128, a dword per lane) or
+  // 16 rows x 2 lane groups x 2 dwords (a half-wavefront of 8-byte writes) must spread over the 64 banks: a pitch of
+  // 4 dwords modulo 64.
+  constexpr int RS = RB + 16;
   static_assert(offsetof(Smem, arow) >= (size_t)BM * RS, "the staged output tile overlays the operand stages only");
   uint8_t *const stage = (uint8_t *)&sm;
   if (GATED && BF16) {
