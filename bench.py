@@ -407,11 +407,30 @@ def main():
             omoe = build_layer(pkg, ocfg, dev)
             osec, oroof, _ = bench_prefill(pkg, omoe, ocfg, dev, args.steps, args.warmup)
             oflops = gemm_flops(ocfg, ocfg["T"])
-            others.append(dict(workload=f"{name}: {ocfg['desc']}", ms_per_step=osec * 1e3, tflops=oflops / osec / 1e12,
-                               mfma_frac_of_peak=oflops / osec / 1e12 / PEAK_FP8_TFLOPS,
-                               tokens_per_s=ocfg["T"] / osec, first_gemm_ms=oroof["launch_ms"],
-                               first_gemm_tflops=oroof["mfma_tflops"], second_gemm_ms=oroof["second_gemm"]["launch_ms"],
-                               second_gemm_tflops=oroof["second_gemm"]["mfma_tflops"]))
+            rec = dict(workload=f"{name}: {ocfg['desc']}", ms_per_step=osec * 1e3, tflops=oflops / osec / 1e12,
+                       mfma_frac_of_peak=oflops / osec / 1e12 / PEAK_FP8_TFLOPS,
+                       tokens_per_s=ocfg["T"] / osec, first_gemm_ms=oroof["launch_ms"],
+                       first_gemm_tflops=oroof["mfma_tflops"], second_gemm_ms=oroof["second_gemm"]["launch_ms"],
+                       second_gemm_tflops=oroof["second_gemm"]["mfma_tflops"])
+            if name == "c2_prefill":
+                # the same few-expert layer at decode sizes: bytes of the experts a batch touches per second
+                small = []
+                for Ts in (1, 8, 64):
+                    g = torch.Generator(device=dev).manual_seed(300 + Ts)
+                    pool = [torch.randn(Ts, ocfg["H"], generator=g, device=dev).to(torch.bfloat16) for _ in range(8)]
+                    outs_ = torch.empty(Ts, ocfg["H"], dtype=torch.bfloat16, device=dev)
+                    state = {"i": 0}
+
+                    def small_step():
+                        omoe(pool[state["i"] % len(pool)], out=outs_)
+                        state["i"] += 1
+
+                    ssec = time_steps(small_step, max(args.steps, 32), max(args.warmup, 16))
+                    touched = sum(int(torch.unique(omoe.route(xp)[1]).numel()) for xp in pool) / len(pool)
+                    small.append(dict(T=Ts, ms_per_step=ssec * 1e3, experts_touched_avg=touched,
+                                      weight_gbs=touched * expert_bytes(ocfg["H"], ocfg["I"]) / ssec / 1e9))
+                rec["decode_sizes"] = small
+            others.append(rec)
             del omoe
         result["other_shapes"] = others
     if not args.no_cpu:
