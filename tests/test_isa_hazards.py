@@ -56,3 +56,22 @@ def test_gemm_kernels_have_no_scratch_and_no_in_flight_register_use(gemm_asm):
         assert "s_waitcnt vmcnt" in body and "global_load_lds_dwordx4" in body
         bad = hazards(body)
         assert not bad, f"{name}: {bad[:5]}"
+
+
+@pytest.mark.parametrize("source", ["route.hip", "permute.hip", "quant_reduce.hip", "dense_small.hip", "decode_prep.hip",
+                                    "router_front.hip"])
+def test_no_kernel_of_the_library_spills(source, tmp_path):
+    """Every other kernel source: compiled to gfx950 assembly, no kernel may need scratch memory."""
+    hipcc = "/opt/rocm/bin/hipcc" if os.path.exists("/opt/rocm/bin/hipcc") else "hipcc"
+    out = tmp_path / (source + ".s")
+    cmd = [hipcc, "--offload-arch=gfx950", "--cuda-device-only", "-O3", "-std=c++17", "-S", "-Wno-inline-asm",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           os.path.join(ROOT, "torch-tpu_amd", "csrc", source), "-o", str(out)]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        pytest.fail("hipcc failed:\n" + r.stdout[-2000:])
+    sizes = scratch_bytes(out.read_text())
+    assert sizes, "no kernel found"
+    spills = {n: b for n, b in sizes.items() if b}
+    assert not spills, f"kernels spill to scratch: {spills}"
+
