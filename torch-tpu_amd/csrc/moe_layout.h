@@ -26,10 +26,10 @@ static inline int choose_tile_m(int T, int K, int E) {
   // that holds a typical expert whole.
   // Up to ~48 rows per expert the 64-row tile wins although a few experts then need two tiles: its
   // kernel keeps both operands in LDS and fetches the weights in whole cache lines (measured on the
-  // DeepSeek-V3 shape: 64 best up to T=1536, 128 up to T=3072, 192 above).
+  // DeepSeek-V3 shape: 64 best up to T=1536, 128 at T=2048, 192 from T=3072 on).
   const double mean = (double)T * K / E;
   if (mean <= 48.0) return 64;
-  return mean > 96.0 ? 192 : 128;
+  return mean > 84.0 ? 192 : 128;
 }
 
 struct PermuteWs {
