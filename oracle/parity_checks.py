@@ -1,0 +1,182 @@
+"""Parity checks of the HIP path against the CPU oracle at FULL layer size, on a sample of tokens.
+
+TEST INFRASTRUCTURE ONLY (like moe_oracle.py): imported by tests/, by __graft_entry__.smoke() and by
+bench.py's CPU-baseline leg.  The package under test is handed in as an argument; nothing here is used by it.
+
+The criterion is rtol 2e-2 / atol 1e-2 against the oracle's fp32 arithmetic on the same quantised operands.
+Between the two GEMMs the SwiGLU output is re-quantised to e4m3, and the FP8 matrix instruction's sums differ
+from fp32 sums in the 4th-5th digit, so an element that sits on an e4m3 rounding boundary can land on the
+neighbouring code on the device.  A fraction allowance alone ("at most x % of the outputs outside") would also
+pass a kernel that corrupts a few rows, so the comparison is made in strict steps instead:
+
+  (0) quantised activations: bit-exact;
+  (1) re-quantised SwiGLU output: every device code within ONE e4m3 step of the oracle's, >= 99 % identical,
+      scales within 5e-4;
+  (2) second GEMM: EVERY element of the per-slot results (the reference op's output form, [T,K,H]) within
+      rtol 2e-2 / atol 1e-2 of the oracle evaluated on the codes the device produced; the weighted sum over the
+      slots (+ shared expert): every element within atol + rtol * (sum of the terms' magnitudes) - the plain
+      tolerance wherever the terms do not cancel - and exactly the fp32 weighted sum of the device's slot results;
+  (3) end to end against the oracle's own codes: reported (fraction outside, worst violation) and bounded.
+      (1) and (2) together bound it: the two oracle results differ by (code differences) x W2, one step each.
+
+A token's bits do not depend on the batch it arrives in (asserted where a big batch's rows are passed in), so
+the staged kernels on the sampled tokens, with the full-size weights, stand for the big batch.
+"""
+from __future__ import annotations
+
+import torch
+
+RTOL, ATOL = 2e-2, 1e-2
+# end-to-end caps against the oracle's own codes, with (1) and (2) holding: share of elements outside the
+# tolerance, and the worst |got - ref| / (atol + rtol |ref|).  One e4m3 step (1/8 relative at most) on a handful
+# of a row's I elements moves an output by a few atol at most; measured <= 0.2 % and <= 4.
+MAX_OUTSIDE = 5e-3
+MAX_WORST = 12.0
+
+
+def outside_fraction(got: torch.Tensor, ref: torch.Tensor) -> float:
+    return ((got - ref).abs() > ATOL + RTOL * ref.abs()).float().mean().item()
+
+
+def worst_violation(got: torch.Tensor, ref: torch.Tensor) -> float:
+    """max |got - ref| / (atol + rtol |ref|): <= 1 means every element is within tolerance."""
+    if got.numel() == 0:
+        return 0.0
+    return ((got - ref).abs() / (ATOL + RTOL * ref.abs())).max().item()
+
+
+def assert_all_within(got: torch.Tensor, ref: torch.Tensor, what: str):
+    w = worst_violation(got, ref)
+    assert w <= 1.0, f"{what}: worst |got-ref|/(atol+rtol|ref|) = {w:.3f} > 1"
+    return w
+
+
+def assert_codes_within_one_step(oracle, hq_dev, hs_dev, hq_ref, hs_ref, what: str) -> float:
+    """(1): hq_* uint8 [rows, I], hs_* fp32 [rows, I/128], rows in the same order.  Returns the identical share."""
+    assert torch.allclose(hs_dev, hs_ref, rtol=5e-4, atol=0), f"{what}: a re-quantisation scale is off"
+    v_dev = hq_dev.view(torch.float8_e4m3fn).float()
+    v_ref = hq_ref.view(torch.float8_e4m3fn).float()
+    assert torch.isfinite(v_dev).all(), f"{what}: NaN code"
+    # one grid step, or (for elements far below the group maximum, where the grid is finer than the fp32 sums'
+    # absolute error) 1.4e-4 of the group maximum = 1/16 in units of the scale
+    ok = (v_dev - v_ref).abs() <= oracle.e4m3_step(hq_ref) + 0.0625
+    assert ok.all(), f"{what}: {int((~ok).sum())} re-quantised codes are more than one e4m3 step off"
+    same = (hq_dev == hq_ref).float().mean().item() if hq_dev.numel() else 1.0
+    assert same >= 0.99, f"{what}: only {same:.4f} of the re-quantised codes match"
+    return same
+
+
+def _localise(ids_host: torch.Tensor):
+    """Expert ids of a sample -> (ids renumbered 0..n_used-1, the used expert ids): only those experts' weights
+    have to come to the host."""
+    used = torch.unique(ids_host).tolist()
+    remap = {int(e): i for i, e in enumerate(used)}
+    local = torch.tensor([[remap[int(e)] for e in row] for row in ids_host.tolist()], dtype=torch.int32)
+    return local.reshape(ids_host.shape), used
+
+
+def staged_experts(pkg, x_s, ids_s, layer_dev):
+    """The staged kernels through the C ABI on a (small) batch: -> y [n,K,H] bf16 (slot order), and the device's
+    re-quantised SwiGLU codes / scales in slot order (uint8 [n*K, I], fp32 [n*K, I/128]) plus xq, xs."""
+    n, K = ids_s.shape
+    w13, w13s, w2, w2s = layer_dev
+    E, _, I = w2.shape
+    xq, xs = pkg.act_quant(x_s)
+    ss, off, s2r, ws = pkg.moe_permute(ids_s, E, return_workspace=True)
+    hq, hs = pkg.gemm1_swiglu(xq, xs, w13, w13s, (n, K), ss, off, ws)
+    y = pkg.gemm2(hq, hs, w2, w2s, (n, K), ss, off, ws)
+    torch.cuda.synchronize()
+    slot = ss.cpu().long()
+    hq_dev = torch.empty(n * K, I, dtype=torch.uint8)
+    hs_dev = torch.empty(n * K, I // 128, dtype=torch.float32)
+    hq_dev[slot] = hq.cpu().view(torch.uint8)
+    hs_dev[slot] = hs.cpu()
+    return y, hq_dev, hs_dev, xq, xs
+
+
+def check_sample(pkg, oracle, x_s, ids_s, layer_dev, w_s=None, shared_dev=None, y_big=None, out_big=None,
+                 what: str = "sample", unit: float = 1.0):
+    """Steps (0)-(3) on a sample of tokens, with the full-size weights on the device.
+
+    x_s [n,H] bf16, ids_s [n,K] int32, w_s [n,K] fp32 (all on the device); layer_dev / shared_dev the packed
+    weights on the device (shared: leading dimension 1).  y_big [n,K,H]: the sampled tokens' per-slot rows out of
+    a bigger batch - must equal the staged result bit for bit.  out_big [n,H]: their rows of a weighted (+ shared)
+    output out of a bigger batch - must equal the device's weighted sum of the staged results bit for bit.
+    unit: outputs are compared in this unit (the tolerance's atol is an absolute number made for outputs of
+    order one; a layer whose outputs are of another order hands in their magnitude).
+    Returns a report dict; raises AssertionError when a step fails."""
+    n, K = ids_s.shape
+    H = x_s.shape[1]
+    I = layer_dev[2].shape[2]
+    rep = {"tokens_checked": n}
+    y, hq_dev, hs_dev, xq, xs = staged_experts(pkg, x_s, ids_s, layer_dev)
+    if y_big is not None:
+        assert torch.equal(y.view(torch.int16), y_big.view(torch.int16)), f"{what}: a token's slot results depend on its batch"
+    ids_host = ids_s.cpu()
+    local, used = _localise(ids_host)
+    idx = torch.tensor(used, device=x_s.device)
+    small = tuple(t[idx].cpu() for t in layer_dev)
+    x_host = x_s.cpu()
+    ref, (xq_ref, xs_ref, hq_ref, hs_ref) = oracle.experts_w8a8_fp32(x_host, local, *small, return_mid=True)
+    # (0)
+    assert torch.equal(xq.cpu().view(torch.uint8), xq_ref.view(torch.uint8)) and torch.equal(xs.cpu(), xs_ref), \
+        f"{what}: quantised activations differ"
+    # (1)
+    rep["codes_identical"] = assert_codes_within_one_step(oracle, hq_dev, hs_dev, hq_ref.reshape(n * K, I),
+                                                          hs_ref.reshape(n * K, -1), what + " routed")
+    # (2)
+    y_mid = oracle.experts_w8a8_fp32(x_host, local, *small, mid=(hq_dev.reshape(n, K, I), hs_dev.reshape(n, K, -1))) / unit
+    got = y.float().cpu() / unit
+    ref = ref / unit
+    rep["worst_given_device_codes"] = assert_all_within(got, y_mid, what + " second GEMM on the device's codes")
+    # (3)
+    rep["outside_per_slot"] = outside_fraction(got, ref)
+    rep["worst_per_slot"] = worst_violation(got, ref)
+    rep["cos_diff"] = oracle.cal_diff(ref, got)[0]
+    if w_s is not None:
+        sh_y = sh_mid = sh_ref = None
+        if shared_dev is not None:
+            zeros = torch.zeros(n, 1, dtype=torch.int32, device=x_s.device)
+            sh_y, sh_hq, sh_hs, _, _ = staged_experts(pkg, x_s, zeros, shared_dev)
+            sh_host = tuple(t.cpu() for t in shared_dev)
+            I_sh = shared_dev[2].shape[2]
+            z = zeros.cpu()
+            sh_ref, (_, _, shq_ref, shs_ref) = oracle.experts_w8a8_fp32(x_host, z, *sh_host, return_mid=True)
+            rep["shared_codes_identical"] = assert_codes_within_one_step(
+                oracle, sh_hq, sh_hs, shq_ref.reshape(n, I_sh), shs_ref.reshape(n, -1), what + " shared")
+            sh_mid = oracle.experts_w8a8_fp32(x_host, z, *sh_host, mid=(sh_hq.reshape(n, 1, I_sh), sh_hs.reshape(n, 1, -1)))
+            assert_all_within(sh_y.float().cpu() / unit, sh_mid / unit, what + " shared second GEMM on the device's codes")
+            sh_y, sh_mid, sh_ref = sh_y[:, 0].contiguous(), sh_mid[:, 0] / unit, sh_ref[:, 0] / unit
+        out = pkg.weighted_reduce(y, w_s, sh_y)
+        torch.cuda.synchronize()
+        if out_big is not None:
+            assert torch.equal(out.view(torch.int16), out_big.view(torch.int16)), \
+                f"{what}: the big batch's output rows differ from the staged kernels on the same tokens"
+        w_host = w_s.cpu()
+        # the weighted sum of the device's own bf16 slot results (+ its shared rows): only the sum is under test
+        red_dev = oracle.weighted_reduce(got, w_host)
+        red_mid = oracle.weighted_reduce(y_mid, w_host)
+        red_ref = oracle.weighted_reduce(ref, w_host)
+        if shared_dev is not None:
+            red_dev, red_mid, red_ref = red_dev + sh_y.float().cpu() / unit, red_mid + sh_mid, red_ref + sh_ref
+        o = out.float().cpu() / unit
+        assert_all_within(o, red_dev, what + " weighted sum of the device's slot results")
+        # The output is a sum of K (+1) terms, each a bf16 per-slot result (the reference op's own output form) that
+        # step (2) held to the tolerance.  A sum whose terms cancel cannot be held to rtol of its own, smaller,
+        # magnitude: the bound that the terms' tolerances imply is atol + rtol * (sum of the terms' magnitudes), the
+        # plain tolerance wherever the terms do not cancel.  Every element must meet it; the plain figure is reported.
+        mag = torch.einsum("tk,tkh->th", w_host.abs(), y_mid.abs())
+        if shared_dev is not None:
+            mag = mag + sh_mid.abs()
+        excess = ((o - red_mid).abs() / (ATOL + RTOL * mag)).max().item()
+        assert excess <= 1.0, f"{what} output on the device's codes: worst |got-ref|/(atol+rtol*sum|terms|) = {excess:.3f} > 1"
+        rep["worst_reduced_given_device_codes"] = worst_violation(o, red_mid)
+        rep["outside_reduced"] = outside_fraction(o, red_ref)
+        rep["worst_reduced"] = worst_violation(o, red_ref)
+        rep["cos_diff_reduced"] = oracle.cal_diff(red_ref, o)[0]
+    for k in ("outside_per_slot", "outside_reduced"):
+        assert rep.get(k, 0.0) <= MAX_OUTSIDE, f"{what}: {k} = {rep[k]:.2e}"
+    for k in ("worst_per_slot", "worst_reduced"):
+        assert rep.get(k, 0.0) <= MAX_WORST, f"{what}: {k} = {rep[k]:.2f}"
+    assert rep["cos_diff"] < 1e-5, f"{what}: cos_diff {rep['cos_diff']:.2e}"
+    return rep

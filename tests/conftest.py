@@ -21,6 +21,11 @@ def oracle():
 
 
 @pytest.fixture(scope="session")
+def checks():
+    return entry.load_parity_checks()
+
+
+@pytest.fixture(scope="session")
 def pkg():
     """The package under test; importing it loads libmoe_hip.so and fails loudly if absent."""
     return entry.load_package()

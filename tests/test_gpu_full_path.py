@@ -1,0 +1,126 @@
+"""The paths the benchmark times, at their real sizes, against the CPU oracle, through the C ABI on a real MI355X:
+
+  * the DeepSeek-V3-shaped layer at T=4096 through the one-call entry point - router product on the matrix
+    cores, 192-row tiles, the shared expert's tiles riding in the routed launches;
+  * the same layer at decode sizes T = 1, 8, 32 (two-launch front end, 16/32-row tiles, narrow second GEMM).
+
+The oracle cannot run a whole 11 GB layer; what is compared is (a) the router's logits for every token against an
+fp64 product, (b) ids and weights for every token, exactly, given the scores the device selected on, (c) a sample
+of tokens through the strict steps of oracle/parity_checks.py with only the experts they use brought to the host,
+and (d) bit-equality of the big batch's rows with the staged kernels on the sampled tokens alone.
+"""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+H, I, E, K, I_SH = 7168, 2048, 256, 8, 2048
+G, TG, SCALE = 8, 4, 2.5
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def _weights(pkg, dev, n_experts, n, k, seed):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    q = torch.empty(n_experts, n, k, dtype=torch.float8_e4m3fn, device=dev)
+    s = torch.empty(n_experts, n // 128, k // 128, dtype=torch.float32, device=dev)
+    step = max(1, (1 << 27) // (n * k))
+    for e0 in range(0, n_experts, step):
+        e1 = min(n_experts, e0 + step)
+        w = (torch.randn(e1 - e0, n, k, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+        q[e0:e1], s[e0:e1] = pkg.quant_weight_block128(w)
+    return q, s
+
+
+@pytest.fixture(scope="module")
+def ds_layer(pkg, dev):
+    """The DeepSeek-V3-shaped layer (256 routed experts + 1 shared), random weights made on the device."""
+    say("building the full-size layer")
+    layer = (*_weights(pkg, dev, E, 2 * I, H, 1), *_weights(pkg, dev, E, H, I, 2))
+    shared = (*_weights(pkg, dev, 1, 2 * I_SH, H, 3), *_weights(pkg, dev, 1, H, I_SH, 4))
+    g = torch.Generator(device=dev).manual_seed(5)
+    wr = (torch.randn(E, H, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    yield layer, shared, wr
+    del layer, shared, wr
+    torch.cuda.empty_cache()
+
+
+def _check_router(pkg, oracle, x, wr, bias, logits, w, ids):
+    """(a) + (b) for every token of the batch."""
+    exact = x.double().cpu() @ wr.double().cpu().t()
+    err = (logits.double().cpu() - exact).abs()
+    bound = exact.abs() * 2.0 ** -8 + 1e-4 * x.double().cpu().norm(dim=1, keepdim=True) * wr.double().cpu().norm(dim=1)[None]
+    assert bool((err <= bound).all()), float((err - bound).max())
+    # the stand-alone routing entry point on the same logits: same bits, and it shows the scores it selected on
+    w2, ids2, scores = pkg.moe_route(logits, K, "sigmoid", bias=bias, n_groups=G, topk_groups=TG, renorm=True,
+                                     scale=SCALE, return_scores=True)
+    assert torch.equal(ids, ids2) and torch.equal(w, w2)
+    scores = scores.cpu()
+    assert torch.allclose(scores, torch.sigmoid(logits.float().cpu()), rtol=1e-6, atol=1e-7)
+    w_ref, ids_ref = oracle.select_sigmoid_grouped(scores, None if bias is None else bias.cpu(), K, G, TG, SCALE, True)
+    assert torch.equal(ids.cpu(), ids_ref), "routing ids differ from the oracle's on the device's scores"
+    assert torch.allclose(w.cpu(), w_ref, rtol=1e-5, atol=1e-7)
+    assert all(len(set(row)) == K for row in ids_ref.tolist())
+
+
+def test_timed_prefill_path_deepseek_shape_with_shared_expert(pkg, oracle, dev, checks, ds_layer):
+    layer, shared, wr = ds_layer
+    T = 4096
+    say("C3 timed path, T =", T, "tile rows", pkg.tile_rows(T, K, E))
+    assert pkg.tile_rows(T, K, E) == 192
+    g = torch.Generator(device=dev).manual_seed(11)
+    x = torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16)
+    bias = torch.zeros(E, device=dev)
+    out, logits, w, ids = pkg.layer_fp8(x, wr, *layer, K, "sigmoid", bias=bias, n_groups=G, topk_groups=TG, renorm=True,
+                                        scale=SCALE, shared=shared, return_routing=True)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    _check_router(pkg, oracle, x, wr, bias, logits, w, ids)
+    # permutation of the whole batch
+    ss, off, s2r = pkg.moe_permute(ids, E)
+    ss_ref, off_ref, s2r_ref = oracle.permute_counting_sort(ids.cpu(), E)
+    assert torch.equal(ss.cpu(), ss_ref) and torch.equal(off.cpu(), off_ref) and torch.equal(s2r.cpu(), s2r_ref)
+    # the staged entry point on the same routing gives the same bits as the one-call entry point
+    out2 = pkg.fused_experts_fp8(x, *layer, ids, w, shared=shared)
+    torch.cuda.synchronize()
+    assert torch.equal(out2.view(torch.int16), out.view(torch.int16))
+    # sampled tokens: first and last of the batch, rows that land in different row tiles of their experts
+    pick = torch.tensor([0, 1, 517, 1033, 2048, 2999, 3584, 4095], device=dev)
+    y = pkg.fused_experts_fp8(x, *layer, ids)                    # per-slot rows of the whole batch, 192-row tiles
+    torch.cuda.synchronize()
+    rep = checks.check_sample(pkg, oracle, x[pick].contiguous(), ids[pick].contiguous(), layer,
+                              w_s=w[pick].contiguous(), shared_dev=shared, y_big=y[pick].contiguous(),
+                              out_big=out[pick].contiguous(), what="C3 T=4096")
+    say("   ", rep)
+
+
+@pytest.mark.parametrize("T", [1, 8, 32])
+def test_decode_deepseek_shape_full_size(pkg, oracle, dev, checks, ds_layer, T):
+    layer, shared, wr = ds_layer
+    say("C4 decode, T =", T, "tile rows", pkg.tile_rows(T, K, E))
+    g = torch.Generator(device=dev).manual_seed(100 + T)
+    x = torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16)
+    bias = torch.zeros(E, device=dev)               # uniform router bias
+    out, logits, w, ids = pkg.layer_fp8(x, wr, *layer, K, "sigmoid", bias=bias, n_groups=G, topk_groups=TG, renorm=True,
+                                        scale=SCALE, shared=shared, return_routing=True)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    _check_router(pkg, oracle, x, wr, bias, logits, w, ids)
+    ss, off, s2r = pkg.moe_permute(ids, E)
+    ss_ref, off_ref, s2r_ref = oracle.permute_counting_sort(ids.cpu(), E)
+    assert torch.equal(ss.cpu(), ss_ref) and torch.equal(off.cpu(), off_ref) and torch.equal(s2r.cpu(), s2r_ref)
+    # per-slot rows of the whole batch, then the sample against the oracle (the whole batch up to 8 tokens)
+    y = pkg.fused_experts_fp8(x, *layer, ids)
+    torch.cuda.synchronize()
+    pick = torch.arange(T, device=dev) if T <= 8 else torch.tensor([0, 5, 13, 21, 30, 31], device=dev)
+    rep = checks.check_sample(pkg, oracle, x[pick].contiguous(), ids[pick].contiguous(), layer,
+                              w_s=w[pick].contiguous(), shared_dev=shared, y_big=y[pick].contiguous(),
+                              out_big=out[pick].contiguous(), what=f"C4 T={T}")
+    say("   ", rep)
+    # a second call gives the same bits
+    again = pkg.layer_fp8(x, wr, *layer, K, "sigmoid", bias=bias, n_groups=G, topk_groups=TG, renorm=True, scale=SCALE,
+                          shared=shared)
+    torch.cuda.synchronize()
+    assert torch.equal(again.view(torch.int16), out.view(torch.int16))

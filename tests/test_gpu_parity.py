@@ -10,6 +10,8 @@ import numpy as np
 import pytest
 import torch
 
+import __graft_entry__ as entry
+
 pytestmark = pytest.mark.gpu
 
 RTOL, ATOL = 2e-2, 1e-2
@@ -267,6 +269,11 @@ def check_experts(pkg, oracle, dev, x, layer, ids, w, shared=None):
     say(f"   codes identical {same:.5f}; outside tolerance: per-slot {frac:.2e}, reduced {frac2:.2e}; cos_diff {cd:.2e}")
     assert frac <= MAX_OUTSIDE and frac2 <= MAX_OUTSIDE
     assert oracle.cos_sim(ref.numpy(), got.numpy()) > 0.9999 and cd < 1e-5
+    # the same steps as the full-size tests run them, shared expert included: its re-quantised codes within one step,
+    # the final output strict on the device's own codes, the worst end-to-end violation bounded
+    rep = entry.load_parity_checks().check_sample(pkg, oracle, xd, idd, (w13q, w13s, w2q, w2s), w_s=w.to(dev),
+                                                  shared_dev=sh_dev, y_big=y, out_big=out2, what="experts")
+    say(f"   worst violation: per-slot {rep['worst_per_slot']:.2f}, reduced {rep['worst_reduced']:.2f}")
     return got
 
 
@@ -300,7 +307,7 @@ def test_fused_experts_with_shared_expert_and_empty_experts(pkg, oracle, dev, T,
     check_experts(pkg, oracle, dev, x, layer, ids, w, shared=shared)
 
 
-def test_my_ops_drop_in_reference_layout(pkg, oracle, dev):
+def test_my_ops_drop_in_reference_layout(pkg, oracle, dev, checks):
     """The reference's call, argument for argument (python/regression/test_llm/test_moe.py:119-140):
     separate gate/up weights, pre-transposed down, bf16 scales, [T,K,H] output."""
     say("my_ops drop-in")
@@ -331,6 +338,11 @@ def test_my_ops_drop_in_reference_layout(pkg, oracle, dev):
     scale = ref_w8a8.abs().max().item()
     assert outside_fraction(got / scale, ref_w8a8 / scale) <= MAX_OUTSIDE
     assert oracle.cos_sim(ref_bf16.numpy(), got.numpy()) > 0.99
+    # the strict steps on the same call: the op's output rows are the staged kernels' bits on the packed weights
+    packed = pkg.pack_expert_weights(w0.to(dev), w1.to(dev), w2.transpose(1, 2).contiguous().to(dev), s0.to(dev), s1.to(dev),
+                                     s2.transpose(1, 2).contiguous().to(dev))
+    rep = checks.check_sample(pkg, oracle, x.to(dev), sel.to(dev), packed, y_big=out, what="drop-in", unit=scale)
+    say("   ", rep)
     out.zero_()
     torch.ops.my_ops.fused_moe_fused_experts_v2(*args, scratch[0], scratch[1], scratch[2], scratch[3], *tail)
     torch.cuda.synchronize()
@@ -382,7 +394,7 @@ def test_my_ops_other_block_sizes(pkg, oracle, dev, block):
         assert outside_fraction(got / scale, ref / scale) <= MAX_OUTSIDE
 
 
-def test_layer_module_end_to_end_toy_config(pkg, oracle, dev):
+def test_layer_module_end_to_end_toy_config(pkg, oracle, dev, checks):
     say("toy config end to end")
     T, H, I, E, K = 16, 256, 512, 8, 2
     layer = oracle.make_layer(E, H, I, seed=0)
@@ -399,10 +411,11 @@ def test_layer_module_end_to_end_toy_config(pkg, oracle, dev):
     assert torch.equal(ids.cpu(), ids_ref)
     ref = oracle.moe_w8a8_fp32(x, ids_ref, w_ref, *layer)
     assert outside_fraction(out.float().cpu(), ref) <= MAX_OUTSIDE
+    checks.check_sample(pkg, oracle, xd, ids, tuple(t.to(dev) for t in layer), w_s=w, out_big=out, what="toy config")
 
 
 # ----------------------------------------------------------------------------- full size, graphs
-def test_full_size_properties_deepseek_shape(pkg, oracle, dev):
+def test_full_size_properties_deepseek_shape(pkg, oracle, dev, checks):
     """DeepSeek-V3 layer shape at T=4096 (too large for the oracle as a whole): routing and permutation
     are checked exactly, the expert output through properties that do not depend on size, and a
     sample of tokens against the oracle."""
@@ -445,14 +458,14 @@ def test_full_size_properties_deepseek_shape(pkg, oracle, dev):
     ids_rev = ids[sub].flip(1).contiguous()
     y_rev = pkg.fused_experts_fp8(x[sub].contiguous(), w13, w13s, w2, w2s, ids_rev)
     assert torch.equal(y_rev.flip(1).view(torch.int16), y[sub].view(torch.int16))
-    # (c) sixteen tokens against the oracle
-    pick = torch.arange(5, T, 256)
-    xs = x[pick.to(dev)].cpu()
-    layer = tuple(t.cpu() for t in (w13, w13s, w2, w2s))
-    ref = oracle.experts_w8a8_fp32(xs, ids_ref[pick], *layer)
-    got = y[pick.to(dev)].float().cpu()
-    assert outside_fraction(got, ref) <= MAX_OUTSIDE
-    assert oracle.cal_diff(ref, got)[0] < 1e-5
+    # (c) eight tokens through the strict steps (codes within one e4m3 step; second GEMM and weighted sum strict
+    # on the device's own codes; worst end-to-end violation bounded), their rows of the big batch bit-equal to the
+    # staged kernels on those tokens alone
+    pick = torch.arange(5, T, 512, device=dev)
+    rep = checks.check_sample(pkg, oracle, x[pick].contiguous(), ids[pick].contiguous(), (w13, w13s, w2, w2s),
+                              w_s=w[pick].contiguous(), y_big=y[pick].contiguous(), out_big=out[pick].contiguous(),
+                              what="C3 experts")
+    say("   ", rep)
 
 
 def test_hip_graph_replay_matches_eager(pkg, oracle, dev):
@@ -506,7 +519,7 @@ def _layer_on_device(pkg, dev, E, H, I, seed):
     return w13, w13s, w2, w2s
 
 
-def _full_size_checks(pkg, oracle, dev, x, layer, ids, w, pick):
+def _full_size_checks(pkg, oracle, checks, dev, x, layer, ids, w, pick):
     """Size-independent properties of the expert computation plus a few tokens against the oracle."""
     w13, w13s, w2, w2s = layer
     T = x.shape[0]
@@ -520,20 +533,15 @@ def _full_size_checks(pkg, oracle, dev, x, layer, ids, w, pick):
     assert torch.equal(y_sub.view(torch.int16), y[sub].view(torch.int16)), "a token's result depends on the batch"
     y_rev = pkg.fused_experts_fp8(x[sub].contiguous(), w13, w13s, w2, w2s, ids[sub].flip(1).contiguous())
     assert torch.equal(y_rev.flip(1).view(torch.int16), y[sub].view(torch.int16)), "a token's result depends on slot order"
-    # only the experts those tokens use are brought to the host
-    sel = ids[pick.to(dev)].cpu()
-    used = torch.unique(sel).tolist()
-    remap = {e: i for i, e in enumerate(used)}
-    sel_local = torch.tensor([[remap[int(e)] for e in row] for row in sel], dtype=torch.int32)
-    idx = torch.tensor(used, device=dev)
-    small = tuple(t[idx].cpu() for t in layer)
-    ref = oracle.experts_w8a8_fp32(x[pick.to(dev)].cpu(), sel_local, *small)
-    got = y[pick.to(dev)].float().cpu()
-    assert outside_fraction(got, ref) <= MAX_OUTSIDE
-    assert oracle.cal_diff(ref, got)[0] < 1e-5
+    # the sampled tokens through the strict steps (only the experts they use are brought to the host); their rows of
+    # the big batch must be the bits the staged kernels give for those tokens alone
+    pick = pick.to(dev)
+    rep = checks.check_sample(pkg, oracle, x[pick].contiguous(), ids[pick].contiguous(), layer, w_s=w[pick].contiguous(),
+                              y_big=y[pick].contiguous(), out_big=out[pick].contiguous(), what="full size")
+    say("   ", rep)
 
 
-def test_full_size_properties_mixtral_shape(pkg, oracle, dev):
+def test_full_size_properties_mixtral_shape(pkg, oracle, dev, checks):
     """Mixtral-8x7B layer shape (8 experts, top-2, 1024 rows per expert: the matrix-core-bound case) at T=4096."""
     say("full size C2")
     T, H, I, E, K = 4096, 4096, 14336, 8, 2
@@ -547,7 +555,7 @@ def test_full_size_properties_mixtral_shape(pkg, oracle, dev):
     ss, off, s2r = pkg.moe_permute(ids, E)
     ss_ref, off_ref, s2r_ref = oracle.permute_counting_sort(ids_ref, E)
     assert torch.equal(ss.cpu(), ss_ref) and torch.equal(off.cpu(), off_ref) and torch.equal(s2r.cpu(), s2r_ref)
-    _full_size_checks(pkg, oracle, dev, x, layer, ids, w, torch.tensor([7, 1900, 4095]))
+    _full_size_checks(pkg, oracle, checks, dev, x, layer, ids, w, torch.tensor([7, 1900, 4095]))
     # the other batch sizes of the same workload (1, 8, 64, 512 tokens: row tiles of 16, 16, 64 and 64/128 rows):
     # the first tokens of the big batch on their own give the same bits, in both output forms
     y = pkg.fused_experts_fp8(x, *layer, ids)
@@ -562,7 +570,7 @@ def test_full_size_properties_mixtral_shape(pkg, oracle, dev):
         assert torch.equal(out_s.view(torch.int16), out[:Ts].view(torch.int16))
 
 
-def test_full_size_properties_skewed_load(pkg, oracle, dev):
+def test_full_size_properties_skewed_load(pkg, oracle, dev, checks):
     """Qwen3-30B-A3B layer shape, T=16384, popularity ~ rank^-1.2 and 13 experts that receive nothing: experts
     with thousands of rows (many row tiles) next to experts with a handful, and empty ones."""
     say("full size C5")
@@ -582,7 +590,7 @@ def test_full_size_properties_skewed_load(pkg, oracle, dev):
     assert torch.equal(ss.cpu(), ss_ref) and torch.equal(off.cpu(), off_ref) and torch.equal(s2r.cpu(), s2r_ref)
     counts = (off_ref[1:] - off_ref[:-1])
     assert int((counts == 0).sum()) >= 13 and int(counts.max()) > 8000
-    _full_size_checks(pkg, oracle, dev, x, layer, ids, w, torch.tensor([0, 5000, 11111, 16383]))
+    _full_size_checks(pkg, oracle, checks, dev, x, layer, ids, w, torch.tensor([0, 5000, 11111, 16383]))
 
 
 # ----------------------------------------------------------------------------- un-quantised experts

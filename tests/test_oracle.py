@@ -43,6 +43,41 @@ def test_e4m3_encode_known_answers(oracle):
     assert np.array_equal(oracle.e4m3_encode_np(np.clip(x, -448, 448)), want)
 
 
+def test_e4m3_step_known_answers_and_closed_form(oracle):
+    """e4m3_step sets the tolerance of the 'every re-quantised code within one step' check: pinned against values
+    written out by hand and against the format's closed form (three mantissa bits: the grid spacing of a code
+    with exponent field e is 2^(max(e,1) - 10); at a binade's lower edge the wider, upper gap counts)."""
+    hand = {
+        0x00: 2.0 ** -9,       # zero: the smallest subnormal is the next value
+        0x03: 2.0 ** -9,       # a subnormal (3 * 2^-9)
+        0x07: 2.0 ** -9,       # the largest subnormal, next to the first normal 2^-6
+        0x08: 2.0 ** -9,       # first normal 2^-6: both neighbours 2^-9 away
+        0x10: 2.0 ** -8,       # binade edge 2^-5: 2^-9 below, 2^-8 above
+        0x38: 0.125,           # 1.0: 0.9375 below, 1.125 above
+        0x3C: 0.125,           # 1.5
+        0x40: 0.25,            # binade edge 2.0: 0.125 below, 0.25 above
+        0x77: 16.0,            # 240
+        0x78: 32.0,            # binade edge 256
+        0x7E: 32.0,            # 448, the largest finite value: 416 below, nothing above
+        0xB8: 0.125,           # -1.0: the sign does not matter
+        0xFE: 32.0,            # -448
+    }
+    codes = torch.tensor(sorted(hand), dtype=torch.uint8)
+    got = oracle.e4m3_step(codes)
+    assert got.dtype == torch.float32
+    assert got.tolist() == [hand[int(c)] for c in codes]
+    every = torch.tensor([c for c in range(256) if (c & 0x7F) != 0x7F], dtype=torch.uint8)
+    closed = torch.tensor([2.0 ** (max((int(c) >> 3) & 15, 1) - 10) for c in every], dtype=torch.float32)
+    assert torch.equal(oracle.e4m3_step(every), closed)
+    # and it is what the decode table says: the larger of the gaps to the two neighbouring magnitudes
+    tab = oracle.e4m3_decode_table()[:0x7F].astype(np.float64)
+    for c in (0x01, 0x08, 0x10, 0x38, 0x7D, 0x7E):
+        gaps = [tab[c + 1] - tab[c] if c < 0x7E else 0.0, tab[c] - tab[c - 1] if c > 0 else 0.0]
+        assert float(oracle.e4m3_step(torch.tensor([c], dtype=torch.uint8))[0]) == max(gaps)
+    # shape is kept (the parity checks hand in [rows, I] code matrices)
+    assert tuple(oracle.e4m3_step(torch.zeros(3, 5, dtype=torch.uint8)).shape) == (3, 5)
+
+
 # ----------------------------------------------------------------------------- block dequant
 @pytest.mark.parametrize("shape,block", [((256, 384), 128), ((200, 300), 128), ((130, 70), 64), ((300, 520), 256)])
 def test_dequant_vectorised_equals_literal_block_loop(oracle, shape, block):
