@@ -41,6 +41,7 @@ extern "C" {
 #define MOE_E_ALIGN          -3   /* H or I not a multiple of 128, or pointer misaligned */
 #define MOE_E_WORKSPACE      -4   /* workspace smaller than moe_workspace_bytes()        */
 #define MOE_E_MODE           -5   /* unknown mode / dtype selector                       */
+#define MOE_E_STATIC_SCRATCH -6   /* needs more scratch than MOE_STATIC_SCRATCH_BYTES    */
 
 #define MOE_DTYPE_F32   0
 #define MOE_DTYPE_BF16  1
@@ -241,6 +242,30 @@ int moe_layer_fp8(void *stream, const void *x_bf16, int T, int H,
                          const uint8_t *shared_w2, const float *shared_w2_scale, int I_shared,
                          void *out_bf16, void *logits_out_bf16, float *weights_out, int32_t *ids_out,
                          void *workspace, size_t workspace_bytes);
+
+/*
+ * moe_layer_fp8 for callers that cannot allocate device memory or hand over a workspace: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference (its ops take
+ * every scratch tensor from the caller, fusedMoE.cpp:237-318).  Same arguments, same kernels and the same
+ * result bits as moe_layer_fp8, minus the workspace: the scratch is an array of MOE_STATIC_SCRATCH_BYTES that
+ * lives inside the library, one copy per GPU, held until the process ends.  It calls no hipMalloc / hipFree.
+ * A problem whose moe_layer_fp8_workspace_bytes() exceeds MOE_STATIC_SCRATCH_BYTES is refused with
+ * MOE_E_STATIC_SCRATCH before anything is launched (the DeepSeek-V3 layer fits up to T = 100 tokens).
+ * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two threads)
+ * race; calls on one stream are ordered and safe.
+ * moe_hip_init() looks the array's device address up for the current device (once per device; the entry
+ * point does the same on its first call there) - call it before capturing a graph on that device.
+ */
+#define MOE_STATIC_SCRATCH_BYTES (16u << 20)
+int moe_hip_init(void);
+int moe_layer_fp8_static(void *stream, const void *x_bf16, int T, int H,
+                         const void *router_w_bf16, const float *router_bias, int E, int K, int mode,
+                         int n_groups, int topk_groups, int renorm, float scale,
+                         const uint8_t *w13, const float *w13_scale,
+                         const uint8_t *w2, const float *w2_scale, int I,
+                         const uint8_t *shared_w13, const float *shared_w13_scale,
+                         const uint8_t *shared_w2, const float *shared_w2_scale, int I_shared,
+                         void *out_bf16, void *logits_out_bf16, float *weights_out, int32_t *ids_out);
 
 /*
  * The router product on its own (any T, E <= 256): logits [T, E] bf16 = x [T, H] . router_w [E, H]^T, the

@@ -40,6 +40,10 @@ SIGNATURES = {
                                      c_int, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                      c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_size_t]),
+    "moe_hip_init": (c_int, []),
+    "moe_layer_fp8_static": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                     c_int, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                     c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "moe_router_logits_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "moe_router_logits": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_size_t]),
     "moe_mm_fp8_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),

@@ -1,4 +1,5 @@
 // The whole-path entry point and the library's housekeeping calls.
+#include <atomic>
 #include "moe_common.h"
 #include "moe_layout.h"
 #include "../../include/moe_hip.h"
@@ -162,6 +163,7 @@ extern "C" const char *moe_hip_strerror(int code) {
     case MOE_E_ALIGN: return "H or I is not a multiple of 128, or a pointer is misaligned";
     case MOE_E_WORKSPACE: return "workspace too small";
     case MOE_E_MODE: return "unknown mode or dtype selector";
+    case MOE_E_STATIC_SCRATCH: return "the problem needs more scratch than the library's built-in array holds (MOE_STATIC_SCRATCH_BYTES)";
     default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
   }
 }
@@ -217,14 +219,14 @@ extern "C" size_t moe_layer_fp8_workspace_bytes(int T, int H, int I, int E, int 
   return moe::layer_layout(nullptr, T, H, I, E, K, I_shared).bytes;
 }
 
-extern "C" int moe_layer_fp8(void *stream, const void *x_bf16, int T, int H, const void *router_w_bf16,
-                             const float *router_bias, int E, int K, int mode, int n_groups, int topk_groups,
-                             int renorm, float scale, const uint8_t *w13, const float *w13_scale, const uint8_t *w2,
-                             const float *w2_scale, int I, const uint8_t *shared_w13, const float *shared_w13_scale,
-                             const uint8_t *shared_w2, const float *shared_w2_scale, int I_shared, void *out_bf16,
-                             void *logits_out_bf16, float *weights_out, int32_t *ids_out, void *workspace,
-                             size_t workspace_bytes) {
-  using namespace moe;
+namespace moe {
+static int layer_fp8_run(void *stream, const void *x_bf16, int T, int H, const void *router_w_bf16,
+                         const float *router_bias, int E, int K, int mode, int n_groups, int topk_groups,
+                         int renorm, float scale, const uint8_t *w13, const float *w13_scale, const uint8_t *w2,
+                         const float *w2_scale, int I, const uint8_t *shared_w13, const float *shared_w13_scale,
+                         const uint8_t *shared_w2, const float *shared_w2_scale, int I_shared, void *out_bf16,
+                         void *logits_out_bf16, float *weights_out, int32_t *ids_out, void *workspace,
+                         size_t workspace_bytes) {
   if (!router_w_bf16 || !w13 || !w13_scale || !w2 || !w2_scale || !workspace) return MOE_E_NULL;
   if (T != 0 && (!x_bf16 || !out_bf16)) return MOE_E_NULL;
   if (T < 0 || H < 1 || I < 1 || E < 1 || E > 256 || K < 1 || K > MOE_MAX_TOPK || K > E) return MOE_E_SHAPE;
@@ -276,6 +278,77 @@ extern "C" int moe_layer_fp8(void *stream, const void *x_bf16, int T, int H, con
   }
   return run_experts(stream, w, pw, T, H, w13, w13_scale, w2, w2_scale, I, E, K, weights, shared_w13, shared_w13_scale,
                      shared_w2, shared_w2_scale, I_sh, out_bf16, 1);
+}
+}  // namespace moe
+
+extern "C" int moe_layer_fp8(void *stream, const void *x_bf16, int T, int H, const void *router_w_bf16,
+                             const float *router_bias, int E, int K, int mode, int n_groups, int topk_groups,
+                             int renorm, float scale, const uint8_t *w13, const float *w13_scale, const uint8_t *w2,
+                             const float *w2_scale, int I, const uint8_t *shared_w13, const float *shared_w13_scale,
+                             const uint8_t *shared_w2, const float *shared_w2_scale, int I_shared, void *out_bf16,
+                             void *logits_out_bf16, float *weights_out, int32_t *ids_out, void *workspace,
+                             size_t workspace_bytes) {
+  return moe::layer_fp8_run(stream, x_bf16, T, H, router_w_bf16, router_bias, E, K, mode, n_groups, topk_groups, renorm,
+                            scale, w13, w13_scale, w2, w2_scale, I, shared_w13, shared_w13_scale, shared_w2,
+                            shared_w2_scale, I_shared, out_bf16, logits_out_bf16, weights_out, ids_out, workspace,
+                            workspace_bytes);
+}
+
+// ---- the same call for callers that cannot allocate: the workspace is an array that lives in the library ----
+//
+// One copy of `scratch` exists per GPU, at an address of its own; the array's name means nothing to host code, so
+// the device address is looked up once per device (with that device current) and that pointer is what the
+// kernels get, exactly as they get the caller's workspace in moe_layer_fp8.  Nothing in the layer's kernels
+// needs the workspace to start at zero (the one counter in it is cleared by the first launch of every call), so
+// the previous call's contents may stay.
+static __device__ __align__(256) unsigned char scratch[MOE_STATIC_SCRATCH_BYTES];
+
+namespace moe {
+constexpr int kMaxDevices = 64;
+static std::atomic<void *> g_scratch_ptr[kMaxDevices];
+
+// device address of `scratch` on the current device; the lookup runs once per device
+static int static_scratch(void **out) {
+  int dev = -1;
+  hipError_t rc = hipGetDevice(&dev);
+  if (rc != hipSuccess) return (int)rc;
+  if (dev < 0 || dev >= kMaxDevices) return MOE_E_SHAPE;
+  void *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    rc = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (rc != hipSuccess) return (int)rc;
+    if (!p || ((uintptr_t)p % 256)) return MOE_E_ALIGN;
+    g_scratch_ptr[dev].store(p, std::memory_order_release);   // two threads racing here store the same address
+  }
+  *out = p;
+  return MOE_OK;
+}
+}  // namespace moe
+
+extern "C" int moe_hip_init(void) {
+  void *p = nullptr;
+  return moe::static_scratch(&p);
+}
+
+extern "C" int moe_layer_fp8_static(void *stream, const void *x_bf16, int T, int H, const void *router_w_bf16,
+                                    const float *router_bias, int E, int K, int mode, int n_groups, int topk_groups,
+                                    int renorm, float scale, const uint8_t *w13, const float *w13_scale,
+                                    const uint8_t *w2, const float *w2_scale, int I, const uint8_t *shared_w13,
+                                    const float *shared_w13_scale, const uint8_t *shared_w2,
+                                    const float *shared_w2_scale, int I_shared, void *out_bf16, void *logits_out_bf16,
+                                    float *weights_out, int32_t *ids_out) {
+  using namespace moe;
+  if (T < 0 || H < 1 || I < 1 || E < 1 || E > 256 || K < 1 || K > MOE_MAX_TOPK || K > E || I_shared < 0) return MOE_E_SHAPE;
+  if (H % kBlock || I % kBlock) return MOE_E_ALIGN;
+  const int I_sh = shared_w13 ? I_shared : 0;
+  // the problem must fit the array: refused here, before anything is launched
+  if (layer_layout(nullptr, T, H, I, E, K, I_sh).bytes > (size_t)MOE_STATIC_SCRATCH_BYTES) return MOE_E_STATIC_SCRATCH;
+  void *ws = nullptr;
+  const int rc = static_scratch(&ws);
+  if (rc) return rc;
+  return layer_fp8_run(stream, x_bf16, T, H, router_w_bf16, router_bias, E, K, mode, n_groups, topk_groups, renorm, scale,
+                       w13, w13_scale, w2, w2_scale, I, shared_w13, shared_w13_scale, shared_w2, shared_w2_scale, I_shared,
+                       out_bf16, logits_out_bf16, weights_out, ids_out, ws, (size_t)MOE_STATIC_SCRATCH_BYTES);
 }
 
 // The router product on its own: logits [T, E] bf16 = x [T, H] . Wr [E, H]^T (fp32 sums, rounded once).

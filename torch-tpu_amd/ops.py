@@ -241,11 +241,13 @@ def layer_workspace_bytes(T, H, I, E, K, I_shared=0) -> int:
 
 def layer_fp8(x, router_weight, w13, w13_scale, w2, w2_scale, top_k: int, mode: str = "softmax", bias=None,
                      n_groups: int = 1, topk_groups: int = 1, renorm: bool = True, scale: float = 1.0, shared=None,
-                     out=None, workspace=None, return_routing: bool = False):
+                     out=None, workspace=None, return_routing: bool = False, static_scratch: bool = False):
     """Router and experts of one layer in one call (E <= 256).
 
     x [T,H] bf16, router_weight [E,H] bf16, the expert weights as in fused_experts_fp8.  Returns out [T,H] bf16,
-    or (out, logits bf16 [T,E], weights fp32 [T,k], ids int32 [T,k]) with return_routing."""
+    or (out, logits bf16 [T,E], weights fp32 [T,k], ids int32 [T,k]) with return_routing.
+    static_scratch: use the library's built-in scratch array instead of a workspace (moe_layer_fp8_static: no
+    device allocation when `out` is given; small batches only, calls on one GPU must not overlap)."""
     modes = {"softmax": ROUTE_SOFTMAX, "sigmoid": ROUTE_SIGMOID}
     _need(mode in modes, f"unknown routing mode {mode!r}")
     _need(x.dim() == 2 and w13.dim() == 3 and w2.dim() == 3 and router_weight.dim() == 2, "bad ranks")
@@ -265,24 +267,29 @@ def layer_fp8(x, router_weight, w13, w13_scale, w2, w2_scale, top_k: int, mode: 
         _need(bias.numel() == E, "bias must hold one value per expert")
         bias_ptr = _dev(bias, "bias", torch.float32)
     sh, I_sh = _shared_args(shared, H)
-    need = layer_workspace_bytes(T, H, I, E, top_k, I_sh)
-    if workspace is None:
-        workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
-    _need(workspace.numel() * workspace.element_size() >= need, "workspace too small")
+    if not static_scratch:
+        need = layer_workspace_bytes(T, H, I, E, top_k, I_sh)
+        if workspace is None:
+            workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+        _need(workspace.numel() * workspace.element_size() >= need, "workspace too small")
     logits = weights = ids = None
     if return_routing:
         logits = torch.empty(T, E, dtype=torch.bfloat16, device=x.device)
         weights = torch.empty(T, top_k, dtype=torch.float32, device=x.device)
         ids = torch.empty(T, top_k, dtype=torch.int32, device=x.device)
-    rc = lib.moe_layer_fp8(
+    args = [
         _stream(), _dev(x, "x", torch.bfloat16), T, H, _dev(router_weight, "router_weight", torch.bfloat16), bias_ptr,
         E, top_k, modes[mode], n_groups, topk_groups, int(renorm), float(scale),
         _dev(w13, "w13", _FP8), _dev(w13_scale, "w13_scale", torch.float32),
         _dev(w2, "w2", _FP8), _dev(w2_scale, "w2_scale", torch.float32), I,
         sh[0], sh[1], sh[2], sh[3], I_sh, _dev(out, "out", torch.bfloat16),
         logits.data_ptr() if return_routing else None, weights.data_ptr() if return_routing else None,
-        ids.data_ptr() if return_routing else None,
-        _dev(workspace, "workspace"), workspace.numel() * workspace.element_size())
+        ids.data_ptr() if return_routing else None]
+    if static_scratch:
+        with torch.cuda.device(x.device):        # the array's address is looked up for the current device
+            rc = lib.moe_layer_fp8_static(*args)
+    else:
+        rc = lib.moe_layer_fp8(*args, _dev(workspace, "workspace"), workspace.numel() * workspace.element_size())
     check(rc, "layer_fp8")
     return (out, logits, weights, ids) if return_routing else out
 
