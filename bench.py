@@ -46,16 +46,8 @@ WORKLOADS = {
 
 
 def make_weights(pkg, E, N, Kd, dev, seed):
-    """[E, N, Kd] ~ N(0, 0.02) bf16 -> e4m3fn + fp32 block scales, generated on the GPU in slices."""
-    g = torch.Generator(device=dev).manual_seed(seed)
-    q = torch.empty(E, N, Kd, dtype=torch.float8_e4m3fn, device=dev)
-    s = torch.empty(E, N // 128, Kd // 128, dtype=torch.float32, device=dev)
-    step = max(1, (1 << 28) // (N * Kd))
-    for e0 in range(0, E, step):
-        e1 = min(E, e0 + step)
-        w = (torch.randn(e1 - e0, N, Kd, generator=g, device=dev) * 0.02).to(torch.bfloat16)
-        q[e0:e1], s[e0:e1] = pkg.quant_weight_block128(w)
-    return q, s
+    """[E, N, Kd] ~ N(0, 0.02) bf16 -> e4m3fn (tile-blocked) + fp32 block scales, generated on the GPU in slices."""
+    return pkg.synthetic_weights(E, N, Kd, dev, seed)
 
 
 def build_layer(pkg, cfg, dev):

@@ -18,6 +18,11 @@
  *   W13      [E, 2*I, H] fp8, rows 0..I-1 = gate projection, rows I..2I-1 = up projection,
  *            fp32 scales [E, 2*I/128, H/128]  (one per 128x128 block).
  *   W2       [E, H, I] fp8, fp32 scales [E, H/128, I/128].
+ *   Every weight matrix handed to a GEMM entry point (w13, w2, shared_*, the dense layers' w, the bf16
+ *   variants' weights) is TILE-BLOCKED, not row-major: moe_pack_weights() below re-orders a row-major
+ *   matrix once, when the checkpoint is loaded (the reference's layout is re-packed at that point anyway:
+ *   separate gate / up, pre-transposed down, python/regression/test_llm/test_moe.py:285-288).  Scales keep
+ *   their plain [.., rows/128, cols/128] order.
  *   acts     bf16 [T, H]; quantised per token per 128 columns: scale = max(amax,1e-10)/448.
  *   ids      int32 [T, K], the K experts of a token are distinct.
  *   H and I must be multiples of 128.
@@ -105,6 +110,20 @@ int moe_tile_rows(int T, int K, int E);
 int moe_permute(void *stream, const int32_t *ids, int T, int K, int E,
                 int32_t *sorted_slot, int32_t *expert_offsets, int32_t *slot_to_row,
                 void *workspace, size_t workspace_bytes);
+
+/*
+ * Weight layout.  The matrix [rows, row_bytes] (rows = all experts' rows stacked, a multiple of 16; row_bytes a
+ * multiple of 128: the reduction dimension in bytes, K for fp8, 2*K for bf16) is cut into tiles of 16 rows and
+ * steps of 128 bytes.  Tile-blocked order: tiles in row order, a tile's steps one after the other, 2 KB per
+ * (tile, step) pair, and inside the 2 KB: half h = 0, 1, then lane l = 0..63, 16 bytes each = row l % 16 of the
+ * tile, bytes 16 * (l / 16 + 4 h) .. + 15 of the step.  That is a wavefront's operand of
+ * v_mfma_f32_16x16x128_f8f6f4: each load instruction of the GEMMs reads 1 KB of consecutive memory and a tile's
+ * steps stream from one contiguous region.  Replaces the weight re-layout the reference's kernel does per call
+ * on its way into local memory (torch_tpu/csrc/ops/my_ops/fusedMoE.pl:298-347, weight prefetch per expert).
+ * Out of place (MOE_E_MODE when source and destination are the same buffer); pointers 16-byte aligned.
+ */
+int moe_pack_weights(void *stream, const void *w_rowmajor, int64_t rows, int row_bytes, void *w_blocked);
+int moe_unpack_weights(void *stream, const void *w_blocked, int64_t rows, int row_bytes, void *w_rowmajor);
 
 /*
  * Activation-scale tensors (the s of moe_act_quant, xs / hs of the stage entry points) hold one

@@ -75,6 +75,12 @@ def _localise(ids_host: torch.Tensor):
     return local.reshape(ids_host.shape), used
 
 
+def _host_layer(pkg, layer_dev):
+    """Packed device layer (tile-blocked weights) -> row-major tensors on the host, as the oracle reads them."""
+    w13, w13s, w2, w2s = layer_dev
+    return (pkg.unpack_weights(w13.contiguous()).cpu(), w13s.cpu(), pkg.unpack_weights(w2.contiguous()).cpu(), w2s.cpu())
+
+
 def staged_experts(pkg, x_s, ids_s, layer_dev):
     """The staged kernels through the C ABI on a (small) batch: -> y [n,K,H] bf16 (slot order), and the device's
     re-quantised SwiGLU codes / scales in slot order (uint8 [n*K, I], fp32 [n*K, I/128]) plus xq, xs."""
@@ -115,7 +121,7 @@ def check_sample(pkg, oracle, x_s, ids_s, layer_dev, w_s=None, shared_dev=None, 
     ids_host = ids_s.cpu()
     local, used = _localise(ids_host)
     idx = torch.tensor(used, device=x_s.device)
-    small = tuple(t[idx].cpu() for t in layer_dev)
+    small = _host_layer(pkg, tuple(t[idx] for t in layer_dev))
     x_host = x_s.cpu()
     ref, (xq_ref, xs_ref, hq_ref, hs_ref) = oracle.experts_w8a8_fp32(x_host, local, *small, return_mid=True)
     # (0)
@@ -138,7 +144,7 @@ def check_sample(pkg, oracle, x_s, ids_s, layer_dev, w_s=None, shared_dev=None, 
         if shared_dev is not None:
             zeros = torch.zeros(n, 1, dtype=torch.int32, device=x_s.device)
             sh_y, sh_hq, sh_hs, _, _ = staged_experts(pkg, x_s, zeros, shared_dev)
-            sh_host = tuple(t.cpu() for t in shared_dev)
+            sh_host = _host_layer(pkg, shared_dev)
             I_sh = shared_dev[2].shape[2]
             z = zeros.cpu()
             sh_ref, (_, _, shq_ref, shs_ref) = oracle.experts_w8a8_fp32(x_host, z, *sh_host, return_mid=True)

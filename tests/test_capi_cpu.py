@@ -117,6 +117,9 @@ def test_my_ops_are_registered_with_reference_arity(pkg):
     assert len(ops.fused_moe_grouped_topk.default._schema.arguments) == 10
     assert len(ops.mlp_w8a16_dq_forward.default._schema.arguments) == 9     # ops.hpp:279-288
     assert len(ops.mm_w8a16_dq_forward.default._schema.arguments) == 5      # ops.hpp:290-295
+    assert len(ops.moe_route.default._schema.arguments) == 9
+    assert len(ops.moe_permute.default._schema.arguments) == 2
+    assert len(ops.moe_pack_weights.default._schema.arguments) == 6
     with pytest.raises(RuntimeError, match="closed-source"):
         ops.fused_moe_grouped_topk(*[torch.zeros(1)] * 10)
     z = torch.zeros(1, 1, 128, dtype=torch.bfloat16)
@@ -138,7 +141,7 @@ def test_checkpoint_layout_conversion_is_pure_data_movement(pkg, oracle):
             state[base + proj + ".weight"], state[base + proj + ".weight_scale_inv"] = q, s
     state[pre + "gate.weight"] = torch.randn(E, H, generator=g)
     state[pre + "gate.e_score_correction_bias"] = torch.randn(E, generator=g)
-    out = pkg.convert_hf_moe_layer(state, pre, E)
+    out = pkg.convert_hf_moe_layer(state, pre, E, tile_block=False)      # the last step (byte order) needs the GPU
     assert out["w13"].shape == (E, 2 * I, H) and out["w2"].shape == (E, H, I) and out["router_weight"].dtype == torch.bfloat16
     for e in range(E):
         gate = oracle.dequant_block(state[f"{pre}experts.{e}.gate_proj.weight"], state[f"{pre}experts.{e}.gate_proj.weight_scale_inv"])
@@ -163,3 +166,60 @@ def test_size_functions_accept_an_empty_batch(pkg):
     assert lib.moe_mm_fp8_workspace_bytes(0, 256, 256) > 0
     assert lib.moe_mlp_fp8_workspace_bytes(0, 256, 128) > 0
     assert lib.moe_tile_rows(0, 2, 8) == 16
+
+
+def test_derived_weight_cache_follows_the_source_tensors(pkg):
+    """The drop-in ops keep packed copies of the caller's weights.  A copy must never outlive or out-date its sources:
+    same tensors -> one pack; a recorded in-place change, new tensors (also on a recycled address), or an explicit
+    invalidation -> a fresh pack; many layers -> every layer keeps its entry."""
+    import gc
+    import torch
+    my_ops = pkg._my_ops
+    cache = my_ops._DerivedCache()
+    calls = []
+
+    def packer(ts):
+        def make():
+            calls.append(1)
+            return tuple(t.clone() for t in ts)
+        return make
+
+    a, b = torch.arange(8.0), torch.ones(4)
+    v1 = cache.get((a, b), "x", packer((a, b)))
+    v2 = cache.get((a, b), "x", packer((a, b)))
+    assert v1 is v2 and len(calls) == 1
+    assert cache.get((a, b), "other use", packer((a, b))) is not v1 and len(calls) == 2       # tags do not mix
+    a.add_(1)                                                  # bumps the version counter
+    v3 = cache.get((a, b), "x", packer((a, b)))
+    assert v3 is not v1 and torch.equal(v3[0], a) and len(calls) == 3
+    # an update through .data leaves no trace in the version counter: documented, cured by invalidation
+    a.data.copy_(torch.zeros(8))
+    assert cache.get((a, b), "x", packer((a, b))) is v3
+    saved, my_ops._weights = my_ops._weights, cache
+    try:
+        pkg.invalidate_weight_cache()
+    finally:
+        my_ops._weights = saved
+    v4 = cache.get((a, b), "x", packer((a, b)))
+    assert v4 is not v3 and torch.equal(v4[0], torch.zeros(8))
+    # freed sources take their entry with them; new tensors never meet an old copy, whatever their address
+    n_before = len(cache)
+    ptr = a.data_ptr()
+    del a, v1, v2, v3, v4
+    gc.collect()
+    assert len(cache) < n_before
+    for _ in range(50):
+        c = torch.full((8,), 7.0)
+        got = cache.get((c, b), "x", packer((c, b)))
+        assert torch.equal(got[0], c)
+        same_address = c.data_ptr() == ptr
+        del c, got
+        if same_address:
+            break
+    # a model with many layers, called layer after layer, twice: every layer is packed exactly once
+    layers = [(torch.randn(4), torch.randn(4)) for _ in range(40)]
+    calls.clear()
+    for _ in range(2):
+        for la in layers:
+            assert torch.equal(cache.get(la, "layer", packer(la))[0], la[0])
+    assert len(calls) == len(layers)

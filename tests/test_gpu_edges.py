@@ -13,7 +13,7 @@ def say(*a):
 def test_empty_batch_is_a_valid_call_everywhere(pkg, oracle, dev):
     say("empty batch")
     H, I, E, K = 256, 128, 8, 2
-    ld = tuple(t.to(dev) for t in oracle.make_layer(E, H, I, seed=3))
+    ld = pkg.pack_layer(*(t.to(dev) for t in oracle.make_layer(E, H, I, seed=3)))
     x = torch.empty(0, H, dtype=torch.bfloat16, device=dev)
     ids = torch.empty(0, K, dtype=torch.int32, device=dev)
     w = torch.empty(0, K, dtype=torch.float32, device=dev)
@@ -86,7 +86,7 @@ def test_slots_without_an_expert_add_nothing(pkg, oracle, dev, T):
     ids_bad[bad] = torch.where(torch.rand(int(bad.sum()), generator=g) < 0.5, torch.tensor(-1), torch.tensor(E)).to(torch.int32)
     ref_slots = oracle.experts_w8a8_fp32(x, ids, *layer)
     ref_slots[bad] = 0.0
-    dl = tuple(t.to(dev) for t in layer)
+    dl = pkg.pack_layer(*(t.to(dev) for t in layer))
     # poisoned outputs and workspace: whatever the call does not write would show
     out3 = torch.full((T, K, H), float("nan"), dtype=torch.bfloat16, device=dev)
     pkg.fused_experts_fp8(x.to(dev), *dl, ids_bad.to(dev), out=out3)
@@ -107,8 +107,8 @@ def test_slots_without_an_expert_add_nothing(pkg, oracle, dev, T):
     ref2 = torch.einsum("tk,tkh->th", w, got3)                  # the device's own slot results, summed on the host
     torch.testing.assert_close(got2, ref2, rtol=2e-2, atol=1e-2 * scale)
     # un-quantised experts take the same route
-    w13b = oracle.dequant_block(layer[0], layer[1]).to(torch.bfloat16).to(dev)
-    w2b = oracle.dequant_block(layer[2], layer[3]).to(torch.bfloat16).to(dev)
+    w13b = pkg.pack_weights(oracle.dequant_block(layer[0], layer[1]).to(torch.bfloat16).to(dev))
+    w2b = pkg.pack_weights(oracle.dequant_block(layer[2], layer[3]).to(torch.bfloat16).to(dev))
     outb = torch.full((T, K, H), float("nan"), dtype=torch.bfloat16, device=dev)
     pkg.fused_experts_bf16(x.to(dev), w13b, w2b, ids_bad.to(dev), out=outb)
     torch.cuda.synchronize()
@@ -121,7 +121,7 @@ def test_slots_without_an_expert_add_nothing(pkg, oracle, dev, T):
 def test_one_workspace_serves_calls_of_different_sizes(pkg, oracle, dev):
     say("workspace reuse")
     H, I, E, K = 512, 256, 16, 4
-    ld = tuple(t.to(dev) for t in oracle.make_layer(E, H, I, seed=4))
+    ld = pkg.pack_layer(*(t.to(dev) for t in oracle.make_layer(E, H, I, seed=4)))
     sizes = [300, 3, 70, 1, 129]
     ws = torch.empty(pkg.fused_experts_workspace_bytes(max(sizes), H, I, E, K), dtype=torch.uint8, device=dev)
     ws.fill_(0xA5)
@@ -145,7 +145,7 @@ def test_largest_expert_and_topk_counts(pkg, oracle, dev):
     w_ref, ids_ref = oracle.route_softmax_topk(logits, K)
     w, ids = pkg.moe_route(logits.to(dev), K, "softmax")
     assert torch.equal(ids.cpu(), ids_ref)
-    out = pkg.fused_experts_fp8(x.to(dev), *(t.to(dev) for t in layer), ids, w)
+    out = pkg.fused_experts_fp8(x.to(dev), *pkg.pack_layer(*(t.to(dev) for t in layer)), ids, w)
     torch.cuda.synchronize()
     ref = oracle.moe_w8a8_fp32(x, ids_ref, w_ref, *layer)
     bad = (out.float().cpu() - ref).abs() > 1e-2 + 2e-2 * ref.abs()
@@ -162,6 +162,7 @@ def test_large_batch_addresses(pkg, oracle, dev):
     w2 = (torch.randn(E, H, I, generator=gg, device=dev) * 0.02).to(torch.bfloat16)
     w13q, w13s = pkg.quant_weight_block128(w13)
     w2q, w2s = pkg.quant_weight_block128(w2)
+    w13q, w2q = pkg.pack_weights(w13q), pkg.pack_weights(w2q)
     del w13, w2
     x = torch.randn(T, H, generator=gg, device=dev).to(torch.bfloat16)
     logits = torch.randn(T, E, generator=gg, device=dev)

@@ -22,24 +22,12 @@ def say(*a):
     print(*a, flush=True)
 
 
-def _weights(pkg, dev, n_experts, n, k, seed):
-    g = torch.Generator(device=dev).manual_seed(seed)
-    q = torch.empty(n_experts, n, k, dtype=torch.float8_e4m3fn, device=dev)
-    s = torch.empty(n_experts, n // 128, k // 128, dtype=torch.float32, device=dev)
-    step = max(1, (1 << 27) // (n * k))
-    for e0 in range(0, n_experts, step):
-        e1 = min(n_experts, e0 + step)
-        w = (torch.randn(e1 - e0, n, k, generator=g, device=dev) * 0.02).to(torch.bfloat16)
-        q[e0:e1], s[e0:e1] = pkg.quant_weight_block128(w)
-    return q, s
-
-
 @pytest.fixture(scope="module")
 def ds_layer(pkg, dev):
     """The DeepSeek-V3-shaped layer (256 routed experts + 1 shared), random weights made on the device."""
     say("building the full-size layer")
-    layer = (*_weights(pkg, dev, E, 2 * I, H, 1), *_weights(pkg, dev, E, H, I, 2))
-    shared = (*_weights(pkg, dev, 1, 2 * I_SH, H, 3), *_weights(pkg, dev, 1, H, I_SH, 4))
+    layer = (*pkg.synthetic_weights(E, 2 * I, H, dev, 1), *pkg.synthetic_weights(E, H, I, dev, 2))
+    shared = (*pkg.synthetic_weights(1, 2 * I_SH, H, dev, 3), *pkg.synthetic_weights(1, H, I_SH, dev, 4))
     g = torch.Generator(device=dev).manual_seed(5)
     wr = (torch.randn(E, H, generator=g, device=dev) * 0.02).to(torch.bfloat16)
     yield layer, shared, wr

@@ -71,7 +71,7 @@ def test_small_batch_routing_equals_large_batch_routing(pkg, oracle, dev, E, K, 
 
 def _shared(pkg, oracle, H, I_sh, seed, dev):
     w13, w13s, w2, w2s = oracle.make_layer(1, H, I_sh, seed=seed)
-    return tuple(t.to(dev) for t in (w13, w13s, w2, w2s))
+    return pkg.pack_layer(*(t.to(dev) for t in (w13, w13s, w2, w2s)))
 
 
 LAYER_CASES = [
@@ -97,19 +97,9 @@ def test_layer_entry_point(pkg, oracle, dev, checks, T, H, I, E, K, mode, G, TG,
     small = 3 * E * H * I <= (1 << 26)
     if small:
         layer = oracle.make_layer(E, H, I, seed=T + E)
-        ld = tuple(t.to(dev) for t in layer)
+        ld = pkg.pack_layer(*(t.to(dev) for t in layer))
     else:                                   # too large to make on the host: random weights made on the device
-        gd = torch.Generator(device=dev).manual_seed(T + E)
-
-        def make(n, k):                      # in slices of experts: the fp32 intermediates of a whole layer are large
-            q = torch.empty(E, n, k, dtype=torch.float8_e4m3fn, device=dev)
-            sc = torch.empty(E, n // 128, k // 128, dtype=torch.float32, device=dev)
-            step = max(1, (1 << 27) // (n * k))
-            for e0 in range(0, E, step):
-                w = (torch.randn(min(step, E - e0), n, k, generator=gd, device=dev) * 0.02).to(torch.bfloat16)
-                q[e0:e0 + step], sc[e0:e0 + step] = pkg.quant_weight_block128(w)
-            return q, sc
-        ld = (*make(2 * I, H), *make(H, I))
+        ld = (*pkg.synthetic_weights(E, 2 * I, H, dev, T + E), *pkg.synthetic_weights(E, H, I, dev, T + E + 1))
     g = torch.Generator().manual_seed(7 * T + E)
     x = torch.randn(T, H, generator=g).to(torch.bfloat16)
     wr = (torch.randn(E, H, generator=g) * 0.05).to(torch.bfloat16)
@@ -180,7 +170,7 @@ def test_router_logits_kernel(pkg, dev, T, H, E):
 def test_layer_entry_point_in_a_hip_graph(pkg, oracle, dev):
     say("decode layer graph")
     T, H, I, E, K = 4, 1024, 256, 64, 4
-    ld = tuple(t.to(dev) for t in oracle.make_layer(E, H, I, seed=5))
+    ld = pkg.pack_layer(*(t.to(dev) for t in oracle.make_layer(E, H, I, seed=5)))
     g = torch.Generator().manual_seed(5)
     wr = (torch.randn(E, H, generator=g) * 0.05).to(torch.bfloat16).to(dev)
     xs = [torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev) for _ in range(3)]
@@ -217,7 +207,7 @@ def test_layer_entry_point_rejects_what_it_does_not_cover(pkg, oracle, dev):
                              0, 1, None, None, None, 256, 1 << 30) == -2
     assert lib.moe_layer_fp8_workspace_bytes(1, H, I, 300, 8, 0) == 0
     E, K = 16, 8
-    ld = tuple(t.to(dev) for t in oracle.make_layer(E, H, I, seed=1))
+    ld = pkg.pack_layer(*(t.to(dev) for t in oracle.make_layer(E, H, I, seed=1)))
     wr = (torch.randn(E, H, generator=g) * 0.05).to(torch.bfloat16).to(dev)
     x = torch.randn(2, H, generator=g).to(torch.bfloat16).to(dev)
     with pytest.raises(RuntimeError):
@@ -227,3 +217,75 @@ def test_layer_entry_point_rejects_what_it_does_not_cover(pkg, oracle, dev):
     out = pkg.layer_fp8(x, wr, *ld, K, "softmax")
     torch.cuda.synchronize()
     assert torch.isfinite(out.float()).all()
+
+
+def test_checkpoint_converter_feeds_the_kernels(pkg, oracle, dev, checks):
+    """A DeepSeek-V3-style FP8 checkpoint (per-expert `weight` [out, in] + `weight_scale_inv`, router, correction bias,
+    shared expert) through convert_hf_moe_layer into the module, against the oracle on the checkpoint's own tensors;
+    and the reference's argument layout (separate gate / up, pre-transposed down and scales,
+    python/regression/test_llm/test_moe.py:285-288) through pack_expert_weights gives the same packed bytes."""
+    say("checkpoint converter")
+    E, H, I, K, T = 16, 512, 256, 4, 24
+    g = torch.Generator().manual_seed(31)
+    state, pre = {}, "model.layers.3.mlp."
+    per_expert = {}
+    for e in list(range(E)) + ["s"]:
+        base = pre + ("shared_experts." if e == "s" else f"experts.{e}.")
+        for proj, (n, k) in (("gate_proj", (I, H)), ("up_proj", (I, H)), ("down_proj", (H, I))):
+            q, sc = oracle.quant_weight_block128(torch.randn(n, k, generator=g) * 0.05)
+            state[base + proj + ".weight"], state[base + proj + ".weight_scale_inv"] = q, sc
+            per_expert[(e, proj)] = (q, sc)
+    state[pre + "gate.weight"] = (torch.randn(E, H, generator=g) * 0.05).to(torch.bfloat16)
+    state[pre + "gate.e_score_correction_bias"] = torch.randn(E, generator=g) * 0.05
+    conv = pkg.convert_hf_moe_layer(state, pre, E, device=dev)
+    moe = pkg.FusedMoE(conv["router_weight"], conv["w13"], conv["w13_scale"], conv["w2"], conv["w2_scale"], top_k=K,
+                       mode="sigmoid", bias=conv["bias"], n_groups=4, topk_groups=2, renorm=True, scale=2.5,
+                       shared=conv["shared"])
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    xd = x.to(dev)
+    out, logits, w, ids = pkg.layer_fp8(xd, conv["router_weight"], conv["w13"], conv["w13_scale"], conv["w2"],
+                                        conv["w2_scale"], K, "sigmoid", bias=conv["bias"], n_groups=4, topk_groups=2,
+                                        renorm=True, scale=2.5, shared=conv["shared"], return_routing=True)
+    assert torch.equal(moe(xd).view(torch.int16), out.view(torch.int16))
+    torch.cuda.synchronize()
+    # the oracle on the checkpoint's own per-expert tensors (nothing of the converter is reused)
+    stack = lambda proj: (torch.stack([per_expert[(e, proj)][0] for e in range(E)]),
+                          torch.stack([per_expert[(e, proj)][1] for e in range(E)]))
+    (gq, gs), (uq, us), (dq, ds) = stack("gate_proj"), stack("up_proj"), stack("down_proj")
+    layer = (torch.cat([gq, uq], 1), torch.cat([gs, us], 1), dq, ds)
+    sh = (torch.cat([per_expert[("s", "gate_proj")][0], per_expert[("s", "up_proj")][0]], 0)[None],
+          torch.cat([per_expert[("s", "gate_proj")][1], per_expert[("s", "up_proj")][1]], 0)[None],
+          per_expert[("s", "down_proj")][0][None], per_expert[("s", "down_proj")][1][None])
+    scores = pkg.moe_route(logits, K, "sigmoid", bias=conv["bias"], n_groups=4, topk_groups=2, renorm=True, scale=2.5,
+                           return_scores=True)[2].cpu()
+    w_ref, ids_ref = oracle.select_sigmoid_grouped(scores, state[pre + "gate.e_score_correction_bias"], K, 4, 2, 2.5, True)
+    assert torch.equal(ids.cpu(), ids_ref) and torch.allclose(w.cpu(), w_ref, rtol=1e-5, atol=1e-7)
+    ref = oracle.moe_w8a8_fp32(x, ids_ref, w_ref, *layer, shared=sh)
+    got = out.float().cpu()
+    assert checks.outside_fraction(got, ref) <= checks.MAX_OUTSIDE
+    assert oracle.cal_diff(ref, got)[0] < 1e-5
+    # the converter's packed bytes are the oracle's row-major tensors, tile-blocked
+    assert torch.equal(pkg.unpack_weights(conv["w13"]).cpu().view(torch.uint8), layer[0].view(torch.uint8))
+    assert torch.equal(pkg.unpack_weights(conv["w2"]).cpu().view(torch.uint8), layer[2].view(torch.uint8))
+    rep = checks.check_sample(pkg, oracle, xd, ids, (conv["w13"], conv["w13_scale"], conv["w2"], conv["w2_scale"]),
+                              w_s=w, shared_dev=conv["shared"], out_big=out, what="converted checkpoint")
+    say("   ", rep)
+    # the reference's argument form of the same weights: pre-transposed down, bf16-representable scales aside, the
+    # packed bytes are identical
+    packed = pkg.pack_expert_weights(gq.to(dev), uq.to(dev), dq.transpose(1, 2).contiguous().to(dev), gs.to(dev),
+                                     us.to(dev), ds.transpose(1, 2).contiguous().to(dev))
+    torch.cuda.synchronize()
+    for a, b in zip(packed, (conv["w13"], conv["w13_scale"], conv["w2"], conv["w2_scale"])):
+        assert torch.equal(a.view(torch.uint8) if a.dtype == torch.float8_e4m3fn else a,
+                           b.view(torch.uint8) if b.dtype == torch.float8_e4m3fn else b)
+    # and the registered op form of the same packing
+    packed2 = torch.ops.my_ops.moe_pack_weights(gq.to(dev), uq.to(dev), dq.transpose(1, 2).contiguous().to(dev), gs.to(dev),
+                                                us.to(dev), ds.transpose(1, 2).contiguous().to(dev))
+    assert all(torch.equal(a.view(torch.uint8) if a.dtype == torch.float8_e4m3fn else a,
+                           b.view(torch.uint8) if b.dtype == torch.float8_e4m3fn else b) for a, b in zip(packed, packed2))
+    # the router op and the permutation op of the same namespace
+    w_op, ids_op = torch.ops.my_ops.moe_route(xd, conv["router_weight"], conv["bias"], "sigmoid", K, 4, 2, 2.5, True)
+    assert torch.equal(ids_op, ids) and torch.equal(w_op, w)
+    ss, off, s2r = torch.ops.my_ops.moe_permute(ids, E)
+    ss_ref, off_ref, s2r_ref = oracle.permute_counting_sort(ids.cpu(), E)
+    assert torch.equal(ss.cpu(), ss_ref) and torch.equal(off.cpu(), off_ref) and torch.equal(s2r.cpu(), s2r_ref)

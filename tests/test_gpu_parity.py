@@ -47,6 +47,54 @@ def test_act_quant_bit_exact(pkg, oracle, dev, R, C):
     assert torch.equal(q.cpu().view(torch.uint8), q_ref.view(torch.uint8))
 
 
+# ----------------------------------------------------------------------------- weight layout
+def tile_blocked_reference(w):
+    """The tile-blocked byte order written as an index permutation: [tile, row, step, half, chunk, byte] ->
+    [tile, step, half, chunk, row, byte] (16-row tiles, 128-byte steps, 16-byte chunks; chunk c of a step sits in
+    half c // 4 at position c % 4)."""
+    N, K = w.shape[-2:]
+    b = w.contiguous().view(torch.uint8).reshape(-1, N // 16, 16, K * w.element_size() // 128, 2, 4, 16)
+    return b.permute(0, 1, 3, 4, 5, 2, 6).contiguous().reshape(-1).view(w.dtype).reshape(w.shape)
+
+
+@pytest.mark.parametrize("shape,dtype", [((16, 128), torch.uint8), ((3, 32, 256), torch.float8_e4m3fn),
+                                         ((2, 48, 384), torch.bfloat16), ((5, 1024, 7168), torch.float8_e4m3fn),
+                                         ((1536, 7168), torch.float8_e4m3fn)])
+def test_pack_weights_is_the_documented_permutation(pkg, dev, shape, dtype):
+    say("pack weights", shape, dtype)
+    g = torch.Generator().manual_seed(sum(shape))
+    raw = torch.randint(0, 256, (*shape[:-1], shape[-1] * torch.empty(0, dtype=dtype).element_size()), generator=g,
+                        dtype=torch.uint8)
+    w = raw.view(dtype).reshape(shape)
+    packed = pkg.pack_weights(w.to(dev))
+    torch.cuda.synchronize()
+    assert packed.shape == w.shape and packed.dtype == w.dtype
+    assert torch.equal(packed.cpu().view(torch.uint8), tile_blocked_reference(w).view(torch.uint8))
+    back = pkg.unpack_weights(packed)
+    torch.cuda.synchronize()
+    assert torch.equal(back.cpu().view(torch.uint8), w.view(torch.uint8))
+    # lane l of the first instruction of tile 0, step 0 gets row l % 16, bytes 16 * (l // 16) .. + 15
+    flat = packed.cpu().view(torch.uint8).reshape(-1)
+    rows = w.view(torch.uint8).reshape(-1, raw.shape[-1])
+    for l in (0, 1, 17, 63):
+        assert torch.equal(flat[16 * l:16 * l + 16], rows[l % 16, 16 * (l // 16):16 * (l // 16) + 16])
+        assert torch.equal(flat[1024 + 16 * l:1024 + 16 * l + 16], rows[l % 16, 64 + 16 * (l // 16):64 + 16 * (l // 16) + 16])
+
+
+def test_pack_weights_rejects_what_it_cannot_tile(pkg, dev):
+    say("pack weights errors")
+    with pytest.raises(RuntimeError):
+        pkg.pack_weights(torch.zeros(8, 128, dtype=torch.uint8, device=dev))           # rows not a multiple of 16
+    with pytest.raises(RuntimeError):
+        pkg.pack_weights(torch.zeros(16, 64, dtype=torch.uint8, device=dev))           # a row shorter than a step
+    with pytest.raises(RuntimeError):
+        pkg.pack_weights(torch.zeros(16, 128, dtype=torch.uint8))                      # not on the GPU
+    lib = pkg._lib.lib
+    buf = torch.zeros(16, 128, dtype=torch.uint8, device=dev)
+    assert lib.moe_pack_weights(None, buf.data_ptr(), 16, 128, buf.data_ptr()) == -5   # in place
+    assert lib.moe_pack_weights(None, None, 0, 128, None) == 0                         # nothing to do
+
+
 # ----------------------------------------------------------------------------- routing
 @pytest.mark.parametrize("batch", [1, 8, 16, 64, 128])
 def test_noaux_tc_topk_reference_cases(pkg, oracle, dev, batch):
@@ -208,7 +256,7 @@ def check_experts(pkg, oracle, dev, x, layer, ids, w, shared=None):
     T, K = ids.shape
     E, H, I = layer[2].shape
     ref, (xq_ref, xs_ref, hq_ref, hs_ref) = oracle.experts_w8a8_fp32(x, ids, *layer, return_mid=True)
-    w13q, w13s, w2q, w2s = (t.to(dev) for t in layer)
+    w13q, w13s, w2q, w2s = pkg.pack_layer(*(t.to(dev) for t in layer))
     xd, idd = x.to(dev), ids.to(dev)
 
     # ---- staged run through the C ABI
@@ -248,7 +296,7 @@ def check_experts(pkg, oracle, dev, x, layer, ids, w, shared=None):
     pkg.fused_experts_fp8(xd, w13q, w13s, w2q, w2s, idd, None, out=out)
     torch.cuda.synchronize()
     assert torch.equal(out.view(torch.int16).cpu(), y.view(torch.int16).cpu())
-    sh_dev = None if shared is None else tuple(t.to(dev) for t in shared)
+    sh_dev = None if shared is None else pkg.pack_layer(*(t.to(dev) for t in shared))
     out2 = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=dev)
     pkg.fused_experts_fp8(xd, w13q, w13s, w2q, w2s, idd, w.to(dev), out=out2, shared=sh_dev)
     torch.cuda.synchronize()
@@ -401,7 +449,8 @@ def test_layer_module_end_to_end_toy_config(pkg, oracle, dev, checks):
     g = torch.Generator().manual_seed(0)
     x = torch.randn(T, H, generator=g).to(torch.bfloat16)
     wr = (torch.randn(E, H, generator=g) * 0.02).to(torch.bfloat16)
-    moe = pkg.FusedMoE(wr.to(dev), *(t.to(dev) for t in layer), top_k=K, mode="softmax")
+    layer_dev = pkg.pack_layer(*(t.to(dev) for t in layer))
+    moe = pkg.FusedMoE(wr.to(dev), *layer_dev, top_k=K, mode="softmax")
     xd = x.to(dev)
     w, ids = moe.route(xd)
     out = moe.experts(xd, w, ids)
@@ -411,7 +460,7 @@ def test_layer_module_end_to_end_toy_config(pkg, oracle, dev, checks):
     assert torch.equal(ids.cpu(), ids_ref)
     ref = oracle.moe_w8a8_fp32(x, ids_ref, w_ref, *layer)
     assert outside_fraction(out.float().cpu(), ref) <= MAX_OUTSIDE
-    checks.check_sample(pkg, oracle, xd, ids, tuple(t.to(dev) for t in layer), w_s=w, out_big=out, what="toy config")
+    checks.check_sample(pkg, oracle, xd, ids, layer_dev, w_s=w, out_big=out, what="toy config")
 
 
 # ----------------------------------------------------------------------------- full size, graphs
@@ -425,17 +474,8 @@ def test_full_size_properties_deepseek_shape(pkg, oracle, dev, checks):
     x = torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16)
     wr = (torch.randn(E, H, generator=g, device=dev) * 0.02).to(torch.bfloat16)
 
-    def weights(n, k, seed):
-        gg = torch.Generator(device=dev).manual_seed(seed)
-        q = torch.empty(E, n, k, dtype=torch.float8_e4m3fn, device=dev)
-        s = torch.empty(E, n // 128, k // 128, dtype=torch.float32, device=dev)
-        for e0 in range(0, E, 16):
-            w = (torch.randn(16, n, k, generator=gg, device=dev) * 0.02).to(torch.bfloat16)
-            q[e0:e0 + 16], s[e0:e0 + 16] = pkg.quant_weight_block128(w)
-        return q, s
-
-    w13, w13s = weights(2 * I, H, 1)
-    w2, w2s = weights(H, I, 2)
+    w13, w13s = pkg.synthetic_weights(E, 2 * I, H, dev, 1)
+    w2, w2s = pkg.synthetic_weights(E, H, I, dev, 2)
     logits = torch.matmul(x, wr.t()).float()
     w, ids, scores = pkg.moe_route(logits, K, "sigmoid", None, 8, 4, True, 2.5, return_scores=True)
     w_ref, ids_ref = oracle.select_sigmoid_grouped(scores.cpu(), None, K, 8, 4, 2.5)
@@ -473,8 +513,8 @@ def test_hip_graph_replay_matches_eager(pkg, oracle, dev):
     synchronisation in between, every replay must reproduce the eager bits."""
     say("hip graph")
     T, H, I, E, K = 8, 512, 256, 16, 4
-    layer = tuple(t.to(dev) for t in oracle.make_layer(E, H, I, seed=21))
-    shared = tuple(t.to(dev) for t in oracle.make_layer(1, H, I, seed=22))
+    layer = pkg.pack_layer(*(t.to(dev) for t in oracle.make_layer(E, H, I, seed=21)))
+    shared = pkg.pack_layer(*(t.to(dev) for t in oracle.make_layer(1, H, I, seed=22)))
     g = torch.Generator().manual_seed(23)
     wr = (torch.randn(E, H, generator=g) * 0.02).to(torch.bfloat16).to(dev)
     moe = pkg.FusedMoE(wr, *layer, top_k=K, mode="sigmoid", n_groups=4, topk_groups=2, scale=2.5, shared=shared)
@@ -504,19 +544,7 @@ def test_hip_graph_replay_matches_eager(pkg, oracle, dev):
 
 
 def _layer_on_device(pkg, dev, E, H, I, seed):
-    def weights(n, k, sd):
-        gg = torch.Generator(device=dev).manual_seed(sd)
-        q = torch.empty(E, n, k, dtype=torch.float8_e4m3fn, device=dev)
-        s = torch.empty(E, n // 128, k // 128, dtype=torch.float32, device=dev)
-        step = max(1, (1 << 27) // (n * k))
-        for e0 in range(0, E, step):
-            e1 = min(E, e0 + step)
-            w = (torch.randn(e1 - e0, n, k, generator=gg, device=dev) * 0.02).to(torch.bfloat16)
-            q[e0:e1], s[e0:e1] = pkg.quant_weight_block128(w)
-        return q, s
-    w13, w13s = weights(2 * I, H, seed)
-    w2, w2s = weights(H, I, seed + 1)
-    return w13, w13s, w2, w2s
+    return (*pkg.synthetic_weights(E, 2 * I, H, dev, seed), *pkg.synthetic_weights(E, H, I, dev, seed + 1))
 
 
 def _full_size_checks(pkg, oracle, checks, dev, x, layer, ids, w, pick):

@@ -41,8 +41,8 @@ def test_static_scratch_entry_point_equals_workspace_entry_point(pkg, oracle, de
     say("static scratch", H, I, E, K, mode, G, TG, with_bias, I_sh, T1, T2)
     lib = pkg._lib.lib
     assert lib.moe_hip_init() == 0
-    layer = tuple(t.to(dev) for t in oracle.make_layer(E, H, I, seed=H + E))
-    shared = tuple(t.to(dev) for t in oracle.make_layer(1, H, I_sh, seed=77)) if I_sh else None
+    layer = pkg.pack_layer(*(t.to(dev) for t in oracle.make_layer(E, H, I, seed=H + E)))
+    shared = pkg.pack_layer(*(t.to(dev) for t in oracle.make_layer(1, H, I_sh, seed=77))) if I_sh else None
     g = torch.Generator().manual_seed(E + T1)
     wr = (torch.randn(E, H, generator=g) * 0.05).to(torch.bfloat16).to(dev)
     bias = (torch.randn(E, generator=g) * 0.05).to(dev) if with_bias else None

@@ -5,7 +5,7 @@ module raises, and every op built on it is unavailable.
 """
 import ctypes
 import os
-from ctypes import c_char_p, c_float, c_int, c_size_t, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libmoe_hip.so")
@@ -21,6 +21,8 @@ SIGNATURES = {
                                c_int, c_float, c_void_p, c_void_p, c_void_p]),
     "moe_permute_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "moe_permute": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t]),
+    "moe_pack_weights": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_void_p]),
+    "moe_unpack_weights": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     "moe_scale_pitch": (c_int, [c_int]),
     "moe_act_quant": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p]),
     "moe_fused_experts_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),

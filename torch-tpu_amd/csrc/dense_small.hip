@@ -48,8 +48,9 @@ __global__ __launch_bounds__(256) void dense_small_kernel(const SmallArgs a) {
   if (mc >= a.n_mchunks) return;
   const int kb0 = sp * a.split_len, kb1 = min(kb0 + a.split_len, a.NKB);
   if (kb0 >= kb1) return;
-  // lane (li, lg) holds row li of an operand tile and 16-byte reduction chunks lg and lg + 4
-  const uint8_t *wp = a.w + (size_t)(nt * 16 * NTW + li) * a.K + lg * 16;
+  // lane (li, lg) holds row li of an operand tile and 16-byte reduction chunks lg and lg + 4.  The weights are
+  // stored tile-blocked: a (tile, step) pair is 2 KB in operand order, two halves of [lane][16 bytes]
+  const uint8_t *wp = a.w + (size_t)(nt * 16 * NTW) * a.K + lane * 16;
   const size_t wtile = (size_t)16 * a.K;                 // bytes between consecutive weight tiles
   const float *wsp = a.ws + (size_t)((nt * NTW) >> 3) * a.NKB;   // a group of tiles lies inside one 128-row block
   const uint8_t *xp[MT];
@@ -74,8 +75,8 @@ __global__ __launch_bounds__(256) void dense_small_kernel(const SmallArgs a) {
       const float sb = kb + u < kb1 ? wsp[kk] : 0.f;
 #pragma unroll
       for (int j = 0; j < NTW; j++) {
-        wl[u][j] = *(const v4i *)(wp + j * wtile + (size_t)kk * 128);
-        wh[u][j] = *(const v4i *)(wp + j * wtile + (size_t)kk * 128 + 64);
+        wl[u][j] = *(const v4i *)(wp + j * wtile + (size_t)kk * 2048);
+        wh[u][j] = *(const v4i *)(wp + j * wtile + (size_t)kk * 2048 + 1024);
       }
 #pragma unroll
       for (int mt = 0; mt < MT; mt++) {

@@ -252,9 +252,10 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     wrow = min(wrow, a.n_rows_w - 16);                 // tiles past the matrix re-read its last rows
     wtile[j] = wq + ((size_t)e * a.n_rows_w + wrow) * a.Kd;
   }
-  const uint32_t woff = (uint32_t)li * (uint32_t)a.Kd + lg * 16;   // lane's row and first 16-byte chunk in a tile
-  // direct-to-LDS weight loads: lane l fetches row l/8 (of 8) and the chunk that belongs at position l%8
-  const uint32_t wdma_off = (uint32_t)(lane >> 3) * (uint32_t)a.Kd + (((lane & 7) ^ (lane >> 3)) << 4);
+  // Weights are stored tile-blocked: the 2 KB a (16-row tile, 128-byte step) pair needs are contiguous and already
+  // in operand order - two 1 KB halves of [lane][16 bytes] - so every load instruction of a wavefront reads 1 KB of
+  // consecutive memory (whole cache lines, nothing to shuffle), and a tile's steps follow one another in memory.
+  const uint32_t woff = (uint32_t)lane * 16u;
   // The strip's weight-block scales for all steps go to LDS once (two rows: gate/up blocks for
   // the gated GEMM, the strip's two 128-column blocks otherwise): uniform values re-read per
   // step from LDS instead of through the vector-memory queue.  They are asked for together with
@@ -347,8 +348,8 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   auto request_weights_reg = [&](int kb, v4i(&lo)[WT], v4i(&hi)[WT]) {
 #pragma unroll
     for (int j = 0; j < WT; j++) {
-      const uint8_t *base = wtile[j] + (size_t)kb * 128;
-      asm volatile("global_load_dwordx4 %0, %2, %3\n\tglobal_load_dwordx4 %1, %2, %3 offset:64"
+      const uint8_t *base = wtile[j] + (size_t)kb * 2048;
+      asm volatile("global_load_dwordx4 %0, %2, %3\n\tglobal_load_dwordx4 %1, %2, %3 offset:1024"
                    : "=&v"(lo[j]), "=&v"(hi[j]) : "v"(woff), "s"(base) : "memory");
     }
   };
@@ -373,17 +374,16 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   auto request = [&](int kb, int stage) {
 #pragma unroll
     for (int u = 0; u < NTOK; u++) request_tok(kb, stage, u);
-    // weight tiles through LDS: like the token tile, an instruction moves 8 whole rows x 128 bytes
-    // (every cache line it touches is used completely) into swizzled [row][16-byte chunk] order
+    // weight tiles through LDS: an instruction copies one 1 KB half of a tile's step as it lies in memory
     if (!WREG)
 #pragma unroll
     for (int j = 0; j < WT; j++) {
-      const uint8_t *base = wtile[j] + (size_t)kb * 128;
-      const uint8_t *base8 = base + (size_t)8 * a.Kd;
+      const uint8_t *base = wtile[j] + (size_t)kb * 2048;
       const uint32_t m0 = wt_base + stage * kWtStage + j * 2048;
+      // the instruction offset advances the memory address and the LDS address alike
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t"
-                   "s_add_u32 m0, m0, 0x400\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %3"
-                   ::"s"(m0), "v"(wdma_off), "s"(base), "s"(base8) : "memory", "m0", "scc");
+                   "global_load_lds_dwordx4 %1, %2 offset:1024"
+                   ::"s"(m0), "v"(woff), "s"(base) : "memory", "m0");
     }
   };
 
@@ -394,12 +394,11 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   constexpr int MG = MT < 4 ? MT : (MT % 4 == 0 && MT <= 8 ? 4 : (DEPTH >= 3 ? 2 : 3));
   auto compute = [&](int stage, int kb, const v4i(&lo)[WT], const v4i(&hi)[WT]) {
     v8i wc[WT];
-    const uint8_t *wbase = sm.wt[WREG ? 0 : stage] + wave * (WT * 2048) + li * 128;
+    const uint8_t *wbase = sm.wt[WREG ? 0 : stage] + wave * (WT * 2048) + lane * 16;
 #pragma unroll
     for (int j = 0; j < WT; j++) {
       if (WREG) wc[j] = concat8(lo[j], hi[j]);
-      else wc[j] = concat8(*(const v4i *)(wbase + j * 2048 + ((lg ^ (li & 7)) << 4)),
-                           *(const v4i *)(wbase + j * 2048 + (((lg + 4) ^ (li & 7)) << 4)));
+      else wc[j] = concat8(*(const v4i *)(wbase + j * 2048), *(const v4i *)(wbase + j * 2048 + 1024));
     }
     const float s0 = BF16 ? 0.f : sm.sb[sb_row0][kb], s1 = BF16 ? 0.f : sm.sb[sb_row1][kb];
     const uint8_t *tbase = sm.tok[stage] + li * 128;

@@ -1,7 +1,8 @@
-// The two bandwidth-bound elementwise stages around the grouped GEMMs:
+// The bandwidth-bound elementwise stages around the grouped GEMMs:
 //   act_quant        bf16 [R, C] -> e4m3fn [R, C] + fp32 scale per row per 128 columns
 //   weighted_reduce  bf16 [T, K, H] per-slot results -> bf16 [T, H], fp32 weighted sum
-// Both move 16 bytes per lane per access; rows are contiguous so every access is coalesced.
+//   repack_weights   weight bytes row-major <-> tile-blocked (once, when a checkpoint is loaded)
+// All move 16 bytes per lane per access; rows are contiguous so every access is coalesced.
 #include "moe_common.h"
 #include "moe_layout.h"
 #include "act_quant.h"
@@ -77,6 +78,40 @@ __global__ __launch_bounds__(256) void zero_dropped_rows_kernel(const int32_t *_
   for (int i = 0; i < H / 8; i++) row[i] = (v4i){0, 0, 0, 0};
 }
 
+// Weight bytes between row-major order and the tile-blocked order the GEMMs read.  Tile-blocked: the matrix is cut
+// into tiles of 16 rows and steps of 128 bytes; the 2 KB of a (tile, step) pair are contiguous, tiles in row order,
+// a tile's steps one after the other, and inside the 2 KB: half h (0/1), then lane l (0..63), 16 bytes each =
+// row l % 16 of the tile, bytes 16 * (l / 16 + 4 h) .. + 15 of the step - a wavefront's operand of the 16x16x128
+// matrix instruction, so that a load instruction reads 1 KB of consecutive memory.  One thread moves 16 bytes;
+// the tile-blocked side is the coalesced one.
+__global__ __launch_bounds__(256) void repack_weights_kernel(const v4i *__restrict__ src, v4i *__restrict__ dst,
+                                                             size_t n_units, int nkb, int row_units, bool to_blocked) {
+  const size_t o = (size_t)blockIdx.x * 256 + threadIdx.x;      // 16-byte unit in tile-blocked order
+  if (o >= n_units) return;
+  const size_t block = o >> 7;
+  const int u = (int)(o & 127), h = u >> 6, l = u & 63, r = l & 15, g = l >> 4;
+  const size_t tile = block / nkb;
+  const int kb = (int)(block % nkb);
+  const size_t rm = (tile * 16 + r) * (size_t)row_units + (size_t)kb * 8 + g + 4 * h;   // the same unit in row-major order
+  if (to_blocked) dst[o] = src[rm];
+  else dst[rm] = src[o];
+}
+
+static int repack_launch(hipStream_t st, const void *src, int64_t rows, int row_bytes, void *dst, bool to_blocked) {
+  if (rows < 0 || row_bytes < 1) return MOE_E_SHAPE;
+  if (rows % 16 || row_bytes % kBlock) return MOE_E_ALIGN;
+  if (rows == 0) return MOE_OK;
+  if (!src || !dst) return MOE_E_NULL;
+  if (src == dst) return MOE_E_MODE;                             // not an in-place operation
+  if (((uintptr_t)src % 16) || ((uintptr_t)dst % 16)) return MOE_E_ALIGN;
+  const size_t n_units = (size_t)rows * (row_bytes / 16);
+  const size_t blocks = (n_units + 255) / 256;
+  if (blocks > 0x7fffffffull) return MOE_E_SHAPE;
+  repack_weights_kernel<<<(unsigned)blocks, 256, 0, st>>>((const v4i *)src, (v4i *)dst, n_units, row_bytes / kBlock,
+                                                          row_bytes / 16, to_blocked);
+  return (int)hipGetLastError();
+}
+
 int zero_dropped_rows_launch(hipStream_t st, const int32_t *slot_to_row, int TK, int H, uint16_t *y) {
   if (TK < 1) return MOE_OK;
   zero_dropped_rows_kernel<<<(TK + 255) / 256, 256, 0, st>>>(slot_to_row, TK, H, y);
@@ -95,6 +130,14 @@ int weighted_reduce_launch(hipStream_t st, const uint16_t *y, const float *w, co
 }
 
 }  // namespace moe
+
+extern "C" int moe_pack_weights(void *stream, const void *w_rowmajor, int64_t rows, int row_bytes, void *w_blocked) {
+  return moe::repack_launch((hipStream_t)stream, w_rowmajor, rows, row_bytes, w_blocked, true);
+}
+
+extern "C" int moe_unpack_weights(void *stream, const void *w_blocked, int64_t rows, int row_bytes, void *w_rowmajor) {
+  return moe::repack_launch((hipStream_t)stream, w_blocked, rows, row_bytes, w_rowmajor, false);
+}
 
 extern "C" int moe_scale_pitch(int n_groups) { return n_groups < 0 ? 0 : moe::scale_pitch(n_groups); }
 

@@ -3,9 +3,10 @@
 The reference passes three separate weight tensors per call: gate [E,I,H], up [E,I,H] and a
 PRE-TRANSPOSED down [E,I,H], with bf16 block scales of matching orientation
 (python/regression/test_llm/test_moe.py:285-288).  The kernels here want the reduction
-dimension contiguous for both GEMMs, so weights are packed once, at load time:
-W13 = gate rows followed by up rows [E,2I,H], W2 = down in its checkpoint orientation
-[E,H,I], scales widened to fp32.
+dimension contiguous for both GEMMs and the weight bytes in matrix-instruction operand order, so
+weights are packed once, at load time: W13 = gate rows followed by up rows [E,2I,H], W2 = down in
+its checkpoint orientation [E,H,I], scales widened to fp32, then the bytes of W13 and W2 tile-blocked
+(ops.pack_weights).
 """
 from __future__ import annotations
 
@@ -14,14 +15,21 @@ import torch
 from . import ops
 
 
-def pack_expert_weights(gate, up, down_t, gate_scale, up_scale, down_t_scale):
-    """Reference-layout fp8 weights -> (w13, w13_scale, w2, w2_scale) in kernel layout.
-    Pure data movement (concatenate / transpose / widen); values are untouched."""
+def stack_expert_weights(gate, up, down_t, gate_scale, up_scale, down_t_scale):
+    """Reference-layout fp8 weights -> (w13, w13_scale, w2, w2_scale), ROW-MAJOR: gate rows followed by up rows,
+    down back in its checkpoint orientation, scales widened to fp32.  Pure data movement (concatenate / transpose /
+    widen) on whatever device the tensors live; values are untouched."""
     w13 = torch.cat([gate, up], dim=1).contiguous()
     w13_scale = torch.cat([gate_scale, up_scale], dim=1).to(torch.float32).contiguous()
     w2 = down_t.transpose(1, 2).contiguous()
     w2_scale = down_t_scale.transpose(1, 2).to(torch.float32).contiguous()
     return w13, w13_scale, w2, w2_scale
+
+
+def pack_expert_weights(gate, up, down_t, gate_scale, up_scale, down_t_scale):
+    """Reference-layout fp8 weights on the GPU -> (w13, w13_scale, w2, w2_scale) in kernel layout: stacked as
+    stack_expert_weights does, then the weight bytes tile-blocked (ops.pack_weights).  Values are untouched."""
+    return ops.pack_layer(*stack_expert_weights(gate, up, down_t, gate_scale, up_scale, down_t_scale))
 
 
 def quant_weight_block128(w: torch.Tensor):
@@ -38,8 +46,25 @@ def quant_weight_block128(w: torch.Tensor):
     return q.reshape(*lead, N, K), scale
 
 
-def convert_hf_moe_layer(state: dict, prefix: str, num_experts: int, device=None):
+def synthetic_weights(n_experts: int, n: int, k: int, device, seed: int, std: float = 0.02, tile_block: bool = True):
+    """Random weights [n_experts, n, k] ~ N(0, std) in bf16, quantised to e4m3fn with fp32 128x128 block scales on
+    `device`, in slices of experts (the fp32 intermediates of a whole layer are large) -> (codes, scales); the codes
+    tile-blocked unless tile_block=False.  For benchmarks and tests: there are no checkpoints offline."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    q = torch.empty(n_experts, n, k, dtype=torch.float8_e4m3fn, device=device)
+    s = torch.empty(n_experts, n // 128, k // 128, dtype=torch.float32, device=device)
+    step = max(1, (1 << 27) // (n * k))
+    for e0 in range(0, n_experts, step):
+        e1 = min(n_experts, e0 + step)
+        w = (torch.randn(e1 - e0, n, k, generator=g, device=device) * std).to(torch.bfloat16)
+        q[e0:e1], s[e0:e1] = quant_weight_block128(w)
+    return (ops.pack_weights(q) if tile_block else q), s
+
+
+def convert_hf_moe_layer(state: dict, prefix: str, num_experts: int, device=None, tile_block: bool = True):
     """Checkpoint tensors of one DeepSeek-V3-style FP8 MoE layer -> the packed layout of the kernels.
+    tile_block=False stops before the last step (re-ordering the weight bytes on the GPU, ops.pack_weights) and
+    returns the stacked row-major tensors, on any device.
 
     Reads `{prefix}experts.{e}.{gate,up,down}_proj.weight` (e4m3fn `[out, in]`) and the matching
     `.weight_scale_inv` (fp32 `[ceil(out/128), ceil(in/128)]`, the value a block is MULTIPLIED by),
@@ -72,6 +97,10 @@ def convert_hf_moe_layer(state: dict, prefix: str, num_experts: int, device=None
     bias = state.get(prefix + "gate.e_score_correction_bias")
     if bias is not None:
         bias = (bias.to(device) if device is not None else bias).to(torch.float32).contiguous()
+    if tile_block:
+        w13, w2 = ops.pack_weights(w13), ops.pack_weights(w2)
+        if shared is not None:
+            shared = ops.pack_layer(*shared)
     return dict(router_weight=get("gate.weight").to(torch.bfloat16).contiguous(), bias=bias, w13=w13, w13_scale=w13_scale,
                 w2=w2, w2_scale=w2_scale, shared=shared)
 
@@ -86,6 +115,7 @@ class FusedMoE:
 
     def __init__(self, router_weight, w13, w13_scale, w2, w2_scale, top_k, mode="softmax", bias=None,
                  n_groups=1, topk_groups=1, renorm=True, scale=1.0, shared=None):
+        # w13 / w2 (and the shared expert's) are tile-blocked: ops.pack_weights / pack_expert_weights / convert_hf_moe_layer
         self.router_weight = router_weight          # [E, H] bf16
         self.w13, self.w13_scale, self.w2, self.w2_scale = w13, w13_scale, w2, w2_scale
         self.top_k, self.mode, self.bias = top_k, mode, bias

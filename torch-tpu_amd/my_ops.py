@@ -7,6 +7,8 @@ Schemas follow the reference's C++ declarations (torch_tpu/csrc/ops/my_ops/ops.h
 """
 from __future__ import annotations
 
+import weakref
+
 import torch
 
 from . import ops
@@ -31,6 +33,15 @@ _lib.define("noaux_tc_topk(Tensor(a!) values, Tensor(b!) indices, Tensor scores,
 _lib.define("fused_moe_grouped_topk(Tensor topk_experts_res, Tensor topk_weights_res_bf16, Tensor left_bf16, "
             "Tensor right_bf16, Tensor topk_weights_res, Tensor left, Tensor right, Tensor max, Tensor matmul_res, "
             "Tensor softmax_res) -> Tensor")
+
+# What the reference leaves to its callers or to closed code, as ops of the same namespace: the router recipe
+# (python/regression/test_llm/test_torch_ops.py:440-456), the index building of the expert kernel
+# (torch_tpu/csrc/ops/my_ops/fusedMoE.pl:624-756) and the weight re-layout (test_moe.py:285-288).
+_lib.define("moe_route(Tensor x, Tensor router_weight, Tensor? bias, str mode, int top_k, int n_group, int topk_group, "
+            "float scale, bool renorm) -> (Tensor, Tensor)")
+_lib.define("moe_permute(Tensor ids, int num_experts) -> (Tensor, Tensor, Tensor)")
+_lib.define("moe_pack_weights(Tensor gate_weights, Tensor up_weights, Tensor down_weights, Tensor gate_scales, "
+            "Tensor up_scales, Tensor down_scales) -> (Tensor, Tensor, Tensor, Tensor)")
 
 _lib.define("mlp_w8a16_dq_forward(Tensor input, Tensor gate_weight, Tensor up_weight, Tensor down_weight, "
             "Tensor gate_scale, Tensor up_scale, Tensor down_scale, Tensor(a!) output, int blocksize) -> Tensor(a!)")
@@ -60,33 +71,89 @@ def _dequant_bf16(w, s, blocksize=128):
     return (w.to(torch.float32) * full.to(torch.float32)).to(torch.bfloat16)
 
 
-# packed copies of reference-layout weights, keyed by the identity of the six tensors
-_pack_cache: dict = {}
+class _DerivedCache:
+    """Tensors derived from a caller's weight tensors (packed / de-quantised copies), kept for as long as the
+    sources live.
+
+    An entry belongs to the source tensor OBJECTS: it holds weak references to them, is found through their ids, is
+    valid only while every reference still resolves to the very tensor handed in and address, version counter, shape,
+    stride, dtype and device are what they were, and is dropped by a finaliser the moment one of the sources is
+    freed - so new weights that land on a recycled address never meet an old copy, and a model with many layers keeps
+    one entry per layer (nothing is evicted by count).  An in-place write through `.data` does not move the version
+    counter and cannot be seen from here: call `invalidate_weight_cache()` after such an update (or pack explicitly
+    with pack_expert_weights and call torch_tpu_amd.fused_experts_fp8 / FusedMoE).  The derived copy doubles the weight
+    memory unless the caller drops the originals."""
+
+    def __init__(self):
+        self._entries = {}
+
+    @staticmethod
+    def _signature(tensors):
+        return tuple((t.data_ptr(), t._version, tuple(t.shape), tuple(t.stride()), t.dtype, t.device) for t in tensors)
+
+    def get(self, tensors, tag, make):
+        key = (tag,) + tuple(id(t) for t in tensors)
+        entry = self._entries.get(key)
+        if entry is not None:
+            refs, sig, value = entry
+            if all(r() is t for r, t in zip(refs, tensors)) and sig == self._signature(tensors):
+                return value
+        value = make()
+        drop = lambda _ref, k=key, d=self._entries: d.pop(k, None)
+        self._entries[key] = ([weakref.ref(t, drop) for t in tensors], self._signature(tensors), value)
+        return value
+
+    def clear(self):
+        self._entries.clear()
+
+    def __len__(self):
+        return len(self._entries)
 
 
-_dense_cache: dict = {}
+_weights = _DerivedCache()
 
 
-def _dense_packed(key_tensors, make):
-    key = tuple((t.data_ptr(), t._version, tuple(t.shape), tuple(t.stride())) for t in key_tensors)
-    hit = _dense_cache.get(key)
-    if hit is None:
-        if len(_dense_cache) > 32:
-            _dense_cache.clear()
-        hit = make()
-        _dense_cache[key] = hit
-    return hit
+def invalidate_weight_cache() -> None:
+    """Forget every packed / de-quantised copy made for the drop-in ops (needed after weights were overwritten in place
+    through `.data`, which no version counter records)."""
+    _weights.clear()
+
+
+def _dense_packed(key_tensors, make, tag="dense"):
+    return _weights.get(tuple(key_tensors), tag, make)
 
 
 def _packed(gate, up, down, gs, us, ds):
-    key = tuple((t.data_ptr(), t._version, tuple(t.shape)) for t in (gate, up, down, gs, us, ds))
-    hit = _pack_cache.get(key)
-    if hit is None:
-        if len(_pack_cache) > 8:
-            _pack_cache.clear()
-        hit = pack_expert_weights(gate, up, down, gs, us, ds)
-        _pack_cache[key] = hit
-    return hit
+    return _weights.get((gate, up, down, gs, us, ds), "experts", lambda: pack_expert_weights(gate, up, down, gs, us, ds))
+
+
+# One scratch tensor per (device, stream), grown on demand: the ops allocate nothing once it is large enough.
+# Calls that share it are ordered by the stream they were enqueued on.
+_scratch: dict = {}
+
+
+def _workspace(device, nbytes: int):
+    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    ws = _scratch.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _scratch[key] = ws
+    return ws
+
+
+def _routing_f32(routing_weights, device):
+    """The op's routing weights (bf16 in the reference's callers) as fp32 for the weighted sum, in a buffer that is
+    kept per (device, stream) next to the workspace."""
+    if routing_weights.dtype == torch.float32 and routing_weights.is_contiguous():
+        return routing_weights
+    key = (device, torch.cuda.current_stream(device).cuda_stream, "rw")
+    buf = _scratch.get(key)
+    if buf is None or buf.numel() < routing_weights.numel():
+        buf = torch.empty(max(routing_weights.numel(), 4096), dtype=torch.float32, device=device)
+        _scratch[key] = buf
+    out = buf[:routing_weights.numel()].view(routing_weights.shape)
+    out.copy_(routing_weights)
+    return out
 
 
 def _fused_experts(output, input, output_sample, input_sample, gate_weights, up_weights, down_weights,
@@ -110,13 +177,11 @@ def _fused_experts(output, input, output_sample, input_sample, gate_weights, up_
             if t.dtype != torch.bfloat16:
                 raise RuntimeError("weights without scales must be bfloat16")
         w13, w2 = _dense_packed((gate_weights, up_weights, down_weights),
-                                lambda: (torch.cat([gate_weights, up_weights], dim=1).contiguous(),
-                                         down_weights.transpose(1, 2).contiguous()))
+                                lambda: (ops.pack_weights(torch.cat([gate_weights, up_weights], dim=1).contiguous()),
+                                         ops.pack_weights(down_weights.transpose(1, 2).contiguous())), "bf16")
         if w13.shape[0] != num_experts or select_experts.shape[1] != num_experts_per_tok:
             raise RuntimeError("num_experts / num_experts_per_tok do not match the tensors")
-        rw = routing_weights.to(torch.float32) if output.dim() == 2 else None
-        ops.fused_experts_bf16(input, w13, w2, select_experts, rw, out=output)
-        return output
+        return _run_bf16(output, input, w13, w2, select_experts, routing_weights)
     if gate_scales is None or up_scales is None or down_scales is None:
         raise RuntimeError("either all three weight tensors carry block scales or none does")
     if blocksize < 1:
@@ -125,25 +190,37 @@ def _fused_experts(output, input, output_sample, input_sample, gate_weights, up_
     if _numerics == "w8a16" or blocksize % 128:
         w13, w2 = _dense_packed(
             (gate_weights, up_weights, down_weights, gate_scales, up_scales, down_scales),
-            lambda: (torch.cat([_dequant_bf16(gate_weights, gate_scales, blocksize),
-                                _dequant_bf16(up_weights, up_scales, blocksize)], 1).contiguous(),
-                     _dequant_bf16(down_weights, down_scales, blocksize).transpose(1, 2).contiguous()))
-        rw = routing_weights.to(torch.float32) if output.dim() == 2 else None
-        ops.fused_experts_bf16(input, w13, w2, select_experts, rw, out=output)
-        return output
+            lambda: (ops.pack_weights(torch.cat([_dequant_bf16(gate_weights, gate_scales, blocksize),
+                                                 _dequant_bf16(up_weights, up_scales, blocksize)], 1).contiguous()),
+                     ops.pack_weights(_dequant_bf16(down_weights, down_scales, blocksize).transpose(1, 2).contiguous())),
+            f"dequant{blocksize}")
+        return _run_bf16(output, input, w13, w2, select_experts, routing_weights)
     if blocksize != 128:
         # a multiple of 128: every 128-block takes the scale of the block it lies in (the same products, exactly)
         I, H = gate_weights.shape[1:]
-        gate_scales, up_scales, down_scales = _dense_packed(
-            (gate_scales, up_scales, down_scales),
-            lambda: tuple(_scales_128(t, blocksize, I, H) for t in (gate_scales, up_scales, down_scales)))
-    w13, w13s, w2, w2s = _packed(gate_weights, up_weights, down_weights, gate_scales, up_scales, down_scales)
+        scales = (gate_scales, up_scales, down_scales)
+        w13, w13s, w2, w2s = _dense_packed(
+            (gate_weights, up_weights, down_weights, *scales),
+            lambda: pack_expert_weights(gate_weights, up_weights, down_weights,
+                                        *(_scales_128(t, blocksize, I, H) for t in scales)), f"experts{blocksize}")
+    else:
+        w13, w13s, w2, w2s = _packed(gate_weights, up_weights, down_weights, gate_scales, up_scales, down_scales)
     if w13.shape[0] != num_experts or select_experts.shape[1] != num_experts_per_tok:
         raise RuntimeError("num_experts / num_experts_per_tok do not match the tensors")
-    rw = None
-    if output.dim() == 2:
-        rw = routing_weights.to(torch.float32)
-    ops.fused_experts_fp8(input, w13, w13s, w2, w2s, select_experts, rw, out=output)
+    T, H = input.shape
+    E, I2, _ = w13.shape
+    rw = _routing_f32(routing_weights, input.device) if output.dim() == 2 else None
+    ws = _workspace(input.device, ops.fused_experts_workspace_bytes(T, H, I2 // 2, E, select_experts.shape[1]))
+    ops.fused_experts_fp8(input, w13, w13s, w2, w2s, select_experts, rw, out=output, workspace=ws)
+    return output
+
+
+def _run_bf16(output, input, w13, w2, select_experts, routing_weights):
+    T, H = input.shape
+    E, I2, _ = w13.shape
+    rw = _routing_f32(routing_weights, input.device) if output.dim() == 2 else None
+    ws = _workspace(input.device, ops.fused_experts_bf16_workspace_bytes(T, H, I2 // 2, E, select_experts.shape[1]))
+    ops.fused_experts_bf16(input, w13, w2, select_experts, rw, out=output, workspace=ws)
     return output
 
 
@@ -162,6 +239,33 @@ def _fused_experts_v2(output, input, output_sample, input_sample, gate_weights, 
 def _grouped_topk(*args):
     raise RuntimeError("fused_moe_grouped_topk: the reference's fused router is closed-source, untested and "
                        "undocumented; use noaux_tc_topk or torch_tpu_amd.moe_route instead")
+
+
+def _moe_route(x, router_weight, bias, mode, top_k, n_group, topk_group, scale, renorm):
+    """Router of one layer: logits = x . router_weight^T (bf16, fp32 sums rounded once), then top-k selection and
+    weights -> (fp32 weights [T, top_k], int32 ids [T, top_k]).  mode "softmax" | "sigmoid"; bias [E] fp32 takes part in
+    the selection only (a softmax router's bias is added to the logits)."""
+    if x.dim() != 2 or router_weight.dim() != 2 or x.shape[1] != router_weight.shape[1]:
+        raise RuntimeError("x must be [T, H] and router_weight [E, H]")
+    E, H = router_weight.shape
+    if x.dtype == torch.bfloat16 and router_weight.dtype == torch.bfloat16 and E <= 256 and H % 128 == 0:
+        ws = _workspace(x.device, ops.router_logits_workspace_bytes(x.shape[0], H, E))
+        logits = ops.router_logits(x.contiguous(), router_weight.contiguous(), workspace=ws)
+    else:
+        logits = torch.matmul(x, router_weight.t()).contiguous()
+        if logits.dtype not in (torch.float32, torch.bfloat16):
+            logits = logits.float()
+    if mode == "softmax" and bias is not None:
+        logits, bias = (logits.float() + bias), None
+    return ops.moe_route(logits, top_k, mode, bias, n_group, topk_group, renorm, scale)
+
+
+def _moe_permute(ids, num_experts):
+    return ops.moe_permute(ids, num_experts)
+
+
+def _moe_pack_weights(gate_weights, up_weights, down_weights, gate_scales, up_scales, down_scales):
+    return pack_expert_weights(gate_weights, up_weights, down_weights, gate_scales, up_scales, down_scales)
 
 
 def _check_dense(blocksize, *fp8):
@@ -199,9 +303,10 @@ def _mlp_w8a16_dq_forward(input, gate_weight, up_weight, down_weight, gate_scale
     if blocksize % 128:
         w13, w2 = _dense_packed(
             (gate_weight, up_weight, down_weight, gate_scale, up_scale, down_scale),
-            lambda: (torch.cat([_dequant_any(gate_weight, gate_scale, blocksize),
-                                _dequant_any(up_weight, up_scale, blocksize)], 0).unsqueeze(0).contiguous(),
-                     _dequant_any(down_weight, down_scale, blocksize).t().unsqueeze(0).contiguous()))
+            lambda: (ops.pack_weights(torch.cat([_dequant_any(gate_weight, gate_scale, blocksize),
+                                                 _dequant_any(up_weight, up_scale, blocksize)], 0).unsqueeze(0).contiguous()),
+                     ops.pack_weights(_dequant_any(down_weight, down_scale, blocksize).t().unsqueeze(0).contiguous())),
+            f"mlp-dequant{blocksize}")
         # one expert that every row selects; its per-slot result [M, 1, H] is the output itself
         M = input.shape[0]
         ids = torch.zeros(M, 1, dtype=torch.int32, device=input.device)
@@ -209,10 +314,12 @@ def _mlp_w8a16_dq_forward(input, gate_weight, up_weight, down_weight, gate_scale
         return output
     w13, w13s, w2, w2s = _dense_packed(
         (gate_weight, up_weight, down_weight, gate_scale, up_scale, down_scale),
-        lambda: (torch.cat([gate_weight, up_weight], 0).contiguous(),
+        lambda: (ops.pack_weights(torch.cat([gate_weight, up_weight], 0).contiguous()),
                  torch.cat([_scales_128(gate_scale, blocksize, I, H), _scales_128(up_scale, blocksize, I, H)], 0).contiguous(),
-                 down_weight.t().contiguous(), _scales_128(down_scale, blocksize, I, H).t().contiguous()))
-    ops.mlp_fp8(input.contiguous(), w13, w13s, w2, w2s, out=output)
+                 ops.pack_weights(down_weight.t().contiguous()), _scales_128(down_scale, blocksize, I, H).t().contiguous()),
+        f"mlp{blocksize}")
+    ws = _workspace(input.device, ops.mlp_workspace_bytes(input.shape[0], H, I))
+    ops.mlp_fp8(input.contiguous(), w13, w13s, w2, w2s, out=output, workspace=ws)
     return output
 
 
@@ -222,11 +329,13 @@ def _mm_w8a16_dq_forward(input, weight, scale, output, blocksize):
     _check_dense(blocksize, weight)
     N, K = weight.shape
     if blocksize % 128:
-        (w,) = _dense_packed((weight, scale), lambda: (_dequant_any(weight, scale, blocksize),))
+        (w,) = _dense_packed((weight, scale), lambda: (ops.pack_weights(_dequant_any(weight, scale, blocksize)),),
+                             f"mm-dequant{blocksize}")
         ops.mm_bf16(input.contiguous(), w, out=output)
         return output
-    w, ws = _dense_packed((weight, scale), lambda: (weight.contiguous(), _scales_128(scale, blocksize, N, K)))
-    ops.mm_fp8(input.contiguous(), w, ws, out=output)
+    w, ws = _dense_packed((weight, scale), lambda: (ops.pack_weights(weight.contiguous()),
+                                                     _scales_128(scale, blocksize, N, K)), f"mm{blocksize}")
+    ops.mm_fp8(input.contiguous(), w, ws, out=output, workspace=_workspace(input.device, ops.mm_workspace_bytes(input.shape[0], K, N)))
     return output
 
 
@@ -236,3 +345,6 @@ _lib.impl("mm_w8a16_dq_forward", _mm_w8a16_dq_forward, "CompositeExplicitAutogra
 _lib.impl("fused_moe_fused_experts_v2", _fused_experts_v2, "CompositeExplicitAutograd")
 _lib.impl("noaux_tc_topk", ops.noaux_tc_topk, "CompositeExplicitAutograd")
 _lib.impl("fused_moe_grouped_topk", _grouped_topk, "CompositeExplicitAutograd")
+_lib.impl("moe_route", _moe_route, "CompositeExplicitAutograd")
+_lib.impl("moe_permute", _moe_permute, "CompositeExplicitAutograd")
+_lib.impl("moe_pack_weights", _moe_pack_weights, "CompositeExplicitAutograd")

@@ -144,6 +144,36 @@ def act_quant(x):
     return q, s
 
 
+# --------------------------------------------------------------------------- weight layout
+def _repack(w, fn, what):
+    _need(isinstance(w, torch.Tensor) and w.dim() >= 2, f"{what}: weights must be [..., N, K]")
+    _need(w.dtype in (_FP8, torch.bfloat16, torch.uint8), f"{what}: weights must be float8_e4m3fn, bfloat16 or uint8")
+    N, K = w.shape[-2:]
+    row_bytes = K * w.element_size()
+    _need(N % 16 == 0 and row_bytes % 128 == 0, f"{what}: N must be a multiple of 16 and a row a multiple of 128 bytes")
+    out = torch.empty_like(w)
+    rows = w.numel() // K if K else 0
+    check(fn(_stream(), _dev(w, "w"), rows, row_bytes, out.data_ptr()), what)
+    return out
+
+
+def pack_weights(w):
+    """Row-major weights [..., N, K] on the GPU (N a multiple of 16, a row a multiple of 128 bytes) -> a tensor of the
+    same shape and dtype whose bytes are in the tile-blocked order every GEMM entry point reads (see
+    include/moe_hip.h).  Done once, when weights are loaded."""
+    return _repack(w, lib.moe_pack_weights, "pack_weights")
+
+
+def unpack_weights(w):
+    """The inverse of pack_weights: tile-blocked bytes -> row-major."""
+    return _repack(w, lib.moe_unpack_weights, "unpack_weights")
+
+
+def pack_layer(w13, w13_scale, w2, w2_scale):
+    """(w13, w13_scale, w2, w2_scale) with row-major weights on the GPU -> the same with tile-blocked weights."""
+    return pack_weights(w13), w13_scale, pack_weights(w2), w2_scale
+
+
 # --------------------------------------------------------------------------- experts
 def _shared_args(shared, H: int):
     """(four device pointers, intermediate size) of an optional shared expert
@@ -168,7 +198,7 @@ def fused_experts_fp8(x, w13, w13_scale, w2, w2_scale, ids, routing_weights=None
     """The expert computation on packed weights.
 
     x [T,H] bf16; w13 [E,2I,H] e4m3fn + fp32 scales [E,2I/128,H/128]; w2 [E,H,I] e4m3fn + fp32
-    scales [E,H/128,I/128]; ids [T,K] int32.
+    scales [E,H/128,I/128], both weight tensors TILE-BLOCKED (pack_weights); ids [T,K] int32.
     out [T,K,H] bf16: un-weighted per-slot results.  out [T,H] bf16: weighted sum over the
     slots (routing_weights fp32 [T,K] required), plus the shared expert
     shared=(w13 [1,2Is,H], w13_scale, w2 [1,H,Is], w2_scale) if given.
@@ -292,6 +322,22 @@ def layer_fp8(x, router_weight, w13, w13_scale, w2, w2_scale, top_k: int, mode: 
         rc = lib.moe_layer_fp8(*args, _dev(workspace, "workspace"), workspace.numel() * workspace.element_size())
     check(rc, "layer_fp8")
     return (out, logits, weights, ids) if return_routing else out
+
+
+def fused_experts_bf16_workspace_bytes(T, H, I, E, K) -> int:
+    return lib.moe_fused_experts_bf16_workspace_bytes(T, H, I, E, K)
+
+
+def mm_workspace_bytes(M, K, N) -> int:
+    return lib.moe_mm_fp8_workspace_bytes(M, K, N)
+
+
+def mlp_workspace_bytes(M, H, I) -> int:
+    return lib.moe_mlp_fp8_workspace_bytes(M, H, I)
+
+
+def router_logits_workspace_bytes(T, H, E) -> int:
+    return lib.moe_router_logits_workspace_bytes(T, H, E)
 
 
 def fused_experts_bf16(x, w13, w2, ids, routing_weights=None, out=None, workspace=None):
@@ -429,4 +475,5 @@ def weighted_reduce(y, routing_weights, shared_y=None, out=None):
 
 
 __all__ = ["MoeHipError", "noaux_tc_topk", "moe_route", "moe_permute", "act_quant", "fused_experts_fp8",
+           "pack_weights", "unpack_weights", "pack_layer",
            "fused_experts_workspace_bytes", "gemm1_swiglu", "gemm2", "weighted_reduce", "tile_rows"]
