@@ -14,6 +14,7 @@ Prints ONE JSON line.  `value` = algorithmic FP8-GEMM TFLOP/s of the whole step,
 import argparse
 import json
 import os
+import platform
 import sys
 import time
 
@@ -26,8 +27,35 @@ import __graft_entry__ as entry  # noqa: E402
 PEAK_FP8_TFLOPS = 5000.0      # MI355X dense FP8 MFMA, TFLOP/s
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E, GB/s
 
-# (T, H, I, E, K) -> HBM bytes per launch of the first grouped GEMM over the routed experts
-MEASURED_TRAFFIC = {(4096, 7168, 2048, 256, 8): 7.830e9}
+KERNEL_SOURCES = ("gemm_fp8.hip", "moe_layout.h", "moe_common.h")   # what the dominant kernel is compiled from
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "grouped_gemm_c3_prefill.txt")
+
+
+def kernel_source_hash():
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "torch-tpu_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def offline_traffic(shape):
+    """HBM bytes per launch of the first grouped GEMM as two `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE) counted
+    them, read from the line `TRAFFIC {...}` of the committed profile summary.  That is an OFFLINE measurement: it is
+    handed on only when the summary was made from the kernel sources this run was built from (same hash) and for this
+    workload's shape; otherwise the figure is None and the source says why."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            rec = next(json.loads(line.split(None, 1)[1]) for line in f if line.startswith("TRAFFIC "))
+    except (OSError, StopIteration, ValueError):
+        return None, "no TRAFFIC line in profiles/grouped_gemm_c3_prefill.txt"
+    rel = os.path.relpath(TRAFFIC_FILE, ROOT)
+    if tuple(rec.get("shape", ())) != tuple(shape):
+        return None, f"{rel} covers another workload"
+    if rec.get("kernel_source_sha16") != kernel_source_hash():
+        return None, f"{rel} was measured on other kernel sources ({rec.get('kernel_source_sha16')}): stale, not reported"
+    return rec["bytes_per_launch"], f"{rel} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, offline, kernel sources {rec['kernel_source_sha16']})"
 
 WORKLOADS = {
     # the headline configuration: DeepSeek-V3-shaped prefill layer
@@ -164,9 +192,9 @@ def bench_prefill(pkg, moe, cfg, dev, steps, warmup):
     else:
         roof = dict(bound="mfma", achieved=f1 / k1 / 1e12, peak=PEAK_FP8_TFLOPS, unit="TFLOP/s")
     roof["frac"] = roof["achieved"] / roof["peak"]
-    # HBM bytes per launch of this kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a plain
-    # elementwise kernel of known size, see profiles/grouped_gemm_c3_prefill.txt); only known for the profiled workload
-    roof["traffic"] = MEASURED_TRAFFIC.get((T, H, I, E, K))
+    # HBM bytes per launch of this kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a plain elementwise
+    # kernel of known size): an offline figure, only for the profiled workload and only while the kernel is unchanged
+    roof["traffic"], roof["traffic_source"] = offline_traffic((T, H, I, E, K))
     roof.update(kernel="grouped_gemm_kernel<gated> (W13 GEMM + SwiGLU + requant)", launch_ms=k1 * 1e3,
                 algorithmic_bytes=b1, algorithmic_flops=f1, flop_per_byte=intensity,
                 mfma_tflops=f1 / k1 / 1e12, mfma_frac=f1 / k1 / 1e12 / PEAK_FP8_TFLOPS,
@@ -271,65 +299,132 @@ def bench_dense(pkg, dev, steps, warmup):
     return res
 
 
-def cpu_baseline(pkg, moe, cfg, x, sample_tokens):
-    """The CPU oracle (routing, per-expert dequantise + fp32 matmul, weighted reduce) timed on the
-    first `sample_tokens` tokens of the batch; the same pass doubles as a parity check of the
-    device at full layer size."""
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return platform.processor() or "unknown"
+
+
+def _median(v):
+    v = sorted(v)
+    return v[len(v) // 2]
+
+
+def device_step_with_routing(pkg, moe, cfg, x):
+    """The timed step once more on the same batch, through the same entry point, asked for what its router produced:
+    -> (out [T,H], scores the device selected on, weights [T,K], ids [T,K])."""
+    T = x.shape[0]
+    if moe._one_call(T):
+        out, logits, w, ids = pkg.layer_fp8(
+            x, moe.router_weight, moe.w13, moe.w13_scale, moe.w2, moe.w2_scale, cfg["K"], cfg["route"], moe.bias,
+            cfg["n_groups"], cfg["topk_groups"], True, cfg["scale"], shared=moe.shared, return_routing=True,
+            workspace=moe._workspace(T, True))
+    else:
+        logits = torch.matmul(x, moe.router_weight.t())
+        w, ids = moe.route(x)
+        out = moe.experts(x, w, ids)
+    if cfg["route"] == "sigmoid":
+        w2, ids2, scores = pkg.moe_route(logits, cfg["K"], "sigmoid", moe.bias, cfg["n_groups"], cfg["topk_groups"], True,
+                                         cfg["scale"], return_scores=True)
+    else:
+        scores = logits.float() if moe.bias is None else logits.float() + moe.bias
+        w2, ids2 = pkg.moe_route(logits if moe.bias is None else logits + moe.bias, cfg["K"], "softmax")
+    same = bool(torch.equal(ids, ids2) and torch.equal(w, w2))
+    return out, scores, w, ids, same
+
+
+def cpu_baseline(pkg, moe, cfg, x, sample_tokens, reps=3):
+    """The CPU oracle (router product, routing, per-expert dequantise + fp32 matmul on the same quantised operands,
+    weighted reduce) timed on `sample_tokens` tokens spread over the batch, median of `reps` runs; the device side of
+    the comparison is the rows of those tokens in the output of the FULL batch - the step that is timed - and the
+    comparison is made in the strict steps of oracle/parity_checks.py."""
     orc = entry.load_oracle()
-    cores = os.cpu_count() or 1
-    threads = min(cores, 16)
-    torch.set_num_threads(threads)
-    n = sample_tokens
-    # device side of the comparison: scores the device routed on, its picks and its output
-    one_call = moe._one_call(n)
-    if one_call:
-        # the entry point the timed step goes through, asked for what its router produced
-        out_dev, logits_dev, w_one, ids_one = pkg.layer_fp8(
-            x[:n].contiguous(), moe.router_weight, moe.w13, moe.w13_scale, moe.w2, moe.w2_scale, cfg["K"], cfg["route"],
-            moe.bias, cfg["n_groups"], cfg["topk_groups"], True, cfg["scale"], shared=moe.shared, return_routing=True)
-    else:
-        logits_dev = torch.matmul(x[:n], moe.router_weight.t()).float()
-    if cfg["route"] == "sigmoid":
-        w_dev, ids_dev, scores_dev = pkg.moe_route(logits_dev, cfg["K"], "sigmoid", moe.bias, cfg["n_groups"],
-                                                   cfg["topk_groups"], True, cfg["scale"], return_scores=True)
-    else:
-        lg = logits_dev if moe.bias is None else logits_dev + moe.bias
-        w_dev, ids_dev = pkg.moe_route(lg, cfg["K"], "softmax")
-        scores_dev = lg
-    if one_call:
-        same_routing = bool(torch.equal(ids_one, ids_dev) and torch.equal(w_one, w_dev))
-    else:
-        out_dev = moe.experts(x[:n].contiguous(), w_dev, ids_dev)
+    checks = entry.load_parity_checks()
+    threads = torch.get_num_threads()                # the host's share of cores (OMP_NUM_THREADS) unless fewer exist
+    T, K = x.shape[0], cfg["K"]
+    n = min(sample_tokens, T)
+    out, scores, w, ids, same_routing = device_step_with_routing(pkg, moe, cfg, x)
     torch.cuda.synchronize()
-    xs = x[:n].cpu()
-    wr = moe.router_weight.float().cpu()
+    pick = torch.unique(torch.linspace(0, T - 1, n).round().long()).to(x.device)
+    n = pick.numel()
+    layer = (moe.w13, moe.w13_scale, moe.w2, moe.w2_scale)
+    x_s, ids_s, w_s, out_s = x[pick].contiguous(), ids[pick].contiguous(), w[pick].contiguous(), out[pick].contiguous()
+    parity = {"tokens_checked": n, "rows_taken_from": f"the output of the timed step on all T={T} tokens",
+              "routing_of_entry_point_equals_routing_kernel": same_routing}
+    # routing of the WHOLE batch, exactly, given the scores the device selected on
     bias = None if moe.bias is None else moe.bias.cpu()
-    layer = tuple(t.cpu() for t in (moe.w13, moe.w13_scale, moe.w2, moe.w2_scale))
-    shared = None if moe.shared is None else tuple(t.cpu() for t in moe.shared)
-    scores_host = scores_dev.cpu()
-    t0 = time.perf_counter()
-    logits = xs.float() @ wr.T
+    scores_host = scores.float().cpu()
     if cfg["route"] == "sigmoid":
-        orc.route_sigmoid_grouped(logits, bias, cfg["K"], cfg["n_groups"], cfg["topk_groups"], cfg["scale"])
-        w_ref, ids_ref = orc.select_sigmoid_grouped(scores_host, bias, cfg["K"], cfg["n_groups"], cfg["topk_groups"],
-                                                    cfg["scale"])
+        w_ref, ids_ref = orc.select_sigmoid_grouped(scores_host, bias, K, cfg["n_groups"], cfg["topk_groups"], cfg["scale"])
     else:
-        orc.route_softmax_topk(logits if bias is None else logits + bias, cfg["K"])
-        w_ref, ids_ref = orc.route_softmax_topk(scores_host, cfg["K"])
-    ref = orc.moe_w8a8_fp32(xs, ids_ref, w_ref, *layer, shared=shared)
-    sec = time.perf_counter() - t0
-    got = out_dev.float().cpu()
-    parity = {"routing_ids_equal_given_device_scores": bool(torch.equal(ids_dev.cpu(), ids_ref)),
-              "routing_weights_max_abs_diff": (w_dev.cpu() - w_ref).abs().max().item(),
-              "outputs_outside_rtol2e-2_atol1e-2": ((got - ref).abs() > 1e-2 + 2e-2 * ref.abs()).float().mean().item(),
-              "cos_diff": orc.cal_diff(ref, got)[0], "tokens_checked": n}
-    if one_call:
-        parity["one_call_routing_equals_staged_routing"] = same_routing
+        w_ref, ids_ref = orc.route_softmax_topk(scores_host, K)
+    parity["routing_ids_equal_given_device_scores"] = bool(torch.equal(ids.cpu(), ids_ref))
+    parity["routing_weights_max_abs_diff"] = (w.cpu() - w_ref).abs().max().item()
+    try:
+        rep = checks.check_sample(pkg, orc, x_s, ids_s, layer, w_s=w_s, shared_dev=moe.shared, out_big=out_s,
+                                  what=f"sample of the T={T} step")
+        parity["strict_steps"] = "passed"
+        parity.update(rep)
+    except AssertionError as exc:
+        parity["strict_steps"] = f"FAILED: {exc}"
+    # the timed CPU work: the same tokens through the oracle, only the experts they use brought to the host
+    local, used = checks._localise(ids_s.cpu())
+    idx = torch.tensor(used, device=x.device)
+    small = checks._host_layer(pkg, tuple(t[idx] for t in layer))
+    shared = None if moe.shared is None else checks._host_layer(pkg, moe.shared)
+    xs = x_s.cpu()
+    wr = moe.router_weight.float().cpu()
+    w_host = w_s.cpu()
+    torch.set_num_threads(threads)
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        logits = xs.float() @ wr.T
+        if cfg["route"] == "sigmoid":
+            orc.route_sigmoid_grouped(logits, bias, K, cfg["n_groups"], cfg["topk_groups"], cfg["scale"])
+        else:
+            orc.route_softmax_topk(logits if bias is None else logits + bias, K)
+        ref = orc.moe_w8a8_fp32(xs, local, w_host, *small, shared=shared)
+        times.append(time.perf_counter() - t0)
+    sec = _median(times)
+    got = out_s.float().cpu()
+    parity["outputs_outside_rtol2e-2_atol1e-2"] = checks.outside_fraction(got, ref)
+    parity["worst_violation"] = checks.worst_violation(got, ref)
+    parity["cos_diff_end_to_end"] = orc.cal_diff(ref, got)[0]
     base = dict(value=gemm_flops(cfg, n) / sec / 1e12, unit="TFLOP/s", cores=threads, kind="port",
-                sample=f"first {n} tokens of the same batch through the CPU oracle (routing twice, per-expert "
-                       f"dequantise + fp32 matmul, weighted reduce): {sec:.1f} s, {n / sec:.2f} tokens/s",
-                tokens_per_s=n / sec, host_cpus=cores)
+                sample=f"{n} tokens spread over the same batch through the CPU oracle (router product, routing, per-expert "
+                       f"dequantise + fp32 matmul on the quantised operands, weighted reduce, shared expert), median of "
+                       f"{reps} runs: {sec:.2f} s, {n / sec:.2f} tokens/s",
+                tokens_per_s=n / sec, runs_s=[round(t, 3) for t in times], host_cpus=os.cpu_count() or 1,
+                cpu_model=cpu_model())
     return base, parity
+
+
+def literal_reference_loop(pkg, cfg, dev, T, seed):
+    """The reference's own CPU ground truth, literally: one call per (token, slot), each de-quantising its expert's three
+    matrices block by block in Python and running a bf16 chain (python/regression/test_llm/test_moe.py:10-50, 93-98),
+    timed once on a batch of T tokens of the layer `cfg`.  Only feasible for a handful of tokens."""
+    orc = entry.load_oracle()
+    H, I, E, K = cfg["H"], cfg["I"], cfg["E"], cfg["K"]
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    ids = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)]).to(torch.int32)
+    local, used = entry.load_parity_checks()._localise(ids)
+    # only the touched experts are generated: [n_used, ...] in the reference's orientation (gate, up [I,H]; down [H,I])
+    w13q, w13s = (t.cpu() for t in pkg.synthetic_weights(len(used), 2 * I, H, dev, seed + 1, tile_block=False))
+    w2q, w2s = (t.cpu() for t in pkg.synthetic_weights(len(used), H, I, dev, seed + 2, tile_block=False))
+    nb = I // 128
+    t0 = time.perf_counter()
+    orc.experts_ref_bf16_literal(x, local, w13q[:, :I], w13q[:, I:], w2q, w13s[:, :nb].bfloat16(), w13s[:, nb:].bfloat16(),
+                                 w2s.bfloat16())
+    sec = time.perf_counter() - t0
+    return dict(T=T, seconds=sec, tokens_per_s=T / sec, calls=T * K, kind="port, literal per-(token, slot) loop",
+                cores=torch.get_num_threads())
 
 
 def main():
@@ -382,6 +477,17 @@ def main():
         "tokens_per_s": T / sec, "mfma_frac_of_peak": flops / sec / 1e12 / PEAK_FP8_TFLOPS,
         "roofline": roof,
     }
+    # the whole step against the HBM roof: the bytes no implementation of the layer can avoid (every touched expert's
+    # weights and scales once, the shared expert's, x in, out written) over the step time
+    step_bytes = roof["experts_touched"] * expert_bytes(cfg["H"], cfg["I"]) \
+        + (expert_bytes(cfg["H"], cfg["I_sh"]) if cfg["I_sh"] else 0) + 4 * T * cfg["H"]
+    result["step"] = dict(algorithmic_bytes=step_bytes, hbm_gbs=step_bytes / sec / 1e9,
+                          step_hbm_frac=step_bytes / sec / 1e9 / PEAK_HBM_GBS,
+                          first_gemm_alone_ms=roof["launch_ms"], second_gemm_alone_ms=roof["second_gemm"]["launch_ms"],
+                          rest_ms=sec * 1e3 - roof["launch_ms"] - roof["second_gemm"]["launch_ms"],
+                          note="the GEMM figures are the routed experts' launches on their own; inside the step the same "
+                               "launches also carry the shared expert's tiles; rest = router product, routing + activation "
+                               "quantisation, permutation, weighted sum and the shared expert's share")
     if decode is not None:
         result["decode"] = decode
         result["dense"] = bench_dense(pkg, dev, args.steps, args.warmup)
@@ -434,6 +540,11 @@ def main():
         result["other_shapes"] = others
     if not args.no_cpu:
         base, parity = cpu_baseline(pkg, moe, cfg, x, min(args.cpu_sample, T))
+        # the reference's own ground-truth loop, literally (one de-quantisation of three matrices per token and slot),
+        # on the toy layer and on one decode token of the DeepSeek-V3-shaped layer
+        base["literal_reference_loop"] = [
+            dict(workload="c1_toy", **literal_reference_loop(pkg, WORKLOADS["c1_toy"], dev, WORKLOADS["c1_toy"]["T"], 21)),
+            dict(workload="c4_decode T=1", **literal_reference_loop(pkg, WORKLOADS["c3_prefill"], dev, 1, 22))]
         result["cpu_baseline"] = base
         result["parity_on_sample"] = parity
     print(json.dumps(result))
