@@ -201,6 +201,22 @@ int moe_fused_experts_bf16(void *stream, const void *x_bf16, int T, int H, const
                            void *workspace, size_t workspace_bytes);
 
 /*
+ * The reference's own arithmetic on the packed FP8 weights: bf16 activations against weights that are
+ * de-quantised on the way into the matrix instruction, w = bf16(float(code) * block scale) - what
+ * weight_dequant_bc does in front of the reference kernel's bf16 products (fusedMoE.pl:11-34, 217-269) and what
+ * its tests compute on the CPU (python/regression/test_llm/test_moe.py:10-50, 63-98).  No activation
+ * quantisation, bf16 intermediate, fp32 accumulation; the weights are read once, at one byte per element.
+ * Same tensors as moe_fused_experts_fp8 (tile-blocked w13 / w2, fp32 block scales), same workspace as
+ * moe_fused_experts_bf16; the results are those of moe_fused_experts_bf16 on weights de-quantised beforehand, up to
+ * the order of the matrix instructions' internal sums (a few results land on the neighbouring bf16).
+ * H and I multiples of 128 and at most 16384, no shared expert.
+ */
+int moe_fused_experts_w8a16(void *stream, const void *x_bf16, int T, int H, const uint8_t *w13,
+                            const float *w13_scale, const uint8_t *w2, const float *w2_scale, int I, int E,
+                            const int32_t *ids, const float *routing_weights, int K, void *out_bf16,
+                            int out_mode, void *workspace, size_t workspace_bytes);
+
+/*
  * Dense block-scaled FP8 layers: the same kernels with a single "expert" that owns every row.
  *
  * moe_mm_fp8 replaces at::mm_w8a16_dq_forward -> tpudnnMmW8A16DqAsync

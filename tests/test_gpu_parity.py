@@ -660,3 +660,54 @@ def test_experts_with_bf16_weights(pkg, oracle, dev, T, H, I, E, K):
     want = torch.einsum("tk,tkh->th", w.to(torch.bfloat16).float(), got)
     rms2 = want.pow(2).mean().sqrt()
     assert ((out2.float().cpu() - want).abs() <= 2e-2 * want.abs() + 2e-2 * rms2).all()
+
+
+# T x (H, I, E, K) chosen so that every tile height of the grouped kernels runs in this mode: 16, 32 and 64 rows with both
+# operands through LDS (and the narrow strips of the second GEMM), 128 and 192 rows with the weights in a register ring
+@pytest.mark.parametrize("T,H,I,E,K", [
+    (1, 7168, 256, 256, 8), (8, 7168, 256, 256, 8),            # the reference's own shapes (test_moe.py:219-227)
+    (16, 512, 256, 8, 2), (30, 512, 384, 8, 2), (64, 1024, 256, 16, 4), (130, 256, 128, 8, 2),
+    (128, 768, 128, 64, 2), (260, 512, 256, 8, 2), (600, 512, 256, 4, 2),
+])
+def test_experts_w8a16_in_registers(pkg, oracle, dev, T, H, I, E, K):
+    """The reference's arithmetic on the packed FP8 weights (moe_fused_experts_w8a16): equal, up to the order of the
+    matrix instructions' internal sums, to the bf16 kernels on weights de-quantised beforehand by torch,
+    bf16(float(code) * scale), and within the reference's own criterion
+    (cos_sim > 0.99 and cos_diff < 1e-4, python/regression/test_llm/test_moe.py:308) of the reference's CPU ground
+    truth (test_moe.py:10-98) - with nothing de-quantised in memory."""
+    say("w8a16 in registers", T, H, I, E, K, "tile", pkg.tile_rows(T, K, E))
+    g = torch.Generator().manual_seed(T + H)
+    w0, w1 = ((torch.randn(E, I, H, generator=g) * 0.1).to(torch.float8_e4m3fn) for _ in range(2))
+    w2 = (torch.randn(E, H, I, generator=g) * 0.1).to(torch.float8_e4m3fn)
+    s0, s1 = ((torch.randn(E, I // 128, H // 128, generator=g) * 0.1).to(torch.bfloat16) for _ in range(2))
+    s2 = (torch.randn(E, H // 128, I // 128, generator=g) * 0.1).to(torch.bfloat16)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    ids, w = distinct_ids(T, E, K, seed=T + 5)
+    w13 = torch.cat([w0, w1], 1).to(dev)
+    w13s = torch.cat([s0, s1], 1).float().to(dev)
+    w2d, w2s = w2.to(dev), s2.float().to(dev)
+    xd, idd, wd = x.to(dev), ids.to(dev), w.to(dev)
+    got = pkg.fused_experts_w8a16(xd, pkg.pack_weights(w13), w13s, pkg.pack_weights(w2d), w2s, idd)
+    # the same kernels on weights de-quantised in memory
+    deq = lambda q, s: (q.float() * s.repeat_interleave(128, 1).repeat_interleave(128, 2)).to(torch.bfloat16)
+    want = pkg.fused_experts_bf16(xd, pkg.pack_weights(deq(w13, w13s)), pkg.pack_weights(deq(w2d, w2s)), idd)
+    torch.cuda.synchronize()
+    # Same weights, same products; the 64 elements of a step sit in other positions of the matrix instructions' reduction
+    # (a lane holds 16 consecutive codes here, two runs of 8 bf16 there), and the instruction's internal sum is not
+    # associative: fp32 sums differ in the last bits, a few results land on the neighbouring bf16.
+    gf, wf = got.float(), want.float()
+    same = (got.view(torch.int16) == want.view(torch.int16)).float().mean().item()
+    say("    identical to the kernels on weights de-quantised in memory:", same)
+    assert same >= 0.97, same
+    assert ((gf - wf).abs() <= 1.6e-2 * wf.abs() + 2e-3 * wf.pow(2).mean().sqrt()).all()
+    ref = oracle.experts_ref_bf16(x, ids, w0, w1, w2, s0, s1, s2).float()
+    got_h = got.float().cpu()
+    assert torch.isfinite(got_h).all()
+    assert oracle.cos_sim(ref.numpy(), got_h.numpy()) > 0.99
+    cos_diff = oracle.cal_diff(ref, got_h)[0]
+    assert cos_diff < 1e-4, cos_diff
+    # weighted form
+    out2 = pkg.fused_experts_w8a16(xd, pkg.pack_weights(w13), w13s, pkg.pack_weights(w2d), w2s, idd, wd)
+    want2 = pkg.weighted_reduce(got, wd)
+    torch.cuda.synchronize()
+    assert torch.equal(out2.view(torch.int16), want2.view(torch.int16))

@@ -37,6 +37,8 @@ SIGNATURES = {
     "moe_fused_experts_bf16_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
     "moe_fused_experts_bf16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                        c_void_p, c_int, c_void_p, c_int, c_void_p, c_size_t]),
+    "moe_fused_experts_w8a16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                        c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_size_t]),
     "moe_layer_fp8_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
     "moe_layer_fp8": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                      c_int, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,

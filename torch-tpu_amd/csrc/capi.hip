@@ -11,11 +11,11 @@ int permute_launch(hipStream_t st, const int32_t *ids, int T, int K, int E, int 
 int gemm1_launch(hipStream_t st, const uint8_t *xq, const float *xs, int T, int H, const uint8_t *w13,
                  const float *w13s, int I, int E, int K, const int32_t *sorted_slot, const int32_t *expert_offsets,
                  const PermuteWs *pw, int fixed_expert, uint8_t *hq, float *hs, const uint8_t *sh_w13,
-                 const float *sh_w13s, uint8_t *sh_hq, float *sh_hs, bool bf16 = false);
+                 const float *sh_w13s, uint8_t *sh_hq, float *sh_hs, int numerics = kNumericsFp8);
 int gemm2_launch(hipStream_t st, const uint8_t *hq, const float *hs, int rows_a, int T, int H, const uint8_t *w2,
                  const float *w2s, int I, int E, int K, const int32_t *sorted_slot, const int32_t *expert_offsets,
                  const PermuteWs *pw, int fixed_expert, uint16_t *y, const uint8_t *sh_hq, const float *sh_hs,
-                 int sh_rows, const uint8_t *sh_w2, const float *sh_w2s, uint16_t *sh_y, bool bf16 = false);
+                 int sh_rows, const uint8_t *sh_w2, const float *sh_w2s, uint16_t *sh_y, int numerics = kNumericsFp8);
 
 int decode_prep_launch(hipStream_t st, const uint16_t *x, int T, int H, const uint16_t *wr, const float *bias, int E, int K,
                        int mode, int n_groups, int topk_groups, int renorm, float scale, uint16_t *logits, float *weights,
@@ -450,7 +450,7 @@ extern "C" int moe_mm_bf16(void *stream, const void *x_bf16, int M, int K, const
   if (M == 0) return MOE_OK;
   return gemm2_launch((hipStream_t)stream, (const uint8_t *)x_bf16, nullptr, M, M, N, (const uint8_t *)w_bf16, nullptr, K,
                       1, 1, nullptr, nullptr, nullptr, 0, (uint16_t *)out_bf16, nullptr, nullptr, 0, nullptr, nullptr,
-                      nullptr, true);
+                      nullptr, kNumericsBf16);
 }
 
 extern "C" size_t moe_mlp_fp8_workspace_bytes(int M, int H, int I) {
@@ -525,12 +525,14 @@ extern "C" size_t moe_fused_experts_bf16_workspace_bytes(int T, int H, int I, in
   return moe::bf16_layout(nullptr, T, H, I, E, K).bytes;
 }
 
-extern "C" int moe_fused_experts_bf16(void *stream, const void *x_bf16, int T, int H, const void *w13_bf16,
-                                      const void *w2_bf16, int I, int E, const int32_t *ids,
-                                      const float *routing_weights, int K, void *out_bf16, int out_mode,
-                                      void *workspace, size_t workspace_bytes) {
-  using namespace moe;
-  if (!w13_bf16 || !w2_bf16 || !workspace) return MOE_E_NULL;
+namespace moe {
+// bf16 activations against bf16 weights (scales NULL) or against FP8 weights de-quantised in registers
+static int experts_a16_run(void *stream, const void *x_bf16, int T, int H, const void *w13, const float *w13_scale,
+                           const void *w2, const float *w2_scale, int I, int E, const int32_t *ids,
+                           const float *routing_weights, int K, void *out_bf16, int out_mode, void *workspace,
+                           size_t workspace_bytes, int numerics) {
+  if (!w13 || !w2 || !workspace) return MOE_E_NULL;
+  if (numerics == kNumericsW8A16 && (!w13_scale || !w2_scale)) return MOE_E_NULL;
   if (T != 0 && (!x_bf16 || !ids || !out_bf16)) return MOE_E_NULL;
   if (out_mode != 0 && out_mode != 1) return MOE_E_MODE;
   if (T != 0 && out_mode == 1 && !routing_weights) return MOE_E_NULL;
@@ -539,7 +541,7 @@ extern "C" int moe_fused_experts_bf16(void *stream, const void *x_bf16, int T, i
   if (H % kBlock || I % kBlock) return MOE_E_ALIGN;
   if ((double)T * H * 2 >= 2147483648.0 || (double)T * K * I * 2 >= 2147483648.0) return MOE_E_SHAPE;
   if (((uintptr_t)workspace % 256) || ((uintptr_t)x_bf16 % 16) || ((uintptr_t)out_bf16 % 16) ||
-      ((uintptr_t)w13_bf16 % 16) || ((uintptr_t)w2_bf16 % 16))
+      ((uintptr_t)w13 % 16) || ((uintptr_t)w2 % 16))
     return MOE_E_ALIGN;
   Bf16Ws w = bf16_layout(workspace, T, H, I, E, K);
   if (workspace_bytes < w.bytes) return MOE_E_WORKSPACE;
@@ -548,13 +550,30 @@ extern "C" int moe_fused_experts_bf16(void *stream, const void *x_bf16, int T, i
   PermuteWs pw = permute_ws_layout(w.permute, T, K, E);
   int rc = permute_launch(st, ids, T, K, E, choose_tile_m(T, K, E), w.sorted_slot, w.expert_offsets, w.slot_to_row, pw);
   if (rc) return rc;
-  rc = gemm1_launch(st, (const uint8_t *)x_bf16, nullptr, T, H, (const uint8_t *)w13_bf16, nullptr, I, E, K, w.sorted_slot,
-                    w.expert_offsets, &pw, -1, (uint8_t *)w.h, nullptr, nullptr, nullptr, nullptr, nullptr, true);
+  rc = gemm1_launch(st, (const uint8_t *)x_bf16, nullptr, T, H, (const uint8_t *)w13, w13_scale, I, E, K, w.sorted_slot,
+                    w.expert_offsets, &pw, -1, (uint8_t *)w.h, nullptr, nullptr, nullptr, nullptr, nullptr, numerics);
   if (rc) return rc;
   uint16_t *y = out_mode == 0 ? (uint16_t *)out_bf16 : w.y;
-  rc = gemm2_launch(st, (const uint8_t *)w.h, nullptr, T * K, T, H, (const uint8_t *)w2_bf16, nullptr, I, E, K,
-                    w.sorted_slot, w.expert_offsets, &pw, -1, y, nullptr, nullptr, 0, nullptr, nullptr, nullptr, true);
+  rc = gemm2_launch(st, (const uint8_t *)w.h, nullptr, T * K, T, H, (const uint8_t *)w2, w2_scale, I, E, K,
+                    w.sorted_slot, w.expert_offsets, &pw, -1, y, nullptr, nullptr, 0, nullptr, nullptr, nullptr, numerics);
   if (rc) return rc;
   if (out_mode == 0) return zero_dropped_rows_launch(st, w.slot_to_row, T * K, H, y);
   return weighted_reduce_launch(st, y, routing_weights, nullptr, w.slot_to_row, T, K, H, (uint16_t *)out_bf16);
+}
+}  // namespace moe
+
+extern "C" int moe_fused_experts_bf16(void *stream, const void *x_bf16, int T, int H, const void *w13_bf16,
+                                      const void *w2_bf16, int I, int E, const int32_t *ids,
+                                      const float *routing_weights, int K, void *out_bf16, int out_mode,
+                                      void *workspace, size_t workspace_bytes) {
+  return moe::experts_a16_run(stream, x_bf16, T, H, w13_bf16, nullptr, w2_bf16, nullptr, I, E, ids, routing_weights, K,
+                              out_bf16, out_mode, workspace, workspace_bytes, moe::kNumericsBf16);
+}
+
+extern "C" int moe_fused_experts_w8a16(void *stream, const void *x_bf16, int T, int H, const uint8_t *w13,
+                                       const float *w13_scale, const uint8_t *w2, const float *w2_scale, int I, int E,
+                                       const int32_t *ids, const float *routing_weights, int K, void *out_bf16,
+                                       int out_mode, void *workspace, size_t workspace_bytes) {
+  return moe::experts_a16_run(stream, x_bf16, T, H, w13, w13_scale, w2, w2_scale, I, E, ids, routing_weights, K, out_bf16,
+                              out_mode, workspace, workspace_bytes, moe::kNumericsW8A16);
 }

@@ -27,6 +27,12 @@
 //
 // BF16 = true: the same tiles and pipelines on un-quantised operands (no scales, two
 // v_mfma_f32_16x16x32_bf16 per 128-byte step accumulating in place, bf16 intermediate).
+// DQ = true (with BF16): bf16 activations against FP8 weights that are de-quantised on the way into the
+// matrix instruction - bf16(float(code) * block scale), the arithmetic of the reference's own kernel
+// (fusedMoE.pl:217-269) - at the FP8 weights' byte count.  A step is still 128 bytes of a token row = 64
+// elements; its weights are one 1 KB half of a tile-blocked (16 rows x 128 codes) block: the halves of a
+// block are reduction elements 0..63 and 64..127, a lane holding codes 16g..16g+15 of its row in either,
+// which become its operands of the step's two matrix instructions.
 //
 // GATED = true  (first GEMM): the strip is 128 gate columns plus the 128 matching up columns of
 //   W13; wavefront w owns gate columns 16w..16w+15 and the same up columns.  Epilogue:
@@ -118,6 +124,20 @@ __device__ __forceinline__ v8i concat8(v4i lo, v4i hi) {
 
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
+// 16 e4m3fn codes (reduction elements in byte order) -> 16 bf16 = bf16(float(code) * s), the reference's
+// weight_dequant (fusedMoE.pl:11-34; python/regression/test_llm/test_moe.py:10-50), element b in half b % 2 of dword b / 2
+__device__ __forceinline__ v8i dequant16(v4i raw, float s) {
+  v8i r;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const v2f_t a = __builtin_amdgcn_cvt_pk_f32_fp8(raw[i], false);
+    const v2f_t b = __builtin_amdgcn_cvt_pk_f32_fp8(raw[i], true);
+    r[2 * i] = (int)pack2_bf16(a[0] * s, a[1] * s);
+    r[2 * i + 1] = (int)pack2_bf16(b[0] * s, b[1] * s);
+  }
+  return r;
+}
+
 // bf16 operands: the two 16-byte chunks a lane holds of a 128-byte step are the lane's share of two
 // 32-element matrix instructions; all first halves are issued before the second halves so that an
 // accumulator is not needed again right away
@@ -141,10 +161,12 @@ __device__ __forceinline__ void mma_bf16(v4f (&acc)[WT], const v8i (&w)[WT], con
 // TPS    weight tiles (of 16 rows) per strip: 16, or 4 for the second GEMM of a batch that would leave most
 //        of the chip without a strip (narrow strips of 64 output columns; every sum keeps its order)
 // DEPTH  128-steps of weights kept in flight per wavefront (register ring)
+// DQ     BF16 arithmetic on FP8 weights with block scales, de-quantised in registers (a.Kd counts the token row's bytes)
 // BF16   un-quantised mode: both operands are bf16 (a 128-byte step is 64 elements = two
 //        v_mfma_f32_16x16x32_bf16 accumulating in place), no scales, bf16 intermediate
-template <int MT, int NW, int DEPTH, bool GATED, bool WREG, bool BF16 = false, int TPS = 16>
+template <int MT, int NW, int DEPTH, bool GATED, bool WREG, bool BF16 = false, int TPS = 16, bool DQ = false>
 __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a) {
+  static_assert(!DQ || BF16, "de-quantised weights feed the bf16 matrix instructions");
   static_assert(TPS % NW == 0 && (TPS == 16 || (!GATED && !WREG && TPS <= 8)), "narrow strips: second GEMM, operands through LDS");
   constexpr int BM = 16 * MT;
   constexpr int NT = 64 * NW;                         // threads
@@ -250,7 +272,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     if (GATED) wrow = (j < WT / 2 ? 0 : a.N) + strip * 128 + wave * (8 * WT) + (j % (WT / 2)) * 16;
     else wrow = strip * (16 * TPS) + wave * (16 * WT) + j * 16;
     wrow = min(wrow, a.n_rows_w - 16);                 // tiles past the matrix re-read its last rows
-    wtile[j] = wq + ((size_t)e * a.n_rows_w + wrow) * a.Kd;
+    wtile[j] = wq + ((size_t)e * a.n_rows_w + wrow) * (DQ ? a.Kd >> 1 : a.Kd);
   }
   // Weights are stored tile-blocked: the 2 KB a (16-row tile, 128-byte step) pair needs are contiguous and already
   // in operand order - two 1 KB halves of [lane][16 bytes] - so every load instruction of a wavefront reads 1 KB of
@@ -262,14 +284,16 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   // the rows' sources, before either is waited for.
   constexpr int NSB = (2 * kMaxKB + NT - 1) / NT;
   float sbv[NSB];
-  if constexpr (!BF16) {
+  // DQ: a step is half a 128-block of the reduction (64 elements), two steps share a block scale
+  const int NKBW = DQ ? NKB >> 1 : NKB;
+  if constexpr (!BF16 || DQ) {
     // second GEMM: the 128-row blocks the strip's first and ninth tile lie in (a narrow strip lies in one)
     const int blk0 = GATED ? strip : min(strip * TPS / 8, n_wblk - 1);
     const int blk1 = GATED ? (a.N >> 7) + strip : min(strip * TPS / 8 + 1, n_wblk - 1);
 #pragma unroll
     for (int u = 0; u < NSB; u++) {
       const int i = tid + u * NT, r = i >= NKB, kb = i - r * NKB;
-      sbv[u] = i < 2 * NKB ? ws[((size_t)e * n_wblk + (r ? blk1 : blk0)) * NKB + kb] : 0.f;
+      sbv[u] = i < 2 * NKB ? ws[((size_t)e * n_wblk + (r ? blk1 : blk0)) * NKBW + (DQ ? kb >> 1 : kb)] : 0.f;
     }
   }
   for (int i = tid; i < BM; i += NT) {
@@ -279,7 +303,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     sm.arow[i] = min(max(src, 0), rows_a - 1);
     if (!GATED) sm.oslot[i] = direct ? p : a.sorted_slot[p];      // output row (slot) of each tile row
   }
-  if constexpr (!BF16) {
+  if constexpr (!BF16 || DQ) {
 #pragma unroll
     for (int u = 0; u < NSB; u++) {
       const int i = tid + u * NT, r = i >= NKB, kb = i - r * NKB;
@@ -343,19 +367,27 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   //   weights: the wavefront's WT tiles, each as two 1 KB halves laid out [lane][16 bytes] - the
   //            owner reads them back with two linear 128-bit LDS reads per tile;
   //   tokens:  1 KB pieces = 8 rows x 128 bytes, swizzled on the source side.
-  constexpr int L_STEP = NTOK + 2 * WT;                // loads per wavefront and step (scale chunks come on top)
+  constexpr int LPT = DQ ? 1 : 2;                      // load instructions per weight tile and step (1 KB each)
+  constexpr int WSTEP = 1024 * LPT;                    // bytes of a tile's step in memory
+  constexpr int L_STEP = NTOK + LPT * WT;              // loads per wavefront and step (scale chunks come on top)
   v4i wlo[WREG ? DEPTH : 1][WT], whi[WREG ? DEPTH : 1][WT];   // WREG: weight fragments ride in a register ring
   auto request_weights_reg = [&](int kb, v4i(&lo)[WT], v4i(&hi)[WT]) {
 #pragma unroll
     for (int j = 0; j < WT; j++) {
-      const uint8_t *base = wtile[j] + (size_t)kb * 2048;
-      asm volatile("global_load_dwordx4 %0, %2, %3\n\tglobal_load_dwordx4 %1, %2, %3 offset:1024"
-                   : "=&v"(lo[j]), "=&v"(hi[j]) : "v"(woff), "s"(base) : "memory");
+      const uint8_t *base = wtile[j] + (size_t)kb * WSTEP;
+      if constexpr (DQ)
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(lo[j]) : "v"(woff), "s"(base) : "memory");
+      else
+        asm volatile("global_load_dwordx4 %0, %2, %3\n\tglobal_load_dwordx4 %1, %2, %3 offset:1024"
+                     : "=&v"(lo[j]), "=&v"(hi[j]) : "v"(woff), "s"(base) : "memory");
     }
   };
   auto arrived_weights = [&](v4i(&lo)[WT], v4i(&hi)[WT]) {
 #pragma unroll
-    for (int j = 0; j < WT; j++) asm volatile("" : "+v"(lo[j]), "+v"(hi[j]));
+    for (int j = 0; j < WT; j++) {
+      if constexpr (DQ) asm volatile("" : "+v"(lo[j]));
+      else asm volatile("" : "+v"(lo[j]), "+v"(hi[j]));
+    }
   };
   auto request_scales = [&](int chunk) {
     if constexpr (BF16) return;
@@ -378,15 +410,23 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     if (!WREG)
 #pragma unroll
     for (int j = 0; j < WT; j++) {
-      const uint8_t *base = wtile[j] + (size_t)kb * 2048;
+      const uint8_t *base = wtile[j] + (size_t)kb * WSTEP;
       const uint32_t m0 = wt_base + stage * kWtStage + j * 2048;
       // the instruction offset advances the memory address and the LDS address alike
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t"
-                   "global_load_lds_dwordx4 %1, %2 offset:1024"
-                   ::"s"(m0), "v"(woff), "s"(base) : "memory", "m0");
+      if constexpr (DQ)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(woff), "s"(base) : "memory", "m0");
+      else
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t"
+                     "global_load_lds_dwordx4 %1, %2 offset:1024"
+                     ::"s"(m0), "v"(woff), "s"(base) : "memory", "m0");
     }
   };
 
+  // Which two 16-byte chunks of a token row's 128-byte step a lane reads (positions XOR-swizzled by the row).  FP8 and
+  // bf16 operands: chunks g and g + 4, conflict-free for 128-bit LDS reads, and the weights are stored to match.  DQ:
+  // the lane's 16 weight codes are reduction elements 16g..16g+15 of the step, bytes 32g..32g+31 of the token row.
+  auto tok_chunk0 = [](int g, int i) { return ((DQ ? 2 * g : g) ^ (i & 7)) << 4; };
+  auto tok_chunk1 = [](int g, int i) { return ((DQ ? 2 * g + 1 : g + 4) ^ (i & 7)) << 4; };
   // m-tiles are processed in groups of up to four; a group is skipped when it holds no row.  A
   // group first issues all of its LDS reads (one exposed LDS latency per group, not per tile),
   // then its matrix instructions back to back, each tile's scale multiply-adds trailing the
@@ -395,14 +435,15 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   auto compute = [&](int stage, int kb, const v4i(&lo)[WT], const v4i(&hi)[WT]) {
     v8i wc[WT];
     const uint8_t *wbase = sm.wt[WREG ? 0 : stage] + wave * (WT * 2048) + lane * 16;
+    const float s0 = BF16 && !DQ ? 0.f : sm.sb[sb_row0][kb], s1 = BF16 && !DQ ? 0.f : sm.sb[sb_row1][kb];
 #pragma unroll
     for (int j = 0; j < WT; j++) {
-      if (WREG) wc[j] = concat8(lo[j], hi[j]);
+      if constexpr (DQ) wc[j] = dequant16(WREG ? lo[j] : *(const v4i *)(wbase + j * 2048), (GATED && j >= WT / 2) ? s1 : s0);
+      else if (WREG) wc[j] = concat8(lo[j], hi[j]);
       else wc[j] = concat8(*(const v4i *)(wbase + j * 2048), *(const v4i *)(wbase + j * 2048 + 1024));
     }
-    const float s0 = BF16 ? 0.f : sm.sb[sb_row0][kb], s1 = BF16 ? 0.f : sm.sb[sb_row1][kb];
     const uint8_t *tbase = sm.tok[stage] + li * 128;
-    const int o0 = (lg ^ (li & 7)) << 4, o1 = ((lg + 4) ^ (li & 7)) << 4;
+    const int o0 = tok_chunk0(lg, li), o1 = tok_chunk1(lg, li);
     const float *sap = sm.sac[(kb >> 4) & 1] + ((kb & 12) << 4) + li * 4 + (kb & 3);
 #pragma unroll
     for (int mg = 0; mg < MT / MG; mg++) {
@@ -497,9 +538,9 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     static_assert(DEPTH == 2, "the register ring holds two steps");
     constexpr int R = DEPTH;                             // ring slots = steps per pass of the unrolled loop
     constexpr int XB = 4;                                // token operand buffers; R * LIVE is a multiple of it
-    constexpr int L_WAIT = NTOK + 2 * WT * (R - 1);      // loads younger than the ones a step boundary needs
+    constexpr int L_WAIT = NTOK + LPT * WT * (R - 1);    // loads younger than the ones a step boundary needs
     const int last = NKB - 1;
-    const int o0 = (lg ^ (li & 7)) << 4, o1 = ((lg + 4) ^ (li & 7)) << 4;
+    const int o0 = tok_chunk0(lg, li), o1 = tok_chunk1(lg, li);
     auto run = [&](auto live_c) {
       constexpr int LIVE = decltype(live_c)::value;
       static_assert(LIVE % 2 == 0 && LIVE >= 2 && LIVE <= MT, "live m-tiles come in pairs");
@@ -562,7 +603,10 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
           const int kb = s0 + h;
           v8i wc[WT];
 #pragma unroll
-          for (int j = 0; j < WT; j++) wc[j] = concat8(wlo[h][j], whi[h][j]);
+          for (int j = 0; j < WT; j++) {
+            if constexpr (DQ) wc[j] = dequant16(wlo[h][j], sm.sb[(GATED && j >= WT / 2) ? sb_row1 : sb_row0][kb]);
+            else wc[j] = concat8(wlo[h][j], whi[h][j]);
+          }
           // one m-tile: LDS reads two m-tiles ahead, its matrix instructions, then the multiply-adds
           // of the m-tile before it (tp), whose products are complete by now
           // m-tiles are walked from the last live one down to 0 so that the m-tile whose products are
@@ -749,7 +793,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
 
 // Launch shape per tile height.  Eight wavefronts (two per SIMD, two weight tiles each) keep
 // more loads in flight for the bandwidth-bound shapes.
-template <bool GATED, bool BF16 = false>
+template <bool GATED, bool BF16 = false, bool DQ = false>
 static int launch_gemm(hipStream_t st, GemmArgs &a, int tile_m, int max_mtiles) {
   // the kernel keeps one weight-block scale per 128-step in LDS and forms per-lane operand offsets in 32 bits
   if (a.Kd < 128 || a.Kd % 128 || (a.Kd >> 7) > kMaxKB) return MOE_E_SHAPE;
@@ -766,12 +810,12 @@ static int launch_gemm(hipStream_t st, GemmArgs &a, int tile_m, int max_mtiles) 
   if (total <= 0 || total > 0x7fffffffl) return MOE_E_SHAPE;
   a.total_blocks = (int)total;
   dim3 grid((unsigned)total);
-#define MOE_GEMM(MT, NW, D, WREG) grouped_gemm_kernel<MT, NW, D, GATED, WREG, BF16><<<grid, dim3(64 * NW), 0, st>>>(a)
+#define MOE_GEMM(MT, NW, D, WREG) grouped_gemm_kernel<MT, NW, D, GATED, WREG, BF16, 16, DQ><<<grid, dim3(64 * NW), 0, st>>>(a)
   // small tiles: both operands through LDS (few registers, deeper pipeline); large tiles: weights in
   // a register ring so that LDS holds three stages of the bigger token tile
   if constexpr (!GATED) {
     if (narrow) {
-#define MOE_GEMM_NARROW(MT, D) grouped_gemm_kernel<MT, 4, D, false, false, BF16, 4><<<grid, dim3(256), 0, st>>>(a)
+#define MOE_GEMM_NARROW(MT, D) grouped_gemm_kernel<MT, 4, D, false, false, BF16, 4, DQ><<<grid, dim3(256), 0, st>>>(a)
       switch (tile_m) {
         case 16: MOE_GEMM_NARROW(1, 3); break;
         case 32: MOE_GEMM_NARROW(2, 3); break;
@@ -806,7 +850,8 @@ static int check_dims(int T, int H, int I, int E, int K) {
 int gemm1_launch(hipStream_t st, const uint8_t *xq, const float *xs, int T, int H, const uint8_t *w13,
                  const float *w13s, int I, int E, int K, const int32_t *sorted_slot, const int32_t *expert_offsets,
                  const PermuteWs *pw, int fixed_expert, uint8_t *hq, float *hs, const uint8_t *sh_w13,
-                 const float *sh_w13s, uint8_t *sh_hq, float *sh_hs, bool bf16) {
+                 const float *sh_w13s, uint8_t *sh_hq, float *sh_hs, int numerics) {
+  const bool bf16 = numerics != kNumericsFp8;
   GemmArgs a{};
   if (sh_w13) { a.sh_aq = xq; a.sh_as = xs; a.sh_w = sh_w13; a.sh_ws = sh_w13s; a.sh_hq = sh_hq; a.sh_hs = sh_hs; a.sh_rows = T; }
   a.aq = xq; a.as = xs; a.w = w13; a.ws = w13s;
@@ -818,6 +863,7 @@ int gemm1_launch(hipStream_t st, const uint8_t *xq, const float *xs, int T, int 
   a.Kd = bf16 ? 2 * H : H; a.N = I; a.n_rows_w = 2 * I; a.rows_a = T; a.topk = K; a.E = E; a.fixed_expert = fixed_expert;
   const int tile_m = choose_tile_m(T, K, E);
   const int max_mtiles = fixed_expert >= 0 ? (T + tile_m - 1) / tile_m : pw->max_tiles;
+  if (numerics == kNumericsW8A16) return launch_gemm<true, true, true>(st, a, tile_m, max_mtiles + (a.sh_rows + tile_m - 1) / tile_m);
   if (bf16) return launch_gemm<true, true>(st, a, tile_m, max_mtiles + (a.sh_rows + tile_m - 1) / tile_m);
   return launch_gemm<true>(st, a, tile_m, max_mtiles + (a.sh_rows + tile_m - 1) / tile_m);
 }
@@ -825,7 +871,8 @@ int gemm1_launch(hipStream_t st, const uint8_t *xq, const float *xs, int T, int 
 int gemm2_launch(hipStream_t st, const uint8_t *hq, const float *hs, int rows_a, int T, int H, const uint8_t *w2,
                  const float *w2s, int I, int E, int K, const int32_t *sorted_slot, const int32_t *expert_offsets,
                  const PermuteWs *pw, int fixed_expert, uint16_t *y, const uint8_t *sh_hq, const float *sh_hs,
-                 int sh_rows, const uint8_t *sh_w2, const float *sh_w2s, uint16_t *sh_y, bool bf16) {
+                 int sh_rows, const uint8_t *sh_w2, const float *sh_w2s, uint16_t *sh_y, int numerics) {
+  const bool bf16 = numerics != kNumericsFp8;
   GemmArgs a{};
   if (sh_w2) { a.sh_aq = sh_hq; a.sh_as = sh_hs; a.sh_w = sh_w2; a.sh_ws = sh_w2s; a.sh_y = sh_y; a.sh_rows = sh_rows; }
   a.aq = hq; a.as = hs; a.w = w2; a.ws = w2s;
@@ -837,6 +884,7 @@ int gemm2_launch(hipStream_t st, const uint8_t *hq, const float *hs, int rows_a,
   a.Kd = bf16 ? 2 * I : I; a.N = H; a.n_rows_w = H; a.rows_a = rows_a; a.topk = K; a.E = E; a.fixed_expert = fixed_expert;
   const int tile_m = choose_tile_m(T, K, E);
   const int max_mtiles = fixed_expert >= 0 ? (rows_a + tile_m - 1) / tile_m : pw->max_tiles;
+  if (numerics == kNumericsW8A16) return launch_gemm<false, true, true>(st, a, tile_m, max_mtiles + (a.sh_rows + tile_m - 1) / tile_m);
   if (bf16) return launch_gemm<false, true>(st, a, tile_m, max_mtiles + (a.sh_rows + tile_m - 1) / tile_m);
   return launch_gemm<false>(st, a, tile_m, max_mtiles + (a.sh_rows + tile_m - 1) / tile_m);
 }
@@ -856,7 +904,7 @@ extern "C" int moe_gemm1_swiglu(void *stream, const uint8_t *xq, const float *xs
   if (T == 0) return MOE_OK;
   PermuteWs pw = permute_ws_layout(const_cast<void *>(permute_workspace), T, K, E);
   return gemm1_launch((hipStream_t)stream, xq, xs, T, H, w13, w13_scale, I, E, K, sorted_slot, expert_offsets, &pw, -1,
-                      hq, hs, nullptr, nullptr, nullptr, nullptr, false);
+                      hq, hs, nullptr, nullptr, nullptr, nullptr, kNumericsFp8);
 }
 
 extern "C" int moe_gemm2(void *stream, const uint8_t *hq, const float *hs, int T, int H, const uint8_t *w2,
@@ -871,5 +919,5 @@ extern "C" int moe_gemm2(void *stream, const uint8_t *hq, const float *hs, int T
   if (T == 0) return MOE_OK;
   PermuteWs pw = permute_ws_layout(const_cast<void *>(permute_workspace), T, K, E);
   return gemm2_launch((hipStream_t)stream, hq, hs, T * K, T, H, w2, w2_scale, I, E, K, sorted_slot, expert_offsets, &pw,
-                      -1, (uint16_t *)y_bf16, nullptr, nullptr, 0, nullptr, nullptr, nullptr, false);
+                      -1, (uint16_t *)y_bf16, nullptr, nullptr, 0, nullptr, nullptr, nullptr, kNumericsFp8);
 }

@@ -7,6 +7,10 @@ namespace moe {
 
 constexpr int kChunk = 256;   // slots ranked by one wavefront in the permutation kernels
 
+// What the grouped GEMMs multiply: FP8 activations x FP8 weights with scales (the path proper), bf16 x bf16
+// (un-quantised experts), or bf16 activations x FP8 weights de-quantised to bf16 in registers (the reference's arithmetic)
+enum { kNumericsFp8 = 0, kNumericsBf16 = 1, kNumericsW8A16 = 2 };
+
 static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 // Rows of an activation-scale tensor are padded to whole 64-byte pieces: the grouped GEMMs fetch

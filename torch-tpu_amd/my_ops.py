@@ -50,10 +50,11 @@ _lib.define("mm_w8a16_dq_forward(Tensor input, Tensor weight, Tensor scale, Tens
 
 # How quantised expert weights are multiplied.  "w8a8" (default): activations are quantised to FP8 per
 # token and 128 columns and the products run on the FP8 matrix path - the path this package is about.
-# "w8a16": the reference's own arithmetic (python/regression/test_llm/test_moe.py:10-98) - weights are
-# de-quantised ONCE into bf16 (bf16(fp8) * bf16 scale, cached, twice the bytes) and the un-quantised
-# kernels run on bf16 activations; meant for validating against the reference's criterion
-# (cos_diff < 1e-4, test_moe.py:308), not for serving.
+# "w8a16": the reference's own arithmetic (python/regression/test_llm/test_moe.py:10-98; fusedMoE.pl:217-269) - bf16
+# activations against weights de-quantised to bf16(float(code) * block scale) IN REGISTERS on the way into the
+# matrix instructions, from the same packed FP8 copy the default mode reads (one byte per weight element, nothing
+# de-quantised in memory); meets the reference's criterion (cos_diff < 1e-4, test_moe.py:308).  Only block sizes
+# that 128 does not divide still go through a bf16 copy de-quantised once.
 _numerics = "w8a8"
 
 
@@ -186,8 +187,9 @@ def _fused_experts(output, input, output_sample, input_sample, gate_weights, up_
         raise RuntimeError("either all three weight tensors carry block scales or none does")
     if blocksize < 1:
         raise RuntimeError("blocksize must be positive")
-    # block sizes that 128 does not divide cannot share a 128-long FP8 dot product: the reference's arithmetic then
-    if _numerics == "w8a16" or blocksize % 128:
+    # block sizes that 128 does not divide cannot share a 128-long FP8 dot product: the reference's arithmetic then,
+    # on a bf16 copy de-quantised once
+    if blocksize % 128:
         w13, w2 = _dense_packed(
             (gate_weights, up_weights, down_weights, gate_scales, up_scales, down_scales),
             lambda: (ops.pack_weights(torch.cat([_dequant_bf16(gate_weights, gate_scales, blocksize),
@@ -210,6 +212,10 @@ def _fused_experts(output, input, output_sample, input_sample, gate_weights, up_
     T, H = input.shape
     E, I2, _ = w13.shape
     rw = _routing_f32(routing_weights, input.device) if output.dim() == 2 else None
+    if _numerics == "w8a16":
+        ws = _workspace(input.device, ops.fused_experts_bf16_workspace_bytes(T, H, I2 // 2, E, select_experts.shape[1]))
+        ops.fused_experts_w8a16(input, w13, w13s, w2, w2s, select_experts, rw, out=output, workspace=ws)
+        return output
     ws = _workspace(input.device, ops.fused_experts_workspace_bytes(T, H, I2 // 2, E, select_experts.shape[1]))
     ops.fused_experts_fp8(input, w13, w13s, w2, w2s, select_experts, rw, out=output, workspace=ws)
     return output

@@ -371,6 +371,42 @@ def fused_experts_bf16(x, w13, w2, ids, routing_weights=None, out=None, workspac
     return out
 
 
+def fused_experts_w8a16(x, w13, w13_scale, w2, w2_scale, ids, routing_weights=None, out=None, workspace=None):
+    """The expert computation in the reference's own arithmetic on the packed FP8 weights: bf16 activations, weights
+    de-quantised in registers to bf16(float(code) * block scale), bf16 intermediate - no activation quantisation.
+    Same tensors as fused_experts_fp8 (tile-blocked codes, fp32 block scales), workspace of fused_experts_bf16."""
+    _need(x.dim() == 2 and w13.dim() == 3 and w2.dim() == 3 and ids.dim() == 2, "bad ranks")
+    T, H = x.shape
+    E, I2, _ = w13.shape
+    I = I2 // 2
+    K = ids.shape[1]
+    _need(tuple(w13.shape) == (E, 2 * I, H) and tuple(w2.shape) == (E, H, I), "w13 must be [E,2I,H] and w2 [E,H,I]")
+    _need(H % 128 == 0 and I % 128 == 0, "H and I must be multiples of 128")
+    _need(tuple(w13_scale.shape) == (E, 2 * I // 128, H // 128) and tuple(w2_scale.shape) == (E, H // 128, I // 128),
+          "bad scale shapes")
+    _need(ids.shape[0] == T, "ids must be [T, K]")
+    if out is None:
+        out = torch.empty((T, K, H) if routing_weights is None else (T, H), dtype=torch.bfloat16, device=x.device)
+    mode = 1 if out.dim() == 2 else 0
+    _need(tuple(out.shape) == ((T, H) if mode else (T, K, H)), "out must be [T,H] or [T,K,H]")
+    rw_ptr = None
+    if routing_weights is not None:
+        _need(tuple(routing_weights.shape) == (T, K), "routing_weights must be [T, K]")
+        rw_ptr = _dev(routing_weights, "routing_weights", torch.float32)
+    _need(mode == 0 or rw_ptr is not None, "routing_weights are required for a [T,H] output")
+    need = lib.moe_fused_experts_bf16_workspace_bytes(T, H, I, E, K)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+    _need(workspace.numel() * workspace.element_size() >= need, "workspace too small")
+    rc = lib.moe_fused_experts_w8a16(_stream(), _dev(x, "x", torch.bfloat16), T, H, _dev(w13, "w13", _FP8),
+                                     _dev(w13_scale, "w13_scale", torch.float32), _dev(w2, "w2", _FP8),
+                                     _dev(w2_scale, "w2_scale", torch.float32), I, E, _dev(ids, "ids", torch.int32),
+                                     rw_ptr, K, _dev(out, "out", torch.bfloat16), mode, _dev(workspace, "workspace"),
+                                     workspace.numel() * workspace.element_size())
+    check(rc, "fused_experts_w8a16")
+    return out
+
+
 # --------------------------------------------------------------------------- dense layers
 def mm_fp8(x, w, w_scale, out=None, workspace=None):
     """Dense block-scaled linear layer: x [M,K] bf16, w [N,K] e4m3fn, fp32 scales [ceil(N/128), K/128]
