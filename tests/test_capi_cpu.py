@@ -223,3 +223,23 @@ def test_derived_weight_cache_follows_the_source_tensors(pkg):
         for la in layers:
             assert torch.equal(cache.get(la, "layer", packer(la))[0], la[0])
     assert len(calls) == len(layers)
+
+
+def test_ragged_weights_are_padded_to_whole_blocks_with_zero_codes(pkg):
+    """H or I that 128 does not divide (the reference's weight_dequant_bc takes ceil(n/128) blocks,
+    fusedMoE.pl:11-34): stacking pads gate, up and down with zero codes; every value keeps its place and its scale."""
+    E, I, H = 2, 200, 320
+    g = torch.Generator().manual_seed(3)
+    mk = lambda *s: (torch.randn(*s, generator=g) * 0.1).to(torch.float8_e4m3fn)
+    gate, up, down_t = mk(E, I, H), mk(E, I, H), mk(E, I, H)
+    gs, us, ds = (torch.rand(E, 2, 3, generator=g).to(torch.bfloat16) for _ in range(3))
+    w13, w13s, w2, w2s = pkg.stack_expert_weights(gate, up, down_t, gs, us, ds)
+    assert tuple(w13.shape) == (E, 512, 384) and tuple(w2.shape) == (E, 384, 256)
+    assert tuple(w13s.shape) == (E, 4, 3) and tuple(w2s.shape) == (E, 3, 2) and w13s.dtype == torch.float32
+    b = lambda t: t.view(torch.uint8)
+    assert torch.equal(b(w13)[:, :I, :H], b(gate)) and torch.equal(b(w13)[:, 256:256 + I, :H], b(up))
+    assert torch.equal(b(w2)[:, :H, :I], b(down_t).transpose(1, 2))
+    assert int(b(w13)[:, I:256].sum()) == 0 and int(b(w13)[:, 256 + I:].sum()) == 0 and int(b(w13)[:, :, H:].sum()) == 0
+    assert int(b(w2)[:, H:].sum()) == 0 and int(b(w2)[:, :, I:].sum()) == 0
+    assert torch.equal(w13s[:, :2], gs.float()) and torch.equal(w13s[:, 2:], us.float())
+    assert torch.equal(w2s, ds.float().transpose(1, 2))

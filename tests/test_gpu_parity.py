@@ -711,3 +711,48 @@ def test_experts_w8a16_in_registers(pkg, oracle, dev, T, H, I, E, K):
     want2 = pkg.weighted_reduce(got, wd)
     torch.cuda.synchronize()
     assert torch.equal(out2.view(torch.int16), want2.view(torch.int16))
+
+
+@pytest.mark.parametrize("T,H,I,E,K", [(9, 320, 192, 8, 2), (70, 448, 200, 4, 2), (3, 7168, 200, 16, 4)])
+def test_my_ops_ragged_block_edges(pkg, oracle, dev, T, H, I, E, K):
+    """H or I that 128 does not divide: the reference's weight_dequant_bc takes ceil(n/128) blocks, the last one
+    partial (torch_tpu/csrc/ops/my_ops/fusedMoE.pl:11-34); here the packed copy is padded to whole blocks with zero
+    codes.  Checked against the reference's CPU ground truth on the un-padded tensors (test_moe.py:10-98): the default
+    arithmetic within cos_sim > 0.99, the reference's own arithmetic (set_expert_numerics('w8a16')) within its full
+    criterion, cos_diff < 1e-4 (test_moe.py:308)."""
+    say("ragged", T, H, I, E, K)
+    g = torch.Generator().manual_seed(H + I)
+    nb = lambda n: (n + 127) // 128
+    w0, w1 = ((torch.randn(E, I, H, generator=g) * 0.1).to(torch.float8_e4m3fn) for _ in range(2))
+    w2 = (torch.randn(E, H, I, generator=g) * 0.1).to(torch.float8_e4m3fn)
+    s0, s1 = ((torch.randn(E, nb(I), nb(H), generator=g) * 0.1).to(torch.bfloat16) for _ in range(2))
+    s2 = (torch.randn(E, nb(H), nb(I), generator=g) * 0.1).to(torch.bfloat16)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    ids, w = distinct_ids(T, E, K, seed=T + 11)
+    ref = oracle.experts_ref_bf16(x, ids, w0, w1, w2, s0, s1, s2).float()
+    args = [x.to(dev), None, None, w0.to(dev), w1.to(dev), w2.transpose(1, 2).contiguous().to(dev),
+            s0.to(dev), s1.to(dev), s2.transpose(1, 2).contiguous().to(dev), ids.to(dev), w.to(torch.bfloat16).to(dev), None,
+            None, None, 128, E, K, False, 1, 1, None, None, None, False]
+    out = torch.full((T, K, H), float("nan"), dtype=torch.bfloat16, device=dev)
+    r = torch.ops.my_ops.fused_moe_fused_experts(out, *args)
+    torch.cuda.synchronize()
+    assert r.data_ptr() == out.data_ptr()
+    got = out.float().cpu()
+    assert torch.isfinite(got).all()
+    assert oracle.cos_sim(ref.numpy(), got.numpy()) > 0.99
+    assert oracle.cal_diff(ref, got)[0] < 5e-3
+    pkg.set_expert_numerics("w8a16")
+    try:
+        out16 = torch.full((T, K, H), float("nan"), dtype=torch.bfloat16, device=dev)
+        torch.ops.my_ops.fused_moe_fused_experts(out16, *args)
+        out_w = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=dev)
+        torch.ops.my_ops.fused_moe_fused_experts(out_w, *args)
+        torch.cuda.synchronize()
+    finally:
+        pkg.set_expert_numerics("w8a8")
+    got16 = out16.float().cpu()
+    assert torch.isfinite(got16).all()
+    assert oracle.cos_sim(ref.numpy(), got16.numpy()) > 0.99
+    assert oracle.cal_diff(ref, got16)[0] < 1e-4
+    want = torch.einsum("tk,tkh->th", w.to(torch.bfloat16).float(), got16)
+    assert ((out_w.float().cpu() - want).abs() <= 2e-2 * want.abs() + 2e-2 * want.pow(2).mean().sqrt()).all()

@@ -15,13 +15,30 @@ import torch
 from . import ops
 
 
+def _pad_to(t, rows: int, cols: int):
+    """Zero-pads the last two dimensions of t up to [rows, cols] (code 0 is +0.0 in e4m3fn as in every float type)."""
+    r, c = t.shape[-2:]
+    if r == rows and c == cols:
+        return t
+    if t.dtype == torch.float8_e4m3fn:
+        return torch.nn.functional.pad(t.view(torch.uint8), (0, cols - c, 0, rows - r)).view(torch.float8_e4m3fn)
+    return torch.nn.functional.pad(t, (0, cols - c, 0, rows - r))
+
+
 def stack_expert_weights(gate, up, down_t, gate_scale, up_scale, down_t_scale):
     """Reference-layout fp8 weights -> (w13, w13_scale, w2, w2_scale), ROW-MAJOR: gate rows followed by up rows,
     down back in its checkpoint orientation, scales widened to fp32.  Pure data movement (concatenate / transpose /
-    widen) on whatever device the tensors live; values are untouched."""
-    w13 = torch.cat([gate, up], dim=1).contiguous()
+    widen) on whatever device the tensors live; values are untouched.
+
+    H or I that 128 does not divide (the reference de-quantises ceil(n/128) blocks, the last one partial:
+    torch_tpu/csrc/ops/my_ops/fusedMoE.pl:11-34): gate, up and down are padded with zero codes to the next multiple
+    of 128 in both dimensions - the scale tensors already hold ceil(n/128) blocks - so that every block is whole;
+    zero weights add nothing to any sum, and a caller pads the activations' columns the same way."""
+    I, H = gate.shape[-2:]
+    Ip, Hp = -(-I // 128) * 128, -(-H // 128) * 128
+    w13 = torch.cat([_pad_to(gate, Ip, Hp), _pad_to(up, Ip, Hp)], dim=1).contiguous()
     w13_scale = torch.cat([gate_scale, up_scale], dim=1).to(torch.float32).contiguous()
-    w2 = down_t.transpose(1, 2).contiguous()
+    w2 = _pad_to(down_t, Ip, Hp).transpose(1, 2).contiguous()
     w2_scale = down_t_scale.transpose(1, 2).to(torch.float32).contiguous()
     return w13, w13_scale, w2, w2_scale
 

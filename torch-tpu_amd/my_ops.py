@@ -210,8 +210,26 @@ def _fused_experts(output, input, output_sample, input_sample, gate_weights, up_
     if w13.shape[0] != num_experts or select_experts.shape[1] != num_experts_per_tok:
         raise RuntimeError("num_experts / num_experts_per_tok do not match the tensors")
     T, H = input.shape
-    E, I2, _ = w13.shape
+    E, I2, Hp = w13.shape
     rw = _routing_f32(routing_weights, input.device) if output.dim() == 2 else None
+    real_output = None
+    if Hp != H:
+        # ragged hidden size: the packed weights were padded to whole 128-blocks with zeros; the activations get
+        # zero columns to match (they change no group's maximum and add nothing to any sum) and the result's
+        # padding columns are dropped
+        input = torch.nn.functional.pad(input, (0, Hp - H))
+        real_output, output = output, torch.empty(*output.shape[:-1], Hp, dtype=output.dtype, device=output.device)
+        H = Hp
+    output = _run_packed(output, input, w13, w13s, w2, w2s, select_experts, rw)
+    if real_output is not None:
+        real_output.copy_(output[..., :real_output.shape[-1]])
+        return real_output
+    return output
+
+
+def _run_packed(output, input, w13, w13s, w2, w2s, select_experts, rw):
+    T, H = input.shape
+    E, I2, _ = w13.shape
     if _numerics == "w8a16":
         ws = _workspace(input.device, ops.fused_experts_bf16_workspace_bytes(T, H, I2 // 2, E, select_experts.shape[1]))
         ops.fused_experts_w8a16(input, w13, w13s, w2, w2s, select_experts, rw, out=output, workspace=ws)
