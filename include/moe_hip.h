@@ -243,6 +243,14 @@ int moe_mm_fp8(void *stream, const void *x_bf16, int M, int K, const uint8_t *w,
  * of 16.  No workspace.
  */
 int moe_mm_bf16(void *stream, const void *x_bf16, int M, int K, const void *w_bf16, int N, void *out_bf16);
+/*
+ * The same arithmetic without a de-quantised copy: w [N, K] fp8 (tile-blocked) with fp32 scales
+ * [ceil(N/128), K/128] is de-quantised to bf16(float(code) * scale) in registers on the way into the bf16 matrix
+ * instructions (MmW8A16Dq.cpp:185-228; python/regression/test_llm/test_mm_w8a16_dq.py:10-60).  K a multiple of 128
+ * and at most 16384, N a multiple of 16.  No workspace.
+ */
+int moe_mm_w8a16(void *stream, const void *x_bf16, int M, int K, const uint8_t *w, const float *w_scale, int N,
+                 void *out_bf16);
 size_t moe_mlp_fp8_workspace_bytes(int M, int H, int I);
 int moe_mlp_fp8(void *stream, const void *x_bf16, int M, int H, const uint8_t *w13, const float *w13_scale,
                 const uint8_t *w2, const float *w2_scale, int I, void *out_bf16, void *workspace,

@@ -137,3 +137,55 @@ def test_dense_ops_reject_what_they_do_not_support(pkg, dev):
         torch.ops.my_ops.mm_w8a16_dq_forward(x, w, s, out, 0)
     with pytest.raises(RuntimeError):
         torch.ops.my_ops.mm_w8a16_dq_forward(x, w.view(torch.uint8), s, out, 128)
+
+
+@pytest.mark.parametrize("M,K,N", [(32, 7168, 1536), (1, 256, 16), (200, 384, 272), (100, 4096, 8192), (300, 1024, 2048)])
+def test_mm_in_the_references_own_arithmetic(pkg, oracle, dev, M, K, N):
+    """set_expert_numerics('w8a16'): mm_w8a16_dq_forward multiplies bf16 activations with weights de-quantised in
+    registers (MmW8A16Dq.cpp:185-228); against the reference's bf16 ground truth
+    (python/regression/test_llm/test_mm_w8a16_dq.py:52-60) cos_diff < 1e-4, which the FP8-activation path cannot reach."""
+    say("mm w8a16", M, K, N)
+    g = torch.Generator().manual_seed(3000 + M + N)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = torch.randn(N, K, generator=g).to(torch.float8_e4m3fn)
+    s = torch.randn((N + 127) // 128, K // 128, generator=g).to(torch.bfloat16)
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+    pkg.set_expert_numerics("w8a16")
+    try:
+        torch.ops.my_ops.mm_w8a16_dq_forward(x.to(dev), w.to(dev), s.to(dev), out, 128)
+        torch.cuda.synchronize()
+    finally:
+        pkg.set_expert_numerics("w8a8")
+    got = out.float().cpu()
+    assert torch.isfinite(got).all()
+    ref = oracle.mm_w8a16_dq_ref(x, w, s).float()
+    assert oracle.cos_sim(ref.flatten(), got.flatten()) >= 0.99
+    assert oracle.cal_diff(ref, got)[0] < 1e-4
+    # element-wise: one bf16 rounding of an fp32 sum against the reference's bf16 matmul
+    rms = ref.pow(2).mean().sqrt()
+    assert ((got - ref).abs() <= 1.6e-2 * ref.abs() + 1e-2 * rms).all()
+
+
+@pytest.mark.parametrize("M,H,I", [(32, 7168, 256), (1, 256, 128), (200, 512, 384), (300, 1024, 1024)])
+def test_mlp_in_the_references_own_arithmetic(pkg, oracle, dev, M, H, I):
+    """The gated MLP likewise (MlpW8A16Dq.cpp:189-241; python/regression/test_llm/test_mlp_w8a16_dq.py:53-81)."""
+    say("mlp w8a16", M, H, I)
+    g = torch.Generator().manual_seed(4000 + M + I)
+    x = torch.randn(M, H, generator=g).to(torch.bfloat16)
+    wg, wu = (torch.randn(I, H, generator=g).to(torch.float8_e4m3fn) for _ in range(2))
+    wd = torch.randn(H, I, generator=g).to(torch.float8_e4m3fn)
+    sg, su = ((torch.randn(I // 128, H // 128, generator=g) * 0.05).to(torch.bfloat16) for _ in range(2))
+    sd = (torch.randn(H // 128, I // 128, generator=g) * 0.05).to(torch.bfloat16)
+    out = torch.full((M, H), float("nan"), dtype=torch.bfloat16, device=dev)
+    pkg.set_expert_numerics("w8a16")
+    try:
+        torch.ops.my_ops.mlp_w8a16_dq_forward(x.to(dev), wg.to(dev), wu.to(dev), wd.T.to(dev), sg.to(dev), su.to(dev),
+                                              sd.T.to(dev), out, 128)
+        torch.cuda.synchronize()
+    finally:
+        pkg.set_expert_numerics("w8a8")
+    got = out.float().cpu()
+    assert torch.isfinite(got).all()
+    ref = oracle.mlp_w8a16_dq_ref(x, wg, wu, wd, sg, su, sd).float()
+    assert oracle.cos_sim(ref.flatten(), got.flatten()) >= 0.99
+    assert oracle.cal_diff(ref, got)[0] < 1e-4

@@ -53,6 +53,7 @@ SIGNATURES = {
     "moe_mm_fp8_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "moe_mm_fp8": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_size_t]),
     "moe_mm_bf16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p]),
+    "moe_mm_w8a16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]),
     "moe_mlp_fp8_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "moe_mlp_fp8": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                             c_void_p, c_void_p, c_size_t]),

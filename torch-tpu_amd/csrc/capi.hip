@@ -453,6 +453,21 @@ extern "C" int moe_mm_bf16(void *stream, const void *x_bf16, int M, int K, const
                       nullptr, kNumericsBf16);
 }
 
+// The same product in the reference's own arithmetic: bf16 activations against FP8 weights de-quantised in registers
+extern "C" int moe_mm_w8a16(void *stream, const void *x_bf16, int M, int K, const uint8_t *w, const float *w_scale, int N,
+                            void *out_bf16) {
+  using namespace moe;
+  if (!w || !w_scale) return MOE_E_NULL;
+  if (M != 0 && (!x_bf16 || !out_bf16)) return MOE_E_NULL;
+  if (M < 0 || K < 1 || N < 16 || K > 16384 || N > (1 << 20)) return MOE_E_SHAPE;
+  if (K % kBlock || N % 16) return MOE_E_ALIGN;
+  if ((double)M * K * 2 >= 2147483648.0 || (double)M * N >= 2147483648.0 || (double)N * K >= 4294967296.0) return MOE_E_SHAPE;
+  if (((uintptr_t)x_bf16 % 16) || ((uintptr_t)out_bf16 % 16) || ((uintptr_t)w % 16)) return MOE_E_ALIGN;
+  if (M == 0) return MOE_OK;
+  return gemm2_launch((hipStream_t)stream, (const uint8_t *)x_bf16, nullptr, M, M, N, w, w_scale, K, 1, 1, nullptr, nullptr,
+                      nullptr, 0, (uint16_t *)out_bf16, nullptr, nullptr, 0, nullptr, nullptr, nullptr, kNumericsW8A16);
+}
+
 extern "C" size_t moe_mlp_fp8_workspace_bytes(int M, int H, int I) {
   if (M < 0 || H < 1 || I < 1) return 0;
   return moe::dense_layout(nullptr, M, H, I, H).bytes;

@@ -54,7 +54,8 @@ _lib.define("mm_w8a16_dq_forward(Tensor input, Tensor weight, Tensor scale, Tens
 # activations against weights de-quantised to bf16(float(code) * block scale) IN REGISTERS on the way into the
 # matrix instructions, from the same packed FP8 copy the default mode reads (one byte per weight element, nothing
 # de-quantised in memory); meets the reference's criterion (cos_diff < 1e-4, test_moe.py:308).  Only block sizes
-# that 128 does not divide still go through a bf16 copy de-quantised once.
+# that 128 does not divide still go through a bf16 copy de-quantised once.  The dense ops mm_w8a16_dq_forward and
+# mlp_w8a16_dq_forward follow the same switch.
 _numerics = "w8a8"
 
 
@@ -342,6 +343,14 @@ def _mlp_w8a16_dq_forward(input, gate_weight, up_weight, down_weight, gate_scale
                  torch.cat([_scales_128(gate_scale, blocksize, I, H), _scales_128(up_scale, blocksize, I, H)], 0).contiguous(),
                  ops.pack_weights(down_weight.t().contiguous()), _scales_128(down_scale, blocksize, I, H).t().contiguous()),
         f"mlp{blocksize}")
+    if _numerics == "w8a16" and H <= 16384 and I <= 16384:
+        # the reference's own arithmetic: one expert that every row selects, weights de-quantised in registers
+        M = input.shape[0]
+        ids = torch.zeros(M, 1, dtype=torch.int32, device=input.device)
+        ws = _workspace(input.device, ops.fused_experts_bf16_workspace_bytes(M, H, I, 1, 1))
+        ops.fused_experts_w8a16(input.contiguous(), w13.unsqueeze(0), w13s.unsqueeze(0), w2.unsqueeze(0), w2s.unsqueeze(0), ids,
+                                None, out=output.view(M, 1, H), workspace=ws)
+        return output
     ws = _workspace(input.device, ops.mlp_workspace_bytes(input.shape[0], H, I))
     ops.mlp_fp8(input.contiguous(), w13, w13s, w2, w2s, out=output, workspace=ws)
     return output
@@ -359,6 +368,9 @@ def _mm_w8a16_dq_forward(input, weight, scale, output, blocksize):
         return output
     w, ws = _dense_packed((weight, scale), lambda: (ops.pack_weights(weight.contiguous()),
                                                      _scales_128(scale, blocksize, N, K)), f"mm{blocksize}")
+    if _numerics == "w8a16" and K <= 16384:
+        ops.mm_w8a16(input.contiguous(), w, ws, out=output)
+        return output
     ops.mm_fp8(input.contiguous(), w, ws, out=output, workspace=_workspace(input.device, ops.mm_workspace_bytes(input.shape[0], K, N)))
     return output
 

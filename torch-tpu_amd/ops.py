@@ -443,6 +443,24 @@ def mm_bf16(x, w, out=None):
     return out
 
 
+def mm_w8a16(x, w, w_scale, out=None):
+    """Dense block-scaled linear layer in the reference's arithmetic: x [M,K] bf16 (not quantised), w [N,K] e4m3fn
+    (tile-blocked) de-quantised in registers to bf16(float(code) * scale), fp32 scales [ceil(N/128), K/128]
+    -> out [M,N] bf16."""
+    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], "x must be [M,K] and w [N,K]")
+    M, K = x.shape
+    N = w.shape[0]
+    _need(K % 128 == 0, "K must be a multiple of 128")
+    _need(tuple(w_scale.shape) == ((N + 127) // 128, K // 128), "w_scale must be [ceil(N/128), K/128]")
+    if out is None:
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=x.device)
+    _need(tuple(out.shape) == (M, N), "out must be [M,N]")
+    rc = lib.moe_mm_w8a16(_stream(), _dev(x, "x", torch.bfloat16), M, K, _dev(w, "w", _FP8),
+                          _dev(w_scale, "w_scale", torch.float32), N, _dev(out, "out", torch.bfloat16))
+    check(rc, "mm_w8a16")
+    return out
+
+
 def mlp_fp8(x, w13, w13_scale, w2, w2_scale, out=None, workspace=None):
     """Dense gated MLP: x [M,H] bf16, w13 [2I,H] (gate rows then up rows), w2 [H,I], fp32 128x128
     block scales -> out [M,H] bf16 = (silu(x Wg^T) * (x Wu^T)) Wd^T, FP8 matrix products."""
