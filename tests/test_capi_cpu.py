@@ -243,3 +243,23 @@ def test_ragged_weights_are_padded_to_whole_blocks_with_zero_codes(pkg):
     assert int(b(w2)[:, H:].sum()) == 0 and int(b(w2)[:, :, I:].sum()) == 0
     assert torch.equal(w13s[:, :2], gs.float()) and torch.equal(w13s[:, 2:], us.float())
     assert torch.equal(w2s, ds.float().transpose(1, 2))
+
+
+def test_bench_hands_on_the_offline_traffic_only_for_the_profiled_sources():
+    """bench.py's roofline.traffic is an offline rocprofv3 figure kept in the profile summary: it is reported for the
+    profiled workload while the kernel sources hash to the value recorded there, and withheld (None + a reason) otherwise."""
+    import importlib.util
+    here = os.path.dirname(os.path.abspath(__file__))
+    spec = importlib.util.spec_from_file_location("_bench_under_test", os.path.join(here, "..", "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    shape = (4096, 7168, 2048, 256, 8)
+    got, why = bench.offline_traffic(shape)
+    with open(bench.TRAFFIC_FILE) as f:
+        rec = next(__import__("json").loads(l.split(None, 1)[1]) for l in f if l.startswith("TRAFFIC "))
+    if rec["kernel_source_sha16"] == bench.kernel_source_hash():
+        assert got == rec["bytes_per_launch"] and 7.6e9 < got < 8.2e9 and "offline" in why
+    else:
+        assert got is None and "stale" in why
+    other, why2 = bench.offline_traffic((1, 2, 3, 4, 5))
+    assert other is None and "another workload" in why2
