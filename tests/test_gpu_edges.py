@@ -36,6 +36,9 @@ def test_empty_batch_is_a_valid_call_everywhere(pkg, oracle, dev):
     w13b = torch.zeros(E, 2 * I, H, dtype=torch.bfloat16, device=dev)
     w2b = torch.zeros(E, H, I, dtype=torch.bfloat16, device=dev)
     assert pkg.fused_experts_bf16(x, w13b, w2b, ids, w).shape == (0, H)
+    assert pkg.fused_experts_w8a16(x, *ld, ids).shape == (0, K, H)
+    assert pkg.fused_experts_w8a16(x, *ld, ids, w).shape == (0, H)
+    assert pkg.mm_w8a16(x, ld[0][0], ld[1][0]).shape == (0, 2 * I)
     assert pkg.mm_fp8(x, ld[0][0], ld[1][0]).shape == (0, 2 * I)
     assert pkg.mlp_fp8(x, ld[0][0], ld[1][0], ld[2][0], ld[3][0]).shape == (0, H)
     moe = pkg.FusedMoE(wr, *ld, top_k=K, mode="softmax")
@@ -116,6 +119,16 @@ def test_slots_without_an_expert_add_nothing(pkg, oracle, dev, T):
     outb2 = pkg.fused_experts_bf16(x.to(dev), w13b, w2b, ids_bad.to(dev), w.to(dev))
     torch.cuda.synchronize()
     assert torch.isfinite(outb2.float()).all() and bool((outb2.float().cpu()[0] == 0).all())
+    # and so does the reference's arithmetic on the packed FP8 weights
+    outd = torch.full((T, K, H), float("nan"), dtype=torch.bfloat16, device=dev)
+    pkg.fused_experts_w8a16(x.to(dev), *dl, ids_bad.to(dev), out=outd)
+    outd2 = pkg.fused_experts_w8a16(x.to(dev), *dl, ids_bad.to(dev), w.to(dev))
+    torch.cuda.synchronize()
+    gotd = outd.float().cpu()
+    assert torch.isfinite(gotd).all() and bool((gotd[bad] == 0).all())
+    assert torch.isfinite(outd2.float()).all() and bool((outd2.float().cpu()[0] == 0).all())
+    live = ~bad
+    assert oracle.cal_diff(ref_slots[live], gotd[live])[0] < 5e-3      # un-quantised activations against the W8A8 oracle
 
 
 def test_one_workspace_serves_calls_of_different_sizes(pkg, oracle, dev):
