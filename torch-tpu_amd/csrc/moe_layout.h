@@ -28,12 +28,13 @@ static inline int choose_tile_m(int T, int K, int E) {
   // Balanced routing puts T*K/E rows on an expert, give or take a few standard deviations.  A
   // second, nearly empty tile costs as much weight traffic as a full one, so prefer the tile
   // that holds a typical expert whole.
-  // Up to ~48 rows per expert the 64-row tile wins although a few experts then need two tiles: its
-  // kernel keeps both operands in LDS and fetches the weights in whole cache lines (measured on the
-  // DeepSeek-V3 shape: 64 best up to T=1536, 128 at T=2048, 192 from T=3072 on).
+  // Measured on the DeepSeek-V3 shape (tile-blocked weights; step in ms with 64 / 128 / 192 rows forced): T=512 (16 rows
+  // per expert on average) 1.977 / 1.978 / 1.992, T=768 2.035 / 2.023 / 2.034, T=1024 2.076 / 2.053 / 2.082,
+  // T=1536 2.180 / 2.141 / 2.146, T=2048 2.477 / 2.221 / 2.252, T=3072 (96 rows) 2.993 / 2.404 / 2.410,
+  // T=4096 (128 rows) 3.627 / 2.924 / 2.651.
   const double mean = (double)T * K / E;
-  if (mean <= 48.0) return 64;
-  return mean > 84.0 ? 192 : 128;
+  if (mean <= 20.0) return 64;
+  return mean > 104.0 ? 192 : 128;
 }
 
 struct PermuteWs {
