@@ -323,7 +323,7 @@ def device_step_with_routing(pkg, moe, cfg, x):
     T = x.shape[0]
     if moe._one_call(T):
         out, logits, w, ids = pkg.layer_fp8(
-            x, moe.router_weight, moe.w13, moe.w13_scale, moe.w2, moe.w2_scale, cfg["K"], cfg["route"], moe.bias,
+            x, moe.router_weight, moe.w13, moe.w13_scale, moe.w2, moe.w2_scale, cfg["K"], moe.layer_mode(), moe.bias,
             cfg["n_groups"], cfg["topk_groups"], True, cfg["scale"], shared=moe.shared, return_routing=True,
             workspace=moe._workspace(T, True))
     else:

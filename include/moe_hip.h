@@ -54,6 +54,8 @@ extern "C" {
 #define MOE_ROUTE_SOFTMAX 0   /* select on logits; weights = softmax over all experts      */
 #define MOE_ROUTE_SIGMOID 1   /* scores = sigmoid(logit); select on scores + bias          */
 #define MOE_ROUTE_SCORES  2   /* the input already holds scores; select on scores + bias   */
+#define MOE_ROUTE_SOFTMAX_LOGIT_BIAS 3  /* MOE_ROUTE_SOFTMAX on logits + bias: the bias is part of the logits
+                                           (selection AND weights see it), as a softmax router's own bias term */
 
 #define MOE_MAX_EXPERTS 1024
 #define MOE_MAX_TOPK    32
@@ -81,7 +83,8 @@ int moe_noaux_tc_topk(void *stream, const void *scores, int scores_dtype, int T,
  * reference's callers run (python/regression/test_llm/test_torch_ops.py:441-456:
  * sigmoid -> topk -> sum -> div -> mul) and the softmax/top-k variant
  * (torch_tpu/csrc/ops/native_ops/Topk.cpp:91-205).
- * logits [T, E] (dtype selector), bias [E] fp32 or NULL (added for selection only).
+ * logits [T, E] (dtype selector), bias [E] fp32 or NULL (added for selection only; with
+ * MOE_ROUTE_SOFTMAX_LOGIT_BIAS added to the logits themselves, so that selection and weights both see it).
  * n_groups <= 1 disables group limiting.  renorm != 0 divides by the sum of the selected
  * weights; the result is multiplied by `scale`.
  * weights_out [T, K] fp32, ids_out [T, K] int32 (descending selection order),
@@ -267,7 +270,8 @@ int moe_mlp_fp8(void *stream, const void *x_bf16, int M, int H, const uint8_t *w
  * router product runs on the matrix cores with its reduction cut into slices, the routing kernel adds
  * the slices, and the activations are quantised by extra workgroups of that launch.  Either way the logits
  * are fp32 sums rounded once to bf16.
- * router_w_bf16 [E, H] bf16; router_bias [E] fp32 or NULL (selection only, as in moe_route_topk);
+ * router_w_bf16 [E, H] bf16; router_bias [E] fp32 or NULL (selection only, or part of the logits with
+ * MOE_ROUTE_SOFTMAX_LOGIT_BIAS, as in moe_route_topk);
  * mode MOE_ROUTE_SOFTMAX or MOE_ROUTE_SIGMOID; the other routing arguments as in moe_route_topk.
  * out bf16 [T, H] (the weighted sum, shared expert added when its pointers are non-NULL).
  * logits_out_bf16 [T, E], weights_out [T, K], ids_out [T, K]: optional copies of what the router

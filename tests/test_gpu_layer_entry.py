@@ -150,6 +150,40 @@ def test_layer_entry_point(pkg, oracle, dev, checks, T, H, I, E, K, mode, G, TG,
     say("   ", {k: (round(v, 6) if isinstance(v, float) else v) for k, v in rep.items()})
 
 
+@pytest.mark.parametrize("T", [1, 5, 32, 300, 2000])
+def test_softmax_router_whose_bias_is_part_of_the_logits(pkg, oracle, dev, T):
+    """MOE_ROUTE_SOFTMAX_LOGIT_BIAS: softmax over logits + bias (selection and weights see the bias), the form a
+    softmax router's own bias term takes - a skewed-load layer switches experts off with it.  One call through the
+    layer entry point equals the staged road (logits + bias on the host side, plain softmax routing) bit for bit."""
+    say("softmax router with a logit bias", T)
+    H, I, E, K = 1024, 256, 64, 6
+    ld = pkg.pack_layer(*(t.to(dev) for t in oracle.make_layer(E, H, I, seed=T + 1)))
+    g = torch.Generator().manual_seed(17 * T + 3)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+    wr = (torch.randn(E, H, generator=g) * 0.05).to(torch.bfloat16).to(dev)
+    bias = -1.2 * torch.log(torch.randperm(E, generator=g).float() + 1)
+    off = torch.randperm(E, generator=g)[:7]
+    bias[off] = -1e9                                                   # experts that must never be chosen
+    biasd = bias.to(dev)
+    out, logits, w, ids = pkg.layer_fp8(x, wr, *ld, K, "softmax_logit_bias", bias=biasd, return_routing=True)
+    w1, ids1 = pkg.moe_route(logits, K, "softmax_logit_bias", bias=biasd)
+    w2_, ids2 = pkg.moe_route(logits.float() + biasd, K, "softmax")
+    torch.cuda.synchronize()
+    assert torch.equal(ids, ids1) and torch.equal(w, w1)
+    assert torch.equal(ids, ids2) and torch.equal(w, w2_)
+    assert not bool(torch.isin(ids.cpu().long(), off).any())
+    w_ref, ids_ref = oracle.route_softmax_topk(logits.float().cpu() + bias, K)
+    assert torch.equal(ids.cpu(), ids_ref) and torch.allclose(w.cpu(), w_ref, rtol=1e-5, atol=1e-7)
+    ref_out = pkg.fused_experts_fp8(x, *ld, ids, w)
+    assert torch.equal(out.view(torch.int16), ref_out.view(torch.int16))
+    # the module hands a softmax router's bias over in this form by itself
+    moe = pkg.FusedMoE(wr, *ld, top_k=K, mode="softmax", bias=biasd)
+    assert moe._one_call(T) and moe.layer_mode() == "softmax_logit_bias"
+    assert torch.equal(moe(x).view(torch.int16), out.view(torch.int16))
+    wm, im = moe.route(x)                                              # its staged road: torch.matmul logits + bias
+    assert not bool(torch.isin(im.cpu().long(), off).any())
+
+
 @pytest.mark.parametrize("T,H,E", [(1, 128, 1), (5, 7168, 256), (64, 256, 16), (65, 384, 100), (700, 7168, 256),
                                    (4096, 2048, 128), (130, 9216, 37)])
 def test_router_logits_kernel(pkg, dev, T, H, E):

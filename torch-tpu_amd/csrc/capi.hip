@@ -232,7 +232,7 @@ static int layer_fp8_run(void *stream, const void *x_bf16, int T, int H, const v
   if (T < 0 || H < 1 || I < 1 || E < 1 || E > 256 || K < 1 || K > MOE_MAX_TOPK || K > E) return MOE_E_SHAPE;
   if ((long)T * K > (1l << 30)) return MOE_E_SHAPE;
   if (!dims_in_range(T, H, I, K)) return MOE_E_SHAPE;
-  if (mode != MOE_ROUTE_SOFTMAX && mode != MOE_ROUTE_SIGMOID) return MOE_E_MODE;
+  if (mode != MOE_ROUTE_SOFTMAX && mode != MOE_ROUTE_SIGMOID && mode != MOE_ROUTE_SOFTMAX_LOGIT_BIAS) return MOE_E_MODE;
   if (H % kBlock || I % kBlock) return MOE_E_ALIGN;
   const bool has_shared = shared_w13 != nullptr;
   if (has_shared) {

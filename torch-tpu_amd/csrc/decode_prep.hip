@@ -133,7 +133,7 @@ int decode_prep_launch(hipStream_t st, const uint16_t *x, int T, int H, const ui
                        int32_t *ids, int *arrivals, uint8_t *xq, float *xs, int tile_m, int32_t *sorted_slot,
                        int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &pw) {
   if (T < 1 || (long)T * K > kChunk || E > kRouteBlock || H % kBlock) return MOE_E_SHAPE;
-  if (mode != MOE_ROUTE_SOFTMAX && mode != MOE_ROUTE_SIGMOID) return MOE_E_MODE;
+  if (mode != MOE_ROUTE_SOFTMAX && mode != MOE_ROUTE_SIGMOID && mode != MOE_ROUTE_SOFTMAX_LOGIT_BIAS) return MOE_E_MODE;
   const int rc = check_route_shape(T, E, K, n_groups, topk_groups);
   if (rc) return rc;
   const int n_logit_blocks = E * ((T + kLogitTokens - 1) / kLogitTokens);

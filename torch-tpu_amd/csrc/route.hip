@@ -221,6 +221,8 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const void *__restrict_
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (t >= T) return;
+  const bool logit_bias = mode == MOE_ROUTE_SOFTMAX_LOGIT_BIAS;
+  if (logit_bias) mode = MOE_ROUTE_SOFTMAX;
   float raw[PER_LANE];   // score used for the weight (before the bias)
   float v[PER_LANE];     // score used for the selection
   float row_max = -INFINITY;
@@ -237,9 +239,10 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const void *__restrict_
       else x = ((const float *)logits)[(size_t)t * E + e];
     }
     if (mode == MOE_ROUTE_SIGMOID && e < E) x = 1.0f / (1.0f + expf(-x));
+    if (logit_bias && bias != nullptr && e < E) x += bias[e];      // the bias is part of the logits
     raw[j] = x;
     row_max = fmaxf(row_max, x);
-    v[j] = (bias != nullptr && e < E) ? x + bias[e] : x;
+    v[j] = (!logit_bias && bias != nullptr && e < E) ? x + bias[e] : x;
     if (scores_out != nullptr && e < E && mode != MOE_ROUTE_SOFTMAX) scores_out[(size_t)t * E + e] = x;
   }
   float denom_all = 0.f;
@@ -345,7 +348,7 @@ int route_from_partials_launch(hipStream_t st, const float *partial, int n_slice
                                int mode, int n_groups, int topk_groups, int renorm, float scale, float *weights_out,
                                int32_t *ids_out, const uint16_t *x, int H, uint8_t *xq, float *xs) {
   if (E > 256 || n_slices < 1) return MOE_E_SHAPE;
-  if (mode != MOE_ROUTE_SOFTMAX && mode != MOE_ROUTE_SIGMOID) return MOE_E_MODE;
+  if (mode != MOE_ROUTE_SOFTMAX && mode != MOE_ROUTE_SIGMOID && mode != MOE_ROUTE_SOFTMAX_LOGIT_BIAS) return MOE_E_MODE;
   const int rc = check_route_shape(T, E, K, n_groups, topk_groups);
   if (rc) return rc;
   const int route_blocks = (T + 3) / 4;
@@ -395,7 +398,8 @@ extern "C" int moe_route_topk(void *stream, const void *logits, int logits_dtype
   using namespace moe;
   if (T != 0 && (!logits || !weights_out || !ids_out)) return MOE_E_NULL;
   if (logits_dtype != MOE_DTYPE_F32 && logits_dtype != MOE_DTYPE_BF16) return MOE_E_MODE;
-  if (mode != MOE_ROUTE_SOFTMAX && mode != MOE_ROUTE_SIGMOID && mode != MOE_ROUTE_SCORES) return MOE_E_MODE;
+  if (mode != MOE_ROUTE_SOFTMAX && mode != MOE_ROUTE_SIGMOID && mode != MOE_ROUTE_SCORES && mode != MOE_ROUTE_SOFTMAX_LOGIT_BIAS)
+    return MOE_E_MODE;
   int rc = check_route_shape(T, E, K, n_groups, topk_groups);
   if (rc) return rc;
   if (T == 0) return MOE_OK;

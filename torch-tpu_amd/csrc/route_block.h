@@ -45,6 +45,12 @@ __device__ __forceinline__ void route_block(RouteBlockSmem &sm, const void *logi
   float x = -INFINITY;
   if (live) x = logits_bf16 ? bf16_to_f32(((const uint16_t *)logits_row)[e]) : ((const float *)logits_row)[e];
   if (mode == MOE_ROUTE_SIGMOID && live) x = 1.0f / (1.0f + expf(-x));
+  const bool logit_bias = mode == MOE_ROUTE_SOFTMAX_LOGIT_BIAS;     // the bias is part of the logits
+  if (logit_bias) {
+    mode = MOE_ROUTE_SOFTMAX;
+    if (bias != nullptr && live) x += bias[e];
+    bias = nullptr;
+  }
   float raw = x;                                          // what the weight is made of (no bias)
   float v = (bias != nullptr && live) ? x + bias[e] : x;  // what the selection looks at
   if (scores_row != nullptr && live && mode != MOE_ROUTE_SOFTMAX) scores_row[e] = x;

@@ -162,16 +162,17 @@ class FusedMoE:
                                      shared=self.shared, workspace=self._workspace(x.shape[0]))
 
     def _one_call(self, T):
-        # a softmax router's bias belongs to the logits, which the one-call entry point computes itself
-        return (ops.layer_eligible(T, self.w13.shape[0], self.top_k)
-                and not (self.mode == "softmax" and self.bias is not None)
-                and self.router_weight.dtype == torch.bfloat16)
+        return ops.layer_eligible(T, self.w13.shape[0], self.top_k) and self.router_weight.dtype == torch.bfloat16
+
+    def layer_mode(self):
+        """The routing mode handed to the one-call entry point: a softmax router's bias is part of the logits."""
+        return "softmax_logit_bias" if self.mode == "softmax" and self.bias is not None else self.mode
 
     def __call__(self, x, out=None):
         T = x.shape[0]
         if self._one_call(T):      # router and experts behind one entry point
             return ops.layer_fp8(x, self.router_weight, self.w13, self.w13_scale, self.w2, self.w2_scale,
-                                        self.top_k, self.mode, self.bias, self.n_groups, self.topk_groups, self.renorm,
+                                        self.top_k, self.layer_mode(), self.bias, self.n_groups, self.topk_groups, self.renorm,
                                         self.scale, shared=self.shared, out=out, workspace=self._workspace(T, True))
         weights, ids = self.route(x)
         return self.experts(x, weights, ids, out)

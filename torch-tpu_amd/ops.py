@@ -12,7 +12,7 @@ import torch
 
 from ._lib import MoeHipError, check, lib
 
-ROUTE_SOFTMAX, ROUTE_SIGMOID, ROUTE_SCORES = 0, 1, 2
+ROUTE_SOFTMAX, ROUTE_SIGMOID, ROUTE_SCORES, ROUTE_SOFTMAX_LOGIT_BIAS = 0, 1, 2, 3
 _FP8 = torch.float8_e4m3fn
 
 
@@ -67,7 +67,8 @@ def moe_route(logits, k: int, mode: str = "softmax", bias=None, n_groups: int = 
               renorm: bool = True, scale: float = 1.0, return_scores: bool = False):
     """Top-k routing from router logits -> (fp32 weights [T,k], int32 ids [T,k][, fp32 scores [T,E]]).
     mode: "softmax" | "sigmoid" | "scores" (the input already holds scores)."""
-    modes = {"softmax": ROUTE_SOFTMAX, "sigmoid": ROUTE_SIGMOID, "scores": ROUTE_SCORES}
+    modes = {"softmax": ROUTE_SOFTMAX, "sigmoid": ROUTE_SIGMOID, "scores": ROUTE_SCORES,
+             "softmax_logit_bias": ROUTE_SOFTMAX_LOGIT_BIAS}     # softmax over logits + bias (the bias is part of the logits)
     _need(mode in modes, f"unknown routing mode {mode!r}")
     _need(logits.dim() == 2, "logits must be [T, E]")
     T, E = logits.shape
@@ -278,7 +279,7 @@ def layer_fp8(x, router_weight, w13, w13_scale, w2, w2_scale, top_k: int, mode: 
     or (out, logits bf16 [T,E], weights fp32 [T,k], ids int32 [T,k]) with return_routing.
     static_scratch: use the library's built-in scratch array instead of a workspace (moe_layer_fp8_static: no
     device allocation when `out` is given; small batches only, calls on one GPU must not overlap)."""
-    modes = {"softmax": ROUTE_SOFTMAX, "sigmoid": ROUTE_SIGMOID}
+    modes = {"softmax": ROUTE_SOFTMAX, "sigmoid": ROUTE_SIGMOID, "softmax_logit_bias": ROUTE_SOFTMAX_LOGIT_BIAS}
     _need(mode in modes, f"unknown routing mode {mode!r}")
     _need(x.dim() == 2 and w13.dim() == 3 and w2.dim() == 3 and router_weight.dim() == 2, "bad ranks")
     T, H = x.shape
