@@ -143,6 +143,16 @@ def _workspace(device, nbytes: int):
     return ws
 
 
+def _zero_ids(device, rows: int):
+    """[rows, 1] int32 zeros (every row selects expert 0), kept per device and grown on demand."""
+    key = (device, "zero_ids")
+    buf = _scratch.get(key)
+    if buf is None or buf.numel() < rows:
+        buf = torch.zeros(max(rows, 1024), 1, dtype=torch.int32, device=device)
+        _scratch[key] = buf
+    return buf[:rows]
+
+
 def _routing_f32(routing_weights, device):
     """The op's routing weights (bf16 in the reference's callers) as fp32 for the weighted sum, in a buffer that is
     kept per (device, stream) next to the workspace."""
@@ -334,8 +344,9 @@ def _mlp_w8a16_dq_forward(input, gate_weight, up_weight, down_weight, gate_scale
             f"mlp-dequant{blocksize}")
         # one expert that every row selects; its per-slot result [M, 1, H] is the output itself
         M = input.shape[0]
-        ids = torch.zeros(M, 1, dtype=torch.int32, device=input.device)
-        ops.fused_experts_bf16(input.contiguous(), w13, w2, ids, None, out=output.view(M, 1, H))
+        ws = _workspace(input.device, ops.fused_experts_bf16_workspace_bytes(M, H, I, 1, 1))
+        ops.fused_experts_bf16(input.contiguous(), w13, w2, _zero_ids(input.device, M), None, out=output.view(M, 1, H),
+                               workspace=ws)
         return output
     w13, w13s, w2, w2s = _dense_packed(
         (gate_weight, up_weight, down_weight, gate_scale, up_scale, down_scale),
@@ -346,7 +357,7 @@ def _mlp_w8a16_dq_forward(input, gate_weight, up_weight, down_weight, gate_scale
     if _numerics == "w8a16" and H <= 16384 and I <= 16384:
         # the reference's own arithmetic: one expert that every row selects, weights de-quantised in registers
         M = input.shape[0]
-        ids = torch.zeros(M, 1, dtype=torch.int32, device=input.device)
+        ids = _zero_ids(input.device, M)
         ws = _workspace(input.device, ops.fused_experts_bf16_workspace_bytes(M, H, I, 1, 1))
         ops.fused_experts_w8a16(input.contiguous(), w13.unsqueeze(0), w13s.unsqueeze(0), w2.unsqueeze(0), w2s.unsqueeze(0), ids,
                                 None, out=output.view(M, 1, H), workspace=ws)
