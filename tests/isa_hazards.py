@@ -12,11 +12,13 @@ import re
 
 
 def _regs(tok):
+    """Vector registers named in an operand string: v0.. as 0.., accumulation registers a0.. as 1000.. ."""
     out = set()
-    for m in re.finditer(r"v\[(\d+):(\d+)\]", tok):
-        out |= set(range(int(m.group(1)), int(m.group(2)) + 1))
-    for m in re.finditer(r"(?<![\w\[:])v(\d+)\b", tok):
-        out.add(int(m.group(1)))
+    for file, base in (("v", 0), ("a", 1000)):
+        for m in re.finditer(r"(?<![\w])%s\[(\d+):(\d+)\]" % file, tok):
+            out |= set(range(base + int(m.group(1)), base + int(m.group(2)) + 1))
+        for m in re.finditer(r"(?<![\w\[:])%s(\d+)\b" % file, tok):
+            out.add(base + int(m.group(1)))
     return frozenset(out)
 
 
