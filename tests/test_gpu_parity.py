@@ -355,6 +355,42 @@ def test_fused_experts_with_shared_expert_and_empty_experts(pkg, oracle, dev, T,
     check_experts(pkg, oracle, dev, x, layer, ids, w, shared=shared)
 
 
+def random_case(seed):
+    """A layer shape, a batch size and a routing drawn from the seed: dimensions are multiples of 128 up to 1024, up to 48
+    experts, batches from one token to several row tiles of the largest expert, routing uniform or skewed towards a few
+    experts (so that one expert holds several row tiles while others stay empty), with or without a shared expert."""
+    r = random.Random(seed)
+    H, I = 128 * r.randint(1, 8), 128 * r.randint(1, 6)
+    E = r.choice([1, 2, 3, 5, 8, 16, 33, 48])
+    K = r.randint(1, min(E, 8))
+    T = r.choice([1, 2, 7, 15, 16, 17, 31, 33, 63, 64, 65, 100, 129, 257, 400, 650])
+    g = torch.Generator().manual_seed(seed)
+    skew = r.random() < 0.5
+    scores = torch.rand(T, E, generator=g)
+    if skew:                       # popularity falls off with the expert's rank; every fifth expert is never chosen
+        pop = 1.0 / torch.arange(1, E + 1).float() ** 1.2
+        dead = [e for e in range(E) if e % 5 == 4 and E - len(range(4, E, 5)) >= K]
+        scores = scores ** (1.0 / pop)
+        scores[:, dead] = -1.0
+    ids = torch.argsort(scores, dim=-1, descending=True)[:, :K].to(torch.int32).contiguous()
+    w = torch.rand(T, K, generator=g) + 0.1
+    w = (w / w.sum(-1, keepdim=True)).float()
+    I_sh = r.choice([0, 0, I, 128 * r.randint(1, 4)])
+    return T, H, I, E, K, ids, w, I_sh
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_fused_experts_random_shapes(pkg, oracle, dev, seed):
+    T, H, I, E, K, ids, w, I_sh = random_case(1000 + seed)
+    say("random shape", seed, (T, H, I, E, K), "shared", I_sh, "largest expert",
+        int(torch.bincount(ids.flatten().long(), minlength=E).max()))
+    assert all(len(set(row.tolist())) == K for row in ids)      # a token's experts are distinct
+    layer = oracle.make_layer(E, H, I, seed=seed)
+    shared = oracle.make_layer(1, H, I_sh, seed=seed + 77) if I_sh else None
+    x = torch.randn(T, H, generator=torch.Generator().manual_seed(seed)).to(torch.bfloat16)
+    check_experts(pkg, oracle, dev, x, layer, ids, w, shared=shared)
+
+
 def test_my_ops_drop_in_reference_layout(pkg, oracle, dev, checks):
     """The reference's call, argument for argument (python/regression/test_llm/test_moe.py:119-140):
     separate gate/up weights, pre-transposed down, bf16 scales, [T,K,H] output."""
