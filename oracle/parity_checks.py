@@ -32,6 +32,7 @@ RTOL, ATOL = 2e-2, 1e-2
 # of a row's I elements moves an output by a few atol at most; measured <= 0.2 % and <= 4.
 MAX_OUTSIDE = 5e-3
 MAX_WORST = 12.0
+MAX_COS_DIFF = 3e-5
 
 
 def outside_fraction(got: torch.Tensor, ref: torch.Tensor) -> float:
@@ -184,5 +185,7 @@ def check_sample(pkg, oracle, x_s, ids_s, layer_dev, w_s=None, shared_dev=None, 
         assert rep.get(k, 0.0) <= MAX_OUTSIDE, f"{what}: {k} = {rep[k]:.2e}"
     for k in ("worst_per_slot", "worst_reduced"):
         assert rep.get(k, 0.0) <= MAX_WORST, f"{what}: {k} = {rep[k]:.2f}"
-    assert rep["cos_diff"] < 1e-5, f"{what}: cos_diff {rep['cos_diff']:.2e}"
+    # the reference's own gate is 1e-4 (python/regression/test_llm/test_moe.py:308); measured 2e-6 to 4e-6 at full layer
+    # size and up to 1.0e-5 on a 50-row sample of a layer whose intermediate is 256 wide (fewer terms per output)
+    assert rep["cos_diff"] < MAX_COS_DIFF, f"{what}: cos_diff {rep['cos_diff']:.2e}"
     return rep

@@ -93,6 +93,34 @@ LAYER_CASES = [
 
 @pytest.mark.parametrize("T,H,I,E,K,mode,G,TG,with_bias,I_sh", LAYER_CASES)
 def test_layer_entry_point(pkg, oracle, dev, checks, T, H, I, E, K, mode, G, TG, with_bias, I_sh):
+    run_layer_case(pkg, oracle, dev, checks, T, H, I, E, K, mode, G, TG, with_bias, I_sh)
+
+
+def random_layer_case(seed):
+    """Layer shape, batch size and router drawn from the seed: batches either side of the decode size, grouped sigmoid
+    routing with at least two experts per group, or softmax."""
+    import random
+    r = random.Random(seed)
+    mode = r.choice(["softmax", "sigmoid", "sigmoid"])
+    G = r.choice([1, 1, 2, 4, 8]) if mode == "sigmoid" else 1
+    per = r.choice([2, 3, 4, 8, 16, 32])
+    E = min(256, G * per) if G > 1 else r.choice([2, 5, 8, 17, 64, 100, 256])
+    per = E // G
+    TG = r.randint(1, G)
+    K = r.randint(1, min(8, TG * per))
+    H, I = 128 * r.randint(1, 16), 128 * r.randint(1, 4)
+    T = r.choice([1, 2, 3, 9, 16, 31, 32, 33, 64, 65, 129, 300, 700])
+    I_sh = r.choice([0, I, 128 * r.randint(1, 3)])
+    with_bias = r.random() < 0.5 and mode == "sigmoid"     # a softmax router's bias has a test of its own below
+    return T, H, I, E, K, mode, G, TG, with_bias, I_sh
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_layer_entry_point_random_cases(pkg, oracle, dev, checks, seed):
+    run_layer_case(pkg, oracle, dev, checks, *random_layer_case(500 + seed))
+
+
+def run_layer_case(pkg, oracle, dev, checks, T, H, I, E, K, mode, G, TG, with_bias, I_sh):
     say("decode layer", T, H, I, E, K, mode, G, TG, with_bias, I_sh)
     small = 3 * E * H * I <= (1 << 26)
     if small:
