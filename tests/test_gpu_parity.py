@@ -792,3 +792,59 @@ def test_my_ops_ragged_block_edges(pkg, oracle, dev, T, H, I, E, K):
     assert oracle.cal_diff(ref, got16)[0] < 1e-4
     want = torch.einsum("tk,tkh->th", w.to(torch.bfloat16).float(), got16)
     assert ((out_w.float().cpu() - want).abs() <= 2e-2 * want.abs() + 2e-2 * want.pow(2).mean().sqrt()).all()
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_my_ops_random_shapes_both_arithmetics(pkg, oracle, dev, seed):
+    """The registered op in the reference's argument layout (python/regression/test_llm/test_moe.py:285-295) on shapes
+    drawn from the seed - hidden and intermediate sizes that 128 may or may not divide, one to 64 experts, batches up to
+    a few row tiles - through both entry names, against the reference's CPU ground truth (test_moe.py:10-98): the
+    reference's own arithmetic within its full criterion (cos_sim > 0.99 and cos_diff < 1e-4, test_moe.py:308), the FP8
+    activation path within cos_sim > 0.99, and the [T, H] output form equal to the weighted sum of the [T, K, H] one."""
+    r = random.Random(2000 + seed)
+    H = r.choice([128 * r.randint(1, 8), 8 * r.randint(9, 120)])
+    I = r.choice([128 * r.randint(1, 4), 8 * r.randint(3, 60)])
+    E = r.choice([1, 2, 4, 7, 16, 64])
+    K = r.randint(1, min(E, 8))
+    T = r.choice([1, 3, 8, 17, 40, 96, 200, 330])
+    say("my_ops random", seed, (T, H, I, E, K))
+    g = torch.Generator().manual_seed(seed)
+    nb = lambda n: (n + 127) // 128
+    w0, w1 = ((torch.randn(E, I, H, generator=g) * 0.1).to(torch.float8_e4m3fn) for _ in range(2))
+    w2 = (torch.randn(E, H, I, generator=g) * 0.1).to(torch.float8_e4m3fn)
+    s0, s1 = ((torch.rand(E, nb(I), nb(H), generator=g) * 0.2 + 0.02).to(torch.bfloat16) for _ in range(2))
+    s2 = (torch.rand(E, nb(H), nb(I), generator=g) * 0.2 + 0.02).to(torch.bfloat16)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    ids, w = distinct_ids(T, E, K, seed=seed + 3)
+    ref = oracle.experts_ref_bf16(x, ids, w0, w1, w2, s0, s1, s2).float()
+    wb = w.to(torch.bfloat16)
+    args = [x.to(dev), None, None, w0.to(dev), w1.to(dev), w2.transpose(1, 2).contiguous().to(dev),
+            s0.to(dev), s1.to(dev), s2.transpose(1, 2).contiguous().to(dev), ids.to(dev), wb.to(dev), None,
+            None, None]
+    tail = [128, E, K, False, 1, 1, None, None, None, False]
+    scratch = [torch.zeros(E, T, dtype=torch.int32, device=dev), torch.zeros(E, T, K, dtype=torch.int32, device=dev)]
+    results = {}
+    for mode in ("w8a8", "w8a16"):
+        pkg.set_expert_numerics(mode)
+        try:
+            out = torch.full((T, K, H), float("nan"), dtype=torch.bfloat16, device=dev)
+            torch.ops.my_ops.fused_moe_fused_experts(out, *args, *tail)
+            out_v2 = torch.full((T, K, H), float("nan"), dtype=torch.bfloat16, device=dev)
+            torch.ops.my_ops.fused_moe_fused_experts_v2(out_v2, *args, *scratch, *tail)
+            out_w = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device=dev)
+            torch.ops.my_ops.fused_moe_fused_experts(out_w, *args, *tail)
+            torch.cuda.synchronize()
+        finally:
+            pkg.set_expert_numerics("w8a8")
+        assert torch.equal(out.view(torch.int16), out_v2.view(torch.int16)), mode
+        got = out.float().cpu()
+        assert torch.isfinite(got).all(), mode
+        assert oracle.cos_sim(ref.numpy(), got.numpy()) > 0.99, mode
+        cd = oracle.cal_diff(ref, got)[0]
+        say(f"    {mode}: cos_diff {cd:.2e}")
+        assert cd < (1e-4 if mode == "w8a16" else 5e-3), (mode, cd)
+        # the [T, H] form: the fp32 weighted sum of the slot results (bf16 routing weights widened), rounded once
+        want = torch.einsum("tk,tkh->th", wb.float(), got).to(torch.bfloat16).float()
+        gw = out_w.float().cpu()
+        assert ((gw - want).abs() <= 1e-2 * want.abs() + 1e-6).all(), mode
+        results[mode] = got
