@@ -72,7 +72,7 @@ def test_mlp_w8a16_dq_forward(pkg, oracle, dev, M, H, I):
 
 
 @pytest.mark.parametrize("block", [64, 256])
-@pytest.mark.parametrize("M,K,N", [(32, 2048, 512), (16, 2048, 512), (200, 1024, 272)])
+@pytest.mark.parametrize("M,K,N", [(32, 2048, 512), (16, 2048, 512), (200, 1024, 272), (40, 1000, 100), (3, 72, 7)])
 def test_mm_block_sizes(pkg, oracle, dev, M, K, N, block):
     """The reference's block-size grid (python/regression/test_llm/test_deepseek_mm.py:225-248: 64, 128, 256 on
     32 x 2048 -> 512).  256: the FP8 kernels on scales expanded to 128-blocks; 64: the reference's bf16 arithmetic."""
@@ -188,4 +188,88 @@ def test_mlp_in_the_references_own_arithmetic(pkg, oracle, dev, M, H, I):
     assert torch.isfinite(got).all()
     ref = oracle.mlp_w8a16_dq_ref(x, wg, wu, wd, sg, su, sd).float()
     assert oracle.cos_sim(ref.flatten(), got.flatten()) >= 0.99
+    assert oracle.cal_diff(ref, got)[0] < 1e-4
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_mm_random_shapes_both_arithmetics(pkg, oracle, dev, seed):
+    """mm_w8a16_dq_forward on shapes drawn from the seed: row counts either side of the 128 rows up to which the
+    per-wavefront kernel runs, output widths of any size, reductions of 1 to 56 blocks or with a partial last block; FP8
+    activations strict against the fp32 product of the same quantised operands, the reference's own arithmetic against
+    its bf16 ground truth at its criterion (python/regression/test_llm/test_mm_w8a16_dq.py:52-60)."""
+    import random
+    r = random.Random(4000 + seed)
+    M = r.choice([1, 2, 7, 16, 31, 64, 127, 128, 129, 200, 333])
+    K = r.choice([128 * r.choice([1, 2, 3, 8, 16, 33, 56]), 128 * r.choice([1, 2, 3, 8, 16, 33, 56]), 8 * r.randint(1, 150)])
+    N = r.choice([16 * r.randint(1, 40), 128 * r.randint(1, 24), 8 * r.randint(2, 90), r.randint(1, 300)])
+    say("mm random", seed, M, K, N)
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = torch.randn(N, K, generator=g).to(torch.float8_e4m3fn)
+    s = (torch.rand((N + 127) // 128, (K + 127) // 128, generator=g) + 0.1).to(torch.bfloat16)
+    xd, wd, sd = x.to(dev), w.to(dev), s.to(dev)
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+    torch.ops.my_ops.mm_w8a16_dq_forward(xd, wd, sd, out, 128)
+    torch.cuda.synchronize()
+    got = out.float().cpu()
+    assert torch.isfinite(got).all()
+    assert normalised_outside(got, oracle.mm_w8a8_fp32(x, w, s.float())) == 0.0
+    out16 = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+    pkg.set_expert_numerics("w8a16")
+    try:
+        torch.ops.my_ops.mm_w8a16_dq_forward(xd, wd, sd, out16, 128)
+        torch.cuda.synchronize()
+    finally:
+        pkg.set_expert_numerics("w8a8")
+    got16 = out16.float().cpu()
+    ref = oracle.mm_w8a16_dq_ref(x, w, s).float()
+    assert torch.isfinite(got16).all()
+    assert oracle.cos_sim(ref.flatten(), got16.flatten()) >= 0.99
+    assert oracle.cal_diff(ref, got16)[0] < 1e-4
+    rms = ref.pow(2).mean().sqrt()
+    assert ((got16 - ref).abs() <= 1.6e-2 * ref.abs() + 1e-2 * rms).all()
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_mlp_random_shapes_both_arithmetics(pkg, oracle, dev, seed):
+    """mlp_w8a16_dq_forward on shapes drawn from the seed, hidden and intermediate sizes that 128 may not divide
+    (torch_tpu/csrc/ops/my_ops/MlpW8A16Dq.pl:11-34 takes ceil(n/128) blocks): the reference's own arithmetic against its
+    ground truth at its criterion (python/regression/test_llm/test_mlp_w8a16_dq.py:53-81), the FP8 activation path
+    against the fp32 computation on the same quantised operands."""
+    import random
+    r = random.Random(5000 + seed)
+    M = r.choice([1, 5, 16, 33, 64, 127, 129, 250])
+    H = r.choice([128 * r.randint(1, 16), 8 * r.randint(4, 150)])
+    I = r.choice([128 * r.randint(1, 8), 8 * r.randint(4, 100)])
+    say("mlp random", seed, M, H, I)
+    g = torch.Generator().manual_seed(seed)
+    nb = lambda n: (n + 127) // 128
+    x = torch.randn(M, H, generator=g).to(torch.bfloat16)
+    wg, wu = (torch.randn(I, H, generator=g).to(torch.float8_e4m3fn) for _ in range(2))
+    wd = torch.randn(H, I, generator=g).to(torch.float8_e4m3fn)
+    sg, su = ((torch.rand(nb(I), nb(H), generator=g) * 0.05 + 0.005).to(torch.bfloat16) for _ in range(2))
+    sd = (torch.rand(nb(H), nb(I), generator=g) * 0.05 + 0.005).to(torch.bfloat16)
+    args = (x.to(dev), wg.to(dev), wu.to(dev), wd.T.to(dev), sg.to(dev), su.to(dev), sd.T.to(dev))
+    out = torch.full((M, H), float("nan"), dtype=torch.bfloat16, device=dev)
+    torch.ops.my_ops.mlp_w8a16_dq_forward(*args, out, 128)
+    out16 = torch.full((M, H), float("nan"), dtype=torch.bfloat16, device=dev)
+    pkg.set_expert_numerics("w8a16")
+    try:
+        torch.ops.my_ops.mlp_w8a16_dq_forward(*args, out16, 128)
+        torch.cuda.synchronize()
+    finally:
+        pkg.set_expert_numerics("w8a8")
+    got, got16 = out.float().cpu(), out16.float().cpu()
+    assert torch.isfinite(got).all() and torch.isfinite(got16).all()
+    truth = oracle.mlp_w8a16_dq_ref(x, wg, wu, wd, sg, su, sd).float()
+    assert oracle.cos_sim(truth.flatten(), got16.flatten()) >= 0.99
+    assert oracle.cal_diff(truth, got16)[0] < 1e-4
+    assert oracle.cos_sim(truth.flatten(), got.flatten()) >= 0.99
+    # the FP8 path against fp32 arithmetic on the same quantised operands, ragged sizes padded with zeros as the device does
+    Hp, Ip = nb(H) * 128, nb(I) * 128
+    pad = lambda t, rows, cols: torch.nn.functional.pad(t.view(torch.uint8), (0, cols - t.shape[1], 0, rows - t.shape[0])).view(t.dtype)
+    w13q = torch.cat([pad(wg, Ip, Hp), pad(wu, Ip, Hp)], 0)
+    ref = oracle.mlp_w8a8_fp32(torch.nn.functional.pad(x, (0, Hp - H)), w13q, torch.cat([sg, su], 0).float(),
+                               pad(wd, Hp, Ip), sd.float())[:, :H]
+    assert normalised_outside(got, ref) <= MAX_OUTSIDE
     assert oracle.cal_diff(ref, got)[0] < 1e-4

@@ -12,7 +12,7 @@ import weakref
 import torch
 
 from . import ops
-from .layer import pack_expert_weights
+from .layer import _pad_to, pack_expert_weights
 
 _lib = torch.library.Library("my_ops", "DEF")
 
@@ -335,36 +335,49 @@ def _mlp_w8a16_dq_forward(input, gate_weight, up_weight, down_weight, gate_scale
     reference's own bf16 arithmetic on weights de-quantised once."""
     _check_dense(blocksize, gate_weight, up_weight, down_weight)
     I, H = gate_weight.shape
+    # I or H that 128 does not divide (the reference de-quantises ceil(n/128) blocks, the last one partial:
+    # torch_tpu/csrc/ops/my_ops/MlpW8A16Dq.pl:11-34): the packed weights are padded to whole blocks with zeros, the
+    # input's columns likewise, and the padded output's first H columns are the result
+    Ip, Hp = -(-I // 128) * 128, -(-H // 128) * 128
+    M = input.shape[0]
+    x = input.contiguous() if Hp == H else torch.nn.functional.pad(input, (0, Hp - H))
+    out = output if Hp == H and output.is_contiguous() else torch.empty(M, Hp, dtype=output.dtype, device=output.device)
+
+    def done():
+        if out is not output:
+            output.copy_(out[:, :H])
+        return output
+
     if blocksize % 128:
         w13, w2 = _dense_packed(
             (gate_weight, up_weight, down_weight, gate_scale, up_scale, down_scale),
-            lambda: (ops.pack_weights(torch.cat([_dequant_any(gate_weight, gate_scale, blocksize),
-                                                 _dequant_any(up_weight, up_scale, blocksize)], 0).unsqueeze(0).contiguous()),
-                     ops.pack_weights(_dequant_any(down_weight, down_scale, blocksize).t().unsqueeze(0).contiguous())),
+            lambda: (ops.pack_weights(torch.cat([_pad_to(_dequant_any(gate_weight, gate_scale, blocksize), Ip, Hp),
+                                                 _pad_to(_dequant_any(up_weight, up_scale, blocksize), Ip, Hp)], 0)
+                                      .unsqueeze(0).contiguous()),
+                     ops.pack_weights(_pad_to(_dequant_any(down_weight, down_scale, blocksize), Ip, Hp).t().unsqueeze(0)
+                                      .contiguous())),
             f"mlp-dequant{blocksize}")
         # one expert that every row selects; its per-slot result [M, 1, H] is the output itself
-        M = input.shape[0]
-        ws = _workspace(input.device, ops.fused_experts_bf16_workspace_bytes(M, H, I, 1, 1))
-        ops.fused_experts_bf16(input.contiguous(), w13, w2, _zero_ids(input.device, M), None, out=output.view(M, 1, H),
-                               workspace=ws)
-        return output
+        ws = _workspace(input.device, ops.fused_experts_bf16_workspace_bytes(M, Hp, Ip, 1, 1))
+        ops.fused_experts_bf16(x, w13, w2, _zero_ids(input.device, M), None, out=out.view(M, 1, Hp), workspace=ws)
+        return done()
     w13, w13s, w2, w2s = _dense_packed(
         (gate_weight, up_weight, down_weight, gate_scale, up_scale, down_scale),
-        lambda: (ops.pack_weights(torch.cat([gate_weight, up_weight], 0).contiguous()),
+        lambda: (ops.pack_weights(torch.cat([_pad_to(gate_weight, Ip, Hp), _pad_to(up_weight, Ip, Hp)], 0).contiguous()),
                  torch.cat([_scales_128(gate_scale, blocksize, I, H), _scales_128(up_scale, blocksize, I, H)], 0).contiguous(),
-                 ops.pack_weights(down_weight.t().contiguous()), _scales_128(down_scale, blocksize, I, H).t().contiguous()),
+                 ops.pack_weights(_pad_to(down_weight, Ip, Hp).t().contiguous()),
+                 _scales_128(down_scale, blocksize, I, H).t().contiguous()),
         f"mlp{blocksize}")
-    if _numerics == "w8a16" and H <= 16384 and I <= 16384:
+    if _numerics == "w8a16" and Hp <= 16384 and Ip <= 16384:
         # the reference's own arithmetic: one expert that every row selects, weights de-quantised in registers
-        M = input.shape[0]
         ids = _zero_ids(input.device, M)
-        ws = _workspace(input.device, ops.fused_experts_bf16_workspace_bytes(M, H, I, 1, 1))
-        ops.fused_experts_w8a16(input.contiguous(), w13.unsqueeze(0), w13s.unsqueeze(0), w2.unsqueeze(0), w2s.unsqueeze(0), ids,
-                                None, out=output.view(M, 1, H), workspace=ws)
-        return output
-    ws = _workspace(input.device, ops.mlp_workspace_bytes(input.shape[0], H, I))
-    ops.mlp_fp8(input.contiguous(), w13, w13s, w2, w2s, out=output, workspace=ws)
-    return output
+        ws = _workspace(input.device, ops.fused_experts_bf16_workspace_bytes(M, Hp, Ip, 1, 1))
+        ops.fused_experts_w8a16(x, w13.unsqueeze(0), w13s.unsqueeze(0), w2.unsqueeze(0), w2s.unsqueeze(0), ids,
+                                None, out=out.view(M, 1, Hp), workspace=ws)
+        return done()
+    ws = _workspace(input.device, ops.mlp_workspace_bytes(M, Hp, Ip))
+    ops.mlp_fp8(x, w13, w13s, w2, w2s, out=out, workspace=ws)
+    return done()
 
 
 def _mm_w8a16_dq_forward(input, weight, scale, output, blocksize):
@@ -372,18 +385,32 @@ def _mm_w8a16_dq_forward(input, weight, scale, output, blocksize):
     Block sizes as in mlp_w8a16_dq_forward."""
     _check_dense(blocksize, weight)
     N, K = weight.shape
+    # N that 16 does not divide, K that 128 does not divide: zero rows / zero columns up to the next multiple in the
+    # packed weight (the reference's blocks at the edges are partial, torch_tpu/csrc/ops/my_ops/MlpW8A16Dq.pl:11-34),
+    # zero columns in the input, and the padded output's first N columns are the result
+    Np, Kp = -(-N // 16) * 16, -(-K // 128) * 128
+    M = input.shape[0]
+    x = input.contiguous() if Kp == K else torch.nn.functional.pad(input, (0, Kp - K))
+    out = output if Np == N and output.is_contiguous() else torch.empty(M, Np, dtype=output.dtype, device=output.device)
+
+    def done():
+        if out is not output:
+            output.copy_(out[:, :N])
+        return output
+
     if blocksize % 128:
-        (w,) = _dense_packed((weight, scale), lambda: (ops.pack_weights(_dequant_any(weight, scale, blocksize)),),
+        (w,) = _dense_packed((weight, scale),
+                             lambda: (ops.pack_weights(_pad_to(_dequant_any(weight, scale, blocksize), Np, Kp).contiguous()),),
                              f"mm-dequant{blocksize}")
-        ops.mm_bf16(input.contiguous(), w, out=output)
-        return output
-    w, ws = _dense_packed((weight, scale), lambda: (ops.pack_weights(weight.contiguous()),
+        ops.mm_bf16(x, w, out=out)
+        return done()
+    w, ws = _dense_packed((weight, scale), lambda: (ops.pack_weights(_pad_to(weight, Np, Kp).contiguous()),
                                                      _scales_128(scale, blocksize, N, K)), f"mm{blocksize}")
-    if _numerics == "w8a16" and K <= 16384:
-        ops.mm_w8a16(input.contiguous(), w, ws, out=output)
-        return output
-    ops.mm_fp8(input.contiguous(), w, ws, out=output, workspace=_workspace(input.device, ops.mm_workspace_bytes(input.shape[0], K, N)))
-    return output
+    if _numerics == "w8a16" and Kp <= 16384:
+        ops.mm_w8a16(x, w, ws, out=out)
+        return done()
+    ops.mm_fp8(x, w, ws, out=out, workspace=_workspace(input.device, ops.mm_workspace_bytes(M, Kp, Np)))
+    return done()
 
 
 _lib.impl("fused_moe_fused_experts", _fused_experts, "CompositeExplicitAutograd")
