@@ -189,11 +189,11 @@ def _fused_experts(output, input, output_sample, input_sample, gate_weights, up_
             if t.dtype != torch.bfloat16:
                 raise RuntimeError("weights without scales must be bfloat16")
         w13, w2 = _dense_packed((gate_weights, up_weights, down_weights),
-                                lambda: (ops.pack_weights(torch.cat([gate_weights, up_weights], dim=1).contiguous()),
-                                         ops.pack_weights(down_weights.transpose(1, 2).contiguous())), "bf16")
+                                lambda: _pack_bf16(gate_weights, up_weights, down_weights), "bf16")
         if w13.shape[0] != num_experts or select_experts.shape[1] != num_experts_per_tok:
             raise RuntimeError("num_experts / num_experts_per_tok do not match the tensors")
-        return _run_bf16(output, input, w13, w2, select_experts, routing_weights)
+        return _padded_io(output, input, w13.shape[2],
+                          lambda o, x: _run_bf16(o, x, w13, w2, select_experts, routing_weights))
     if gate_scales is None or up_scales is None or down_scales is None:
         raise RuntimeError("either all three weight tensors carry block scales or none does")
     if blocksize < 1:
@@ -203,11 +203,12 @@ def _fused_experts(output, input, output_sample, input_sample, gate_weights, up_
     if blocksize % 128:
         w13, w2 = _dense_packed(
             (gate_weights, up_weights, down_weights, gate_scales, up_scales, down_scales),
-            lambda: (ops.pack_weights(torch.cat([_dequant_bf16(gate_weights, gate_scales, blocksize),
-                                                 _dequant_bf16(up_weights, up_scales, blocksize)], 1).contiguous()),
-                     ops.pack_weights(_dequant_bf16(down_weights, down_scales, blocksize).transpose(1, 2).contiguous())),
+            lambda: _pack_bf16(_dequant_bf16(gate_weights, gate_scales, blocksize),
+                               _dequant_bf16(up_weights, up_scales, blocksize),
+                               _dequant_bf16(down_weights, down_scales, blocksize)),
             f"dequant{blocksize}")
-        return _run_bf16(output, input, w13, w2, select_experts, routing_weights)
+        return _padded_io(output, input, w13.shape[2],
+                          lambda o, x: _run_bf16(o, x, w13, w2, select_experts, routing_weights))
     if blocksize != 128:
         # a multiple of 128: every 128-block takes the scale of the block it lies in (the same products, exactly)
         I, H = gate_weights.shape[1:]
@@ -220,21 +221,29 @@ def _fused_experts(output, input, output_sample, input_sample, gate_weights, up_
         w13, w13s, w2, w2s = _packed(gate_weights, up_weights, down_weights, gate_scales, up_scales, down_scales)
     if w13.shape[0] != num_experts or select_experts.shape[1] != num_experts_per_tok:
         raise RuntimeError("num_experts / num_experts_per_tok do not match the tensors")
-    T, H = input.shape
-    E, I2, Hp = w13.shape
     rw = _routing_f32(routing_weights, input.device) if output.dim() == 2 else None
-    real_output = None
-    if Hp != H:
-        # ragged hidden size: the packed weights were padded to whole 128-blocks with zeros; the activations get
-        # zero columns to match (they change no group's maximum and add nothing to any sum) and the result's
-        # padding columns are dropped
-        input = torch.nn.functional.pad(input, (0, Hp - H))
-        real_output, output = output, torch.empty(*output.shape[:-1], Hp, dtype=output.dtype, device=output.device)
-        H = Hp
-    output = _run_packed(output, input, w13, w13s, w2, w2s, select_experts, rw)
-    if real_output is not None:
-        real_output.copy_(output[..., :real_output.shape[-1]])
-        return real_output
+    return _padded_io(output, input, w13.shape[2], lambda o, x: _run_packed(o, x, w13, w13s, w2, w2s, select_experts, rw))
+
+
+def _pack_bf16(gate, up, down_t):
+    """bf16 weights in the reference's argument layout (gate, up and transposed down, all [E, I, H]) -> (w13, w2)
+    tile-blocked, I and H zero-padded to whole 128-blocks like the FP8 weights (layer.stack_expert_weights)."""
+    I, H = gate.shape[-2:]
+    Ip, Hp = -(-I // 128) * 128, -(-H // 128) * 128
+    return (ops.pack_weights(torch.cat([_pad_to(gate, Ip, Hp), _pad_to(up, Ip, Hp)], dim=1).contiguous()),
+            ops.pack_weights(_pad_to(down_t, Ip, Hp).transpose(1, 2).contiguous()))
+
+
+def _padded_io(output, input, Hp, run):
+    """Runs `run(output, input)` on a hidden size padded to Hp.  A ragged hidden size (the packed weights were padded to
+    whole 128-blocks with zeros): the activations get zero columns to match - they change no group's maximum and add
+    nothing to any sum - and the result's padding columns are dropped."""
+    H = input.shape[1]
+    if Hp == H:
+        return run(output, input)
+    padded = torch.empty(*output.shape[:-1], Hp, dtype=output.dtype, device=output.device)
+    run(padded, torch.nn.functional.pad(input, (0, Hp - H)))
+    output.copy_(padded[..., :H])
     return output
 
 
