@@ -187,6 +187,50 @@ def test_route_sigmoid_grouped(pkg, oracle, dev, T, E, K, G, TG, with_bias):
     assert torch.equal(ids3.cpu(), i_ref) and torch.allclose(w3.cpu(), w_ref, rtol=1e-5, atol=1e-7)
 
 
+@pytest.mark.parametrize("seed", range(30))
+def test_routing_random_cases(pkg, oracle, dev, seed):
+    """noaux_tc_topk and moe_route on group structures, expert counts, batch sizes (either side of the small-batch
+    kernel) and dtypes drawn from the seed, half of them with many exact ties: ids bit-exact against the oracle (lowest
+    index wins a tie), values and weights as the oracle's."""
+    r = random.Random(3000 + seed)
+    G = r.choice([1, 1, 2, 3, 4, 8, 16])
+    per = r.choice([2, 3, 4, 7, 16, 32, 64])
+    E = G * per if G > 1 else r.choice([2, 3, 8, 17, 64, 100, 256, 1024])
+    while E > 1024:
+        per //= 2
+        E = G * per
+    per = E // G
+    TG = r.randint(1, G)
+    K = r.randint(1, min(32, TG * per))
+    T = r.choice([1, 2, 7, 33, 64, 65, 150, 1000])
+    dtype = r.choice([torch.float32, torch.bfloat16])
+    say("routing random", seed, (T, E, G, TG, K), dtype)
+    g = torch.Generator().manual_seed(seed)
+    scores = torch.randn(T, E, generator=g)
+    if seed % 2:
+        scores = torch.round(scores * 2) / 2
+    scores = scores.to(dtype)
+    v_ref, i_ref = oracle.noaux_tc_topk(scores, G, TG, K)
+    values = torch.empty(T, K, dtype=dtype, device=dev)
+    indices = torch.empty(T, K, dtype=torch.int32, device=dev)
+    pkg.noaux_tc_topk(values, indices, scores.to(dev), G, TG, K)
+    torch.cuda.synchronize()
+    assert torch.equal(indices.cpu(), i_ref) and torch.equal(values.cpu(), v_ref)
+    # the router recipe on the same numbers as logits
+    bias = (torch.randn(E, generator=g) * 0.1) if r.random() < 0.5 else None
+    bd = None if bias is None else bias.to(dev)
+    w, ids, sc = pkg.moe_route(scores.to(dev), K, "sigmoid", bias=bd, n_groups=G, topk_groups=TG, renorm=True, scale=2.5,
+                               return_scores=True)
+    torch.cuda.synchronize()
+    w_ref, ids_ref = oracle.select_sigmoid_grouped(sc.cpu(), bias, K, G, TG, 2.5, True)
+    assert torch.equal(ids.cpu(), ids_ref)
+    assert torch.allclose(w.cpu(), w_ref, rtol=1e-5, atol=1e-7)
+    ws, ids_s = pkg.moe_route(scores.to(dev), K, "softmax", renorm=bool(seed % 3))
+    ws_ref, ids_s_ref = oracle.route_softmax_topk(scores, K, renorm=bool(seed % 3))
+    assert torch.equal(ids_s.cpu(), ids_s_ref)
+    assert torch.allclose(ws.cpu(), ws_ref, rtol=1e-5, atol=1e-7)
+
+
 # ----------------------------------------------------------------------------- permutation
 def check_permutation(pkg, oracle, dev, sel, E):
     ss_ref, off_ref, s2r_ref = oracle.permute_counting_sort(sel, E)
