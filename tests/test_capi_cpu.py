@@ -117,6 +117,7 @@ def test_my_ops_are_registered_with_reference_arity(pkg):
     assert len(ops.fused_moe_grouped_topk.default._schema.arguments) == 10
     assert len(ops.mlp_w8a16_dq_forward.default._schema.arguments) == 9     # ops.hpp:279-288
     assert len(ops.mm_w8a16_dq_forward.default._schema.arguments) == 5      # ops.hpp:290-295
+    assert len(ops.mlp_w8a8_quant_forward.default._schema.arguments) == 9   # ops.hpp:297-306
     assert len(ops.moe_route.default._schema.arguments) == 9
     assert len(ops.moe_permute.default._schema.arguments) == 2
     assert len(ops.moe_pack_weights.default._schema.arguments) == 6

@@ -273,3 +273,44 @@ def test_mlp_random_shapes_both_arithmetics(pkg, oracle, dev, seed):
                                pad(wd, Hp, Ip), sd.float())[:, :H]
     assert normalised_outside(got, ref) <= MAX_OUTSIDE
     assert oracle.cal_diff(ref, got)[0] < 1e-4
+
+
+@pytest.mark.parametrize("M,H,I", [(32, 7168, 256), (200, 512, 384), (5, 328, 200)])
+def test_mlp_w8a8_quant_forward(pkg, oracle, dev, M, H, I):
+    """mlp_w8a8_quant_forward (torch_tpu/csrc/ops/my_ops/MlpW8A8Quant.cpp:12-52): the FP8-activation arithmetic whatever
+    the numerics switch says, the down projection in either orientation (the W8A16 op's transposed one, or [H, I] as
+    python/test/deepseek_mlp_quant.py:167-177 builds it), against fp32 arithmetic on the same quantised operands.  The
+    reference pins nothing for this op (closed implementation, no test, no CPU function): the comparison is with this
+    package's own definition of the activation quantisation."""
+    say("mlp w8a8", M, H, I)
+    g = torch.Generator().manual_seed(6000 + M + I)
+    nb = lambda n: (n + 127) // 128
+    x = torch.randn(M, H, generator=g).to(torch.bfloat16)
+    wg, wu = (torch.randn(I, H, generator=g).to(torch.float8_e4m3fn) for _ in range(2))
+    wd = torch.randn(H, I, generator=g).to(torch.float8_e4m3fn)
+    sg, su = ((torch.rand(nb(I), nb(H), generator=g) * 0.05 + 0.005).to(torch.bfloat16) for _ in range(2))
+    sd = (torch.rand(nb(H), nb(I), generator=g) * 0.05 + 0.005).to(torch.bfloat16)
+    xd, wgd, wud, wdd, sgd, sud, sdd = (t.to(dev) for t in (x, wg, wu, wd, sg, su, sd))
+    wdt, sdt = wdd.T.contiguous(), sdd.T.contiguous()
+    base = torch.full((M, H), float("nan"), dtype=torch.bfloat16, device=dev)
+    torch.ops.my_ops.mlp_w8a16_dq_forward(xd, wgd, wud, wdt, sgd, sud, sdt, base, 128)       # default numerics: FP8 activations
+    outs = []
+    pkg.set_expert_numerics("w8a16")
+    try:
+        for down, scale in ((wdt, sdt), (wdd, sdd)):
+            out = torch.full((M, H), float("nan"), dtype=torch.bfloat16, device=dev)
+            r = torch.ops.my_ops.mlp_w8a8_quant_forward(xd, wgd, wud, down, sgd, sud, scale, out, 128)
+            assert r.data_ptr() == out.data_ptr()
+            outs.append(out)
+        torch.cuda.synchronize()
+    finally:
+        pkg.set_expert_numerics("w8a8")
+    for out in outs:
+        assert torch.equal(out.view(torch.int16), base.view(torch.int16))
+    got = base.float().cpu()
+    Hp, Ip = nb(H) * 128, nb(I) * 128
+    pad = lambda t, rows, cols: torch.nn.functional.pad(t.view(torch.uint8), (0, cols - t.shape[1], 0, rows - t.shape[0])).view(t.dtype)
+    ref = oracle.mlp_w8a8_fp32(torch.nn.functional.pad(x, (0, Hp - H)), torch.cat([pad(wg, Ip, Hp), pad(wu, Ip, Hp)], 0),
+                               torch.cat([sg, su], 0).float(), pad(wd, Hp, Ip), sd.float())[:, :H]
+    assert normalised_outside(got, ref) <= MAX_OUTSIDE
+    assert oracle.cal_diff(ref, got)[0] < 1e-4

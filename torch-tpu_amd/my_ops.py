@@ -47,6 +47,8 @@ _lib.define("mlp_w8a16_dq_forward(Tensor input, Tensor gate_weight, Tensor up_we
             "Tensor gate_scale, Tensor up_scale, Tensor down_scale, Tensor(a!) output, int blocksize) -> Tensor(a!)")
 _lib.define("mm_w8a16_dq_forward(Tensor input, Tensor weight, Tensor scale, Tensor(a!) output, int blocksize) "
             "-> Tensor(a!)")
+_lib.define("mlp_w8a8_quant_forward(Tensor input, Tensor gate_weight, Tensor up_weight, Tensor down_weight, "
+            "Tensor gate_scale, Tensor up_scale, Tensor down_scale, Tensor(a!) output, int blocksize) -> Tensor(a!)")
 
 # How quantised expert weights are multiplied.  "w8a8" (default): activations are quantised to FP8 per
 # token and 128 columns and the products run on the FP8 matrix path - the path this package is about.
@@ -342,8 +344,33 @@ def _mlp_w8a16_dq_forward(input, gate_weight, up_weight, down_weight, gate_scale
     [I,H] (python/regression/test_llm/test_mlp_w8a16_dq.py:106-109), scales likewise; output [M,H].
     Block sizes that are multiples of 128 run the FP8 kernels on the expanded scales; others run the
     reference's own bf16 arithmetic on weights de-quantised once."""
+    return _mlp_forward(input, gate_weight, up_weight, down_weight, gate_scale, up_scale, down_scale, output, blocksize,
+                        _numerics, True)
+
+
+def _mlp_w8a8_quant_forward(input, gate_weight, up_weight, down_weight, gate_scale, up_scale, down_scale, output,
+                            blocksize):
+    """torch_tpu/csrc/ops/my_ops/MlpW8A8Quant.cpp:12-52: the dense gated MLP with quantised activations, same
+    arguments as mlp_w8a16_dq_forward.  Always the FP8-activation arithmetic of this package (per-token scales over
+    128 columns), whatever set_expert_numerics says.  The reference's implementation is closed and it holds neither a
+    test nor a CPU ground truth for this op, so its activation-quantisation numerics are not pinned by anything: what is
+    checked is this package's own definition.  The one script that builds arguments for an op of this kind
+    (python/test/deepseek_mlp_quant.py:167-177) hands the down projection over as [H, I] with [H/bs, I/bs] scales; that
+    orientation is taken as well as the transposed one of the W8A16 op (told apart by shape; a square layer is read the
+    W8A16 way)."""
+    I, H = gate_weight.shape
+    down_t = not (I != H and tuple(down_weight.shape) == (H, I))
+    return _mlp_forward(input, gate_weight, up_weight, down_weight, gate_scale, up_scale, down_scale, output, blocksize,
+                        "w8a8", down_t)
+
+
+def _mlp_forward(input, gate_weight, up_weight, down_weight, gate_scale, up_scale, down_scale, output, blocksize,
+                 numerics, down_t):
+    """down_t: down_weight and down_scale are given transposed ([I, H] / [I/bs, H/bs])."""
     _check_dense(blocksize, gate_weight, up_weight, down_weight)
     I, H = gate_weight.shape
+    orient = "t" if down_t else "n"
+    as_t = (lambda t: t) if down_t else (lambda t: t.t())        # to the transposed form the packing below expects
     # I or H that 128 does not divide (the reference de-quantises ceil(n/128) blocks, the last one partial:
     # torch_tpu/csrc/ops/my_ops/MlpW8A16Dq.pl:11-34): the packed weights are padded to whole blocks with zeros, the
     # input's columns likewise, and the padded output's first H columns are the result
@@ -363,9 +390,9 @@ def _mlp_w8a16_dq_forward(input, gate_weight, up_weight, down_weight, gate_scale
             lambda: (ops.pack_weights(torch.cat([_pad_to(_dequant_any(gate_weight, gate_scale, blocksize), Ip, Hp),
                                                  _pad_to(_dequant_any(up_weight, up_scale, blocksize), Ip, Hp)], 0)
                                       .unsqueeze(0).contiguous()),
-                     ops.pack_weights(_pad_to(_dequant_any(down_weight, down_scale, blocksize), Ip, Hp).t().unsqueeze(0)
-                                      .contiguous())),
-            f"mlp-dequant{blocksize}")
+                     ops.pack_weights(_pad_to(_dequant_any(as_t(down_weight), as_t(down_scale), blocksize), Ip, Hp).t()
+                                      .unsqueeze(0).contiguous())),
+            f"mlp-dequant{blocksize}{orient}")
         # one expert that every row selects; its per-slot result [M, 1, H] is the output itself
         ws = _workspace(input.device, ops.fused_experts_bf16_workspace_bytes(M, Hp, Ip, 1, 1))
         ops.fused_experts_bf16(x, w13, w2, _zero_ids(input.device, M), None, out=out.view(M, 1, Hp), workspace=ws)
@@ -374,10 +401,10 @@ def _mlp_w8a16_dq_forward(input, gate_weight, up_weight, down_weight, gate_scale
         (gate_weight, up_weight, down_weight, gate_scale, up_scale, down_scale),
         lambda: (ops.pack_weights(torch.cat([_pad_to(gate_weight, Ip, Hp), _pad_to(up_weight, Ip, Hp)], 0).contiguous()),
                  torch.cat([_scales_128(gate_scale, blocksize, I, H), _scales_128(up_scale, blocksize, I, H)], 0).contiguous(),
-                 ops.pack_weights(_pad_to(down_weight, Ip, Hp).t().contiguous()),
-                 _scales_128(down_scale, blocksize, I, H).t().contiguous()),
-        f"mlp{blocksize}")
-    if _numerics == "w8a16" and Hp <= 16384 and Ip <= 16384:
+                 ops.pack_weights(_pad_to(as_t(down_weight), Ip, Hp).t().contiguous()),
+                 _scales_128(as_t(down_scale), blocksize, I, H).t().contiguous()),
+        f"mlp{blocksize}{orient}")
+    if numerics == "w8a16" and Hp <= 16384 and Ip <= 16384:
         # the reference's own arithmetic: one expert that every row selects, weights de-quantised in registers
         ids = _zero_ids(input.device, M)
         ws = _workspace(input.device, ops.fused_experts_bf16_workspace_bytes(M, Hp, Ip, 1, 1))
@@ -424,6 +451,7 @@ def _mm_w8a16_dq_forward(input, weight, scale, output, blocksize):
 
 _lib.impl("fused_moe_fused_experts", _fused_experts, "CompositeExplicitAutograd")
 _lib.impl("mlp_w8a16_dq_forward", _mlp_w8a16_dq_forward, "CompositeExplicitAutograd")
+_lib.impl("mlp_w8a8_quant_forward", _mlp_w8a8_quant_forward, "CompositeExplicitAutograd")
 _lib.impl("mm_w8a16_dq_forward", _mm_w8a16_dq_forward, "CompositeExplicitAutograd")
 _lib.impl("fused_moe_fused_experts_v2", _fused_experts_v2, "CompositeExplicitAutograd")
 _lib.impl("noaux_tc_topk", ops.noaux_tc_topk, "CompositeExplicitAutograd")
