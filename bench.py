@@ -179,6 +179,12 @@ def bench_prefill(pkg, moe, cfg, dev, steps, warmup):
     # straight on, while the chip is in that state: the two GEMMs on their own
     k1 = event_time(gemm1, max(3, steps), warmup=5)
     k2 = event_time(gemm2, max(3, steps), warmup=5)
+    # and, in the same state, what a kernel that only reads reaches: the packed W13 of the layer (far more than the
+    # 256 MB of last-level cache), one workgroup per weight strip as the first GEMM has them
+    probe_buf = moe.w13.view(torch.uint8).reshape(-1)
+    probe_piece = 256 * H
+    kp = event_time(lambda: pkg.hbm_read_probe(probe_buf, probe_piece), max(3, steps), warmup=3)
+    probe_gbs = probe_buf.numel() / kp / 1e9
     touched = int((off[1:] > off[:-1]).sum().item())
     # algorithmic traffic of one launch of the first GEMM: each touched expert's W13 (+scales) once,
     # quantised activations once, re-quantised SwiGLU output once
@@ -203,7 +209,12 @@ def bench_prefill(pkg, moe, cfg, dev, steps, warmup):
                 hbm_gbs=b1 / k1 / 1e9, hbm_frac=b1 / k1 / 1e9 / PEAK_HBM_GBS,
                 second_gemm=dict(launch_ms=k2 * 1e3, mfma_tflops=f2 / k2 / 1e12, hbm_gbs=b2 / k2 / 1e9,
                                  hbm_frac=b2 / k2 / 1e9 / PEAK_HBM_GBS),
-                experts_touched=touched)
+                experts_touched=touched,
+                read_probe=dict(gbs=probe_gbs, frac_of_peak=probe_gbs / PEAK_HBM_GBS, bytes=probe_buf.numel(),
+                                bytes_per_workgroup=probe_piece,
+                                note="a kernel of this library that only reads (moe_hbm_read_probe), same workgroup "
+                                     "decomposition as the first GEMM's weight strips, timed right after it",
+                                kernel_over_probe=(b1 / k1 / 1e9) / probe_gbs))
     return sec, roof, x
 
 

@@ -324,6 +324,15 @@ size_t moe_router_logits_workspace_bytes(int T, int H, int E);
 int moe_router_logits(void *stream, const void *x_bf16, int T, int H, const void *router_w_bf16, int E,
                       void *logits_bf16, void *workspace, size_t workspace_bytes);
 
+/*
+ * A measuring aid with no counterpart in the reference: reads `bytes` of device memory at `buf` once (16-byte
+ * aligned, a multiple of 16), one workgroup of eight wavefronts per contiguous piece of `bytes_per_workgroup`
+ * (a multiple of 16) - the decomposition the grouped GEMMs stream their weights with - and does nothing else.
+ * bench.py times it to report what a pure read reaches on the GPU at hand next to the nominal HBM peak.
+ * `sink`: 4 writable bytes (written practically never; they keep the loads alive).
+ */
+int moe_hbm_read_probe(void *stream, const void *buf, size_t bytes, size_t bytes_per_workgroup, void *sink);
+
 #ifdef __cplusplus
 }
 #endif

@@ -59,7 +59,7 @@ def test_gemm_kernels_have_no_scratch_and_no_in_flight_register_use(gemm_asm):
 
 
 @pytest.mark.parametrize("source", ["route.hip", "permute.hip", "quant_reduce.hip", "dense_small.hip", "decode_prep.hip",
-                                    "router_front.hip"])
+                                    "router_front.hip", "probe.hip"])
 def test_no_kernel_of_the_library_spills(source, tmp_path):
     """Every other kernel source: compiled to gfx950 assembly, no kernel may need scratch memory."""
     hipcc = "/opt/rocm/bin/hipcc" if os.path.exists("/opt/rocm/bin/hipcc") else "hipcc"

@@ -45,6 +45,7 @@ SIGNATURES = {
                                      c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_size_t]),
     "moe_hip_init": (c_int, []),
+    "moe_hbm_read_probe": (c_int, [c_void_p, c_void_p, c_size_t, c_size_t, c_void_p]),
     "moe_layer_fp8_static": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                      c_int, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                      c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),

@@ -12,7 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmoe_hip.so")
 SOURCES = ["route.hip", "permute.hip", "quant_reduce.hip", "gemm_fp8.hip", "dense_small.hip", "decode_prep.hip", "router_front.hip",
-           "capi.hip"]
+           "probe.hip", "capi.hip"]
 # packed fp32 VALU ops are switched off for every kernel in this library
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function", "-Wno-inline-asm",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

@@ -1,0 +1,41 @@
+// A measuring aid, not part of the path: what a pure read of device memory reaches on this GPU, with the
+// decomposition the grouped GEMMs use for their weights - one workgroup of eight wavefronts streams one contiguous
+// piece, 16 bytes per lane and load, eight loads of a lane in flight.  bench.py reports it next to the nominal HBM
+// peak so that a kernel's fraction of the peak can be read against what a kernel that does nothing else reaches.
+#include "moe_common.h"
+#include "../../include/moe_hip.h"
+
+namespace moe {
+
+__global__ __launch_bounds__(512) void hbm_read_probe_kernel(const v4i *__restrict__ p, size_t n_vec, size_t vec_per_wg,
+                                                             int *__restrict__ sink) {
+  const size_t lo = (size_t)blockIdx.x * vec_per_wg;
+  const size_t hi = lo + vec_per_wg < n_vec ? lo + vec_per_wg : n_vec;
+  v4i acc = {0, 0, 0, 0};
+  constexpr int U = 8;
+  size_t i = lo + threadIdx.x;
+  for (; i + (size_t)(U - 1) * 512 < hi; i += (size_t)U * 512) {
+    v4i v[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) v[u] = p[i + (size_t)u * 512];
+#pragma unroll
+    for (int u = 0; u < U; u++) acc ^= v[u];
+  }
+  for (; i < hi; i += 512) acc ^= p[i];
+  // the loads must not be optimised away; the store itself practically never happens
+  if ((acc[0] ^ acc[1]) == 0x5eed1234 && (acc[2] ^ acc[3]) == 0x4321deed) *sink = acc[0];
+}
+
+}  // namespace moe
+
+extern "C" int moe_hbm_read_probe(void *stream, const void *buf, size_t bytes, size_t bytes_per_workgroup, void *sink) {
+  using namespace moe;
+  if (!buf || !sink) return MOE_E_NULL;
+  if (((uintptr_t)buf % 16) || ((uintptr_t)sink % 4)) return MOE_E_ALIGN;
+  if (bytes < 16 || bytes % 16 || bytes_per_workgroup < 16 || bytes_per_workgroup % 16) return MOE_E_SHAPE;
+  const size_t n_vec = bytes / 16, per = bytes_per_workgroup / 16;
+  const size_t blocks = (n_vec + per - 1) / per;
+  if (blocks > 0x7fffffffull) return MOE_E_SHAPE;
+  hbm_read_probe_kernel<<<(unsigned)blocks, 512, 0, (hipStream_t)stream>>>((const v4i *)buf, n_vec, per, (int *)sink);
+  return (int)hipGetLastError();
+}

@@ -170,6 +170,19 @@ def unpack_weights(w):
     return _repack(w, lib.moe_unpack_weights, "unpack_weights")
 
 
+def hbm_read_probe(buf, bytes_per_workgroup: int = 1835008):
+    """Launches one pure read of `buf` (any contiguous GPU tensor whose byte size is a multiple of 16) on the current
+    stream: one workgroup of eight wavefronts per contiguous piece of `bytes_per_workgroup` (default: one weight strip of
+    the DeepSeek-V3 layer's first GEMM, 256 rows x 7168 bytes).  A measuring aid for bench.py; returns nothing."""
+    _need(isinstance(buf, torch.Tensor) and buf.is_cuda and buf.is_contiguous(), "buf must be a contiguous GPU tensor")
+    nbytes = buf.numel() * buf.element_size()
+    _need(nbytes >= 16 and nbytes % 16 == 0 and bytes_per_workgroup >= 16 and bytes_per_workgroup % 16 == 0,
+          "sizes must be multiples of 16 bytes")
+    sink = torch.empty(1, dtype=torch.int32, device=buf.device)
+    rc = lib.moe_hbm_read_probe(_stream(), buf.data_ptr(), nbytes, bytes_per_workgroup, sink.data_ptr())
+    check(rc, "moe_hbm_read_probe")
+
+
 def pack_layer(w13, w13_scale, w2, w2_scale):
     """(w13, w13_scale, w2, w2_scale) with row-major weights on the GPU -> the same with tile-blocked weights."""
     return pack_weights(w13), w13_scale, pack_weights(w2), w2_scale
