@@ -185,6 +185,8 @@ def bench_prefill(pkg, moe, cfg, dev, steps, warmup):
     probe_piece = 256 * H
     kp = event_time(lambda: pkg.hbm_read_probe(probe_buf, probe_piece), max(3, steps), warmup=3)
     probe_gbs = probe_buf.numel() / kp / 1e9
+    # the same bytes read by short-lived workgroups of 8 KB each that sweep the buffer front to back
+    kf = event_time(lambda: pkg.hbm_read_probe(probe_buf, 8192), max(3, steps), warmup=3)
     touched = int((off[1:] > off[:-1]).sum().item())
     # algorithmic traffic of one launch of the first GEMM: each touched expert's W13 (+scales) once,
     # quantised activations once, re-quantised SwiGLU output once
@@ -211,9 +213,10 @@ def bench_prefill(pkg, moe, cfg, dev, steps, warmup):
                                  hbm_frac=b2 / k2 / 1e9 / PEAK_HBM_GBS),
                 experts_touched=touched,
                 read_probe=dict(gbs=probe_gbs, frac_of_peak=probe_gbs / PEAK_HBM_GBS, bytes=probe_buf.numel(),
-                                bytes_per_workgroup=probe_piece,
+                                bytes_per_workgroup=probe_piece, gbs_short_workgroups=probe_buf.numel() / kf / 1e9,
                                 note="a kernel of this library that only reads (moe_hbm_read_probe), same workgroup "
-                                     "decomposition as the first GEMM's weight strips, timed right after it",
+                                     "decomposition as the first GEMM's weight strips, timed right after it; "
+                                     "gbs_short_workgroups: the same read by workgroups of 8 KB each",
                                 kernel_over_probe=(b1 / k1 / 1e9) / probe_gbs))
     return sec, roof, x
 
