@@ -127,11 +127,32 @@ __global__ __launch_bounds__(1024) void permute_scan_kernel(int32_t *__restrict_
   if (e < E) {
     expert_offsets[e] = off;
     tile_prefix[e] = first_tile;
-    write_tiles(e, count, off, first_tile, tile_m, tile_expert, tile_desc, max_tiles);
   }
   if (e == 0) {
     expert_offsets[E] = total;
     tile_prefix[E] = total_tiles;
+  }
+  // The tile list, one thread per tile: under a skewed load one expert holds hundreds of row tiles, and a loop over
+  // them in that expert's thread would be the longest chain of the kernel.  A tile finds its expert by bisection of
+  // the first-tile table (experts without a tile share their successor's entry and are never the answer).
+  __shared__ int t_first[1025], t_count[1024], t_off[1024];
+  t_first[e] = e < E ? first_tile : total_tiles;
+  t_count[e] = count;
+  t_off[e] = off;
+  if (e == 0) t_first[1024] = total_tiles;
+  __syncthreads();
+  const int n_tiles = min(total_tiles, max_tiles);
+  for (int j = threadIdx.x; j < n_tiles; j += 1024) {
+    int lo = 0, hi = E;                                 // t_first[lo] <= j < t_first[hi]
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (t_first[mid] <= j) lo = mid; else hi = mid;
+    }
+    const int c = t_count[lo];
+    tile_expert[j] = lo;
+    v4i *d = (v4i *)(tile_desc + (size_t)j * 8);
+    d[0] = (v4i){lo, t_first[lo], (c + tile_m - 1) / tile_m, t_off[lo]};
+    d[1] = (v4i){c, 0, 0, 0};
   }
 }
 
