@@ -16,7 +16,10 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t *__restri
   act_quant_thread(x, n_groups, groups_per_row, pitch, q, s, (size_t)blockIdx.x * 256 + threadIdx.x);
 }
 
-// One lane produces 8 consecutive columns of one token.
+// One lane produces 8 consecutive columns of one token.  STREAM: the per-slot rows are more than the last-level cache
+// holds and are read exactly once - loaded (and the result stored) with the non-temporal hint, which reads 10-12 %
+// faster there; a small batch, whose rows the second GEMM has just left in the cache, keeps the plain loads.
+template <bool STREAM>
 __global__ __launch_bounds__(256) void weighted_reduce_kernel(const uint16_t *__restrict__ y,
                                                               const float *__restrict__ w,
                                                               const uint16_t *__restrict__ shared_y,
@@ -39,7 +42,7 @@ __global__ __launch_bounds__(256) void weighted_reduce_kernel(const uint16_t *__
       const size_t slot = (size_t)t * K + min(k0 + i, K - 1);
       const bool live = k0 + i < K && (slot_to_row == nullptr || slot_to_row[slot] >= 0);
       wk[i] = live ? w[slot] : 0.f;
-      raw[i] = *(const v4i *)(y + slot * H + c);
+      raw[i] = STREAM ? __builtin_nontemporal_load((const v4i *)(y + slot * H + c)) : *(const v4i *)(y + slot * H + c);
       if (!live) raw[i] = (v4i){0, 0, 0, 0};
     }
 #pragma unroll
@@ -65,7 +68,8 @@ __global__ __launch_bounds__(256) void weighted_reduce_kernel(const uint16_t *__
 #pragma unroll
   for (int i = 0; i < 4; i++)
     o[i] = (int)((uint32_t)f32_to_bf16(acc[2 * i]) | ((uint32_t)f32_to_bf16(acc[2 * i + 1]) << 16));
-  *(v4i *)(out + (size_t)t * H + c) = o;
+  if (STREAM) __builtin_nontemporal_store(o, (v4i *)(out + (size_t)t * H + c));
+  else *(v4i *)(out + (size_t)t * H + c) = o;
 }
 
 // [T, K, H] output form: the rows of slots without an expert (id outside [0, E)) are zero.  One thread per slot; the
@@ -125,7 +129,11 @@ int weighted_reduce_launch(hipStream_t st, const uint16_t *y, const float *w, co
   if (n == 0) return MOE_OK;
   const size_t blocks = (n + 255) / 256;
   if (blocks > 0x7fffffffull) return MOE_E_SHAPE;
-  weighted_reduce_kernel<<<(unsigned)blocks, 256, 0, st>>>(y, w, shared_y, slot_to_row, T, K, H, out);
+  // 256 MB of last-level cache on this GPU
+  if ((size_t)T * K * H * 2 > ((size_t)256 << 20))
+    weighted_reduce_kernel<true><<<(unsigned)blocks, 256, 0, st>>>(y, w, shared_y, slot_to_row, T, K, H, out);
+  else
+    weighted_reduce_kernel<false><<<(unsigned)blocks, 256, 0, st>>>(y, w, shared_y, slot_to_row, T, K, H, out);
   return (int)hipGetLastError();
 }
 
