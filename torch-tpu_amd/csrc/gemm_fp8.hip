@@ -413,11 +413,12 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
       const uint8_t *base = wtile[j] + (size_t)kb * WSTEP;
       const uint32_t m0 = wt_base + stage * kWtStage + j * 2048;
       // the instruction offset advances the memory address and the LDS address alike
+      // and the non-temporal hint: with these tiles an expert's rows fit one row tile, so a weight byte is read once
       if constexpr (DQ)
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(woff), "s"(base) : "memory", "m0");
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(m0), "v"(woff), "s"(base) : "memory", "m0");
       else
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t"
-                     "global_load_lds_dwordx4 %1, %2 offset:1024"
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt\n\t"
+                     "global_load_lds_dwordx4 %1, %2 offset:1024 nt"
                      ::"s"(m0), "v"(woff), "s"(base) : "memory", "m0");
     }
   };
