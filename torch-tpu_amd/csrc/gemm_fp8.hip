@@ -257,6 +257,7 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   const int rows_a = shared ? a.sh_rows : a.rows_a;
   if (rows <= 0) return;
   const int mt_live = (rows + 15) >> 4;               // m-tiles that hold at least one row
+  const bool stream_weights = n_mt == 1;              // the expert's rows fit this one row tile
 
   const int NKB = a.Kd >> 7;
   const int n_wblk = (a.n_rows_w + 127) >> 7;         // weight-scale rows per expert
@@ -406,20 +407,36 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   auto request = [&](int kb, int stage) {
 #pragma unroll
     for (int u = 0; u < NTOK; u++) request_tok(kb, stage, u);
-    // weight tiles through LDS: an instruction copies one 1 KB half of a tile's step as it lies in memory
-    if (!WREG)
+    // weight tiles through LDS: an instruction copies one 1 KB half of a tile's step as it lies in memory (the
+    // instruction offset advances the memory address and the LDS address alike).  With the non-temporal hint when the
+    // expert's rows fit this one row tile - every weight byte is then read exactly once, and hinted loads stream 6-9 %
+    // faster; an expert with several row tiles keeps plain loads, its later tiles find the strip in L2.
+    if (!WREG) {
+      if (stream_weights) {
 #pragma unroll
-    for (int j = 0; j < WT; j++) {
-      const uint8_t *base = wtile[j] + (size_t)kb * WSTEP;
-      const uint32_t m0 = wt_base + stage * kWtStage + j * 2048;
-      // the instruction offset advances the memory address and the LDS address alike
-      // and the non-temporal hint: with these tiles an expert's rows fit one row tile, so a weight byte is read once
-      if constexpr (DQ)
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(m0), "v"(woff), "s"(base) : "memory", "m0");
-      else
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt\n\t"
-                     "global_load_lds_dwordx4 %1, %2 offset:1024 nt"
-                     ::"s"(m0), "v"(woff), "s"(base) : "memory", "m0");
+        for (int j = 0; j < WT; j++) {
+          const uint8_t *base = wtile[j] + (size_t)kb * WSTEP;
+          const uint32_t m0 = wt_base + stage * kWtStage + j * 2048;
+          if constexpr (DQ)
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(m0), "v"(woff), "s"(base) : "memory", "m0");
+          else
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt\n\t"
+                         "global_load_lds_dwordx4 %1, %2 offset:1024 nt"
+                         ::"s"(m0), "v"(woff), "s"(base) : "memory", "m0");
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < WT; j++) {
+          const uint8_t *base = wtile[j] + (size_t)kb * WSTEP;
+          const uint32_t m0 = wt_base + stage * kWtStage + j * 2048;
+          if constexpr (DQ)
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(woff), "s"(base) : "memory", "m0");
+          else
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t"
+                         "global_load_lds_dwordx4 %1, %2 offset:1024"
+                         ::"s"(m0), "v"(woff), "s"(base) : "memory", "m0");
+        }
+      }
     }
   };
 
