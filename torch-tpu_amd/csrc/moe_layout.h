@@ -28,12 +28,15 @@ static inline int choose_tile_m(int T, int K, int E) {
   // Balanced routing puts T*K/E rows on an expert, give or take a few standard deviations.  A
   // second, nearly empty tile costs as much weight traffic as a full one, so prefer the tile
   // that holds a typical expert whole.
-  // Measured on the DeepSeek-V3 shape (tile-blocked weights; step in ms with 64 / 128 / 192 rows forced): T=512 (16 rows
-  // per expert on average) 1.977 / 1.978 / 1.992, T=768 2.035 / 2.023 / 2.034, T=1024 2.076 / 2.053 / 2.082,
-  // T=1536 2.180 / 2.141 / 2.146, T=2048 2.477 / 2.221 / 2.252, T=3072 (96 rows) 2.993 / 2.404 / 2.410,
-  // T=4096 (128 rows) 3.627 / 2.924 / 2.651.
+  // Measured (step in ms with 64 / 128 / 192 rows forced; the 64-row kernel streams its weights into LDS with the
+  // non-temporal hint when an expert's rows fit one tile, which the large tiles' register loads do not profit from):
+  // DeepSeek-V3 shape, T=512 (16 rows per expert on average) 1.827 / 1.999 / -, T=768 1.877 / 2.033, T=1024 1.925 / 2.062,
+  // T=1280 (40 rows) 2.000 / 2.114, T=1536 (48 rows) 2.120 / 2.149, T=2048 (64 rows) 2.412 / 2.227 / 2.252,
+  // T=3072 2.993 / 2.404 / 2.410, T=4096 (128 rows) 3.627 / 2.924 / 2.651; Mixtral shape, T=96 (24 rows) 0.252 / 0.290 / 0.298,
+  // T=192 (48 rows) 0.297 / 0.312 / 0.319, T=256 (64 rows) 0.338 / 0.319 / 0.325; Qwen3 shape under a skewed load, T=512
+  // (32 rows) 0.130 / 0.140, T=768 (48 rows) 0.148 / 0.144, T=1024 0.172 / 0.156.
   const double mean = (double)T * K / E;
-  if (mean <= 20.0) return 64;
+  if (mean <= 40.0) return 64;
   return mean > 104.0 ? 192 : 128;
 }
 
