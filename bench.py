@@ -183,10 +183,10 @@ def bench_prefill(pkg, moe, cfg, dev, steps, warmup):
     # 256 MB of last-level cache), one workgroup per weight strip as the first GEMM has them
     probe_buf = moe.w13.view(torch.uint8).reshape(-1)
     probe_piece = 256 * H
-    kp = event_time(lambda: pkg.hbm_read_probe(probe_buf, probe_piece), max(3, steps), warmup=3)
+    kp = event_time(lambda: hbm_read_probe(probe_buf, probe_piece), max(3, steps), warmup=3)
     probe_gbs = probe_buf.numel() / kp / 1e9
     # the same bytes read by short-lived workgroups of 8 KB each that sweep the buffer front to back
-    kf = event_time(lambda: pkg.hbm_read_probe(probe_buf, 8192), max(3, steps), warmup=3)
+    kf = event_time(lambda: hbm_read_probe(probe_buf, 8192), max(3, steps), warmup=3)
     touched = int((off[1:] > off[:-1]).sum().item())
     # algorithmic traffic of one launch of the first GEMM: each touched expert's W13 (+scales) once,
     # quantised activations once, re-quantised SwiGLU output once
@@ -214,7 +214,7 @@ def bench_prefill(pkg, moe, cfg, dev, steps, warmup):
                 experts_touched=touched,
                 read_probe=dict(gbs=probe_gbs, frac_of_peak=probe_gbs / PEAK_HBM_GBS, bytes=probe_buf.numel(),
                                 bytes_per_workgroup=probe_piece, gbs_short_workgroups=probe_buf.numel() / kf / 1e9,
-                                note="a kernel of this library that only reads (moe_hbm_read_probe), same workgroup "
+                                note="a kernel that only reads (bench_hbm_read_probe in libmoe_bench_probe.so), same workgroup "
                                      "decomposition as the first GEMM's weight strips, timed right after it; "
                                      "gbs_short_workgroups: the same read by workgroups of 8 KB each",
                                 kernel_over_probe=(b1 / k1 / 1e9) / probe_gbs))
@@ -285,6 +285,31 @@ def bench_decode(pkg, moe, cfg, dev, steps, warmup, batches=(1, 8, 32)):
 def _lib():
     from torch_tpu_amd._lib import lib
     return lib
+
+
+_PROBE = None
+
+
+def hbm_read_probe(buf, bytes_per_workgroup=1835008):
+    """Launches one pure read of `buf` (a contiguous GPU tensor whose byte size is a multiple of 16) on the current stream:
+    one workgroup of eight wavefronts per contiguous piece of `bytes_per_workgroup`.  The kernel lives in
+    torch-tpu_amd/libmoe_bench_probe.so, a measuring aid of this benchmark that is not part of the product library."""
+    global _PROBE
+    import ctypes
+    if _PROBE is None:
+        path = os.path.join(ROOT, "torch-tpu_amd", "libmoe_bench_probe.so")
+        if not os.path.exists(path):
+            raise RuntimeError(f"{path} is missing: build it with `python torch-tpu_amd/build.py`")
+        _PROBE = ctypes.CDLL(path).bench_hbm_read_probe
+        _PROBE.restype = ctypes.c_int
+        _PROBE.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_void_p]
+    if not (isinstance(buf, torch.Tensor) and buf.is_cuda and buf.is_contiguous()):
+        raise RuntimeError("buf must be a contiguous GPU tensor")
+    nbytes = buf.numel() * buf.element_size()
+    sink = torch.empty(1, dtype=torch.int32, device=buf.device)
+    rc = _PROBE(torch.cuda.current_stream(buf.device).cuda_stream, buf.data_ptr(), nbytes, bytes_per_workgroup, sink.data_ptr())
+    if rc != 0:
+        raise RuntimeError(f"bench_hbm_read_probe: code {rc}")
 
 
 def bench_dense(pkg, dev, steps, warmup):

@@ -60,7 +60,15 @@ extern "C" {
 #define MOE_MAX_EXPERTS 1024
 #define MOE_MAX_TOPK    32
 
-/* Library version (major*10000 + minor*100 + patch) and the gfx target it was built for. */
+/*
+ * Library version and the gfx target it was built for.  The version changes whenever a caller built against an
+ * older header would get wrong results without an error:
+ *   100  weights row-major;
+ *   200  every GEMM entry point (moe_fused_experts_*, moe_gemm1_swiglu, moe_gemm2, moe_mm_*, moe_mlp_fp8,
+ *        moe_layer_fp8*) reads its weight bytes TILE-BLOCKED: pass them through moe_pack_weights once.
+ * Callers check moe_hip_version() >= MOE_HIP_VERSION at load time.
+ */
+#define MOE_HIP_VERSION 200
 int moe_hip_version(void);
 const char *moe_hip_arch(void);
 /* Text for a code returned by any entry point (static storage). */
@@ -260,12 +268,11 @@ int moe_mlp_fp8(void *stream, const void *x_bf16, int M, int H, const uint8_t *w
                 size_t workspace_bytes);
 
 /*
- * Router and experts of one layer in a single call, E <= 256 experts (MOE_E_SHAPE beyond that: the staged
- * calls cover every size).  Replaces, in one go, what the reference's callers chain on the host for every
+ * Router and experts of one layer in a single call, E <= MOE_MAX_EXPERTS experts.  Replaces, in one go, what the reference's callers chain on the host for every
  * token batch (python/regression/test_llm/test_torch_ops.py:440-456: logits = x Wr^T in bf16 -> sigmoid ->
  * top-k -> renormalise -> scale) and the expert op behind it
  * (torch_tpu/csrc/ops/my_ops/fusedMoE.cpp:117-236).
- * Decode-size batches (T * K <= 256 slots): two launches stand in front of the grouped GEMMs - the router
+ * Decode-size batches (T * K <= 256 slots, E <= 256): two launches stand in front of the grouped GEMMs - the router
  * logits together with the activation quantisation, then routing and permutation.  Larger batches: the
  * router product runs on the matrix cores with its reduction cut into slices, the routing kernel adds
  * the slices, and the activations are quantised by extra workgroups of that launch.  Either way the logits
@@ -302,9 +309,12 @@ int moe_layer_fp8(void *stream, const void *x_bf16, int T, int H,
  * race; calls on one stream are ordered and safe.
  * moe_hip_init() looks the array's device address up for the current device (once per device; the entry
  * point does the same on its first call there) - call it before capturing a graph on that device.
+ * moe_static_scratch_address() reports that device address (for the current device): what the kernels of
+ * moe_layer_fp8_static are handed as their workspace, so that a test can watch the array itself.
  */
 #define MOE_STATIC_SCRATCH_BYTES (16u << 20)
 int moe_hip_init(void);
+int moe_static_scratch_address(void **address);
 int moe_layer_fp8_static(void *stream, const void *x_bf16, int T, int H,
                          const void *router_w_bf16, const float *router_bias, int E, int K, int mode,
                          int n_groups, int topk_groups, int renorm, float scale,
@@ -315,7 +325,7 @@ int moe_layer_fp8_static(void *stream, const void *x_bf16, int T, int H,
                          void *out_bf16, void *logits_out_bf16, float *weights_out, int32_t *ids_out);
 
 /*
- * The router product on its own (any T, E <= 256): logits [T, E] bf16 = x [T, H] . router_w [E, H]^T, the
+ * The router product on its own (any T, E <= MOE_MAX_EXPERTS): logits [T, E] bf16 = x [T, H] . router_w [E, H]^T, the
  * first step of the routing recipe (test_torch_ops.py:440).  The kernel moe_layer_fp8 uses for batches
  * beyond the decode size, followed by the sum over its slices.
  * workspace: moe_router_logits_workspace_bytes(T, H, E) bytes, 256-byte aligned.
@@ -323,15 +333,6 @@ int moe_layer_fp8_static(void *stream, const void *x_bf16, int T, int H,
 size_t moe_router_logits_workspace_bytes(int T, int H, int E);
 int moe_router_logits(void *stream, const void *x_bf16, int T, int H, const void *router_w_bf16, int E,
                       void *logits_bf16, void *workspace, size_t workspace_bytes);
-
-/*
- * A measuring aid with no counterpart in the reference: reads `bytes` of device memory at `buf` once (16-byte
- * aligned, a multiple of 16), one workgroup of eight wavefronts per contiguous piece of `bytes_per_workgroup`
- * (a multiple of 16) - the decomposition the grouped GEMMs stream their weights with - and does nothing else.
- * bench.py times it to report what a pure read reaches on the GPU at hand next to the nominal HBM peak.
- * `sink`: 4 writable bytes (written practically never; they keep the loads alive).
- */
-int moe_hbm_read_probe(void *stream, const void *buf, size_t bytes, size_t bytes_per_workgroup, void *sink);
 
 #ifdef __cplusplus
 }

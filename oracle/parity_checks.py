@@ -10,7 +10,7 @@ neighbouring code on the device.  A fraction allowance alone ("at most x % of th
 pass a kernel that corrupts a few rows, so the comparison is made in strict steps instead:
 
   (0) quantised activations: bit-exact;
-  (1) re-quantised SwiGLU output: every device code within ONE e4m3 step of the oracle's, >= 99 % identical,
+  (1) re-quantised SwiGLU output: every device code within ONE e4m3 step of the oracle's, >= 99.5 % identical,
       scales within 5e-4;
   (2) second GEMM: EVERY element of the per-slot results (the reference op's output form, [T,K,H]) within
       rtol 2e-2 / atol 1e-2 of the oracle evaluated on the codes the device produced; the weighted sum over the
@@ -29,10 +29,13 @@ import torch
 RTOL, ATOL = 2e-2, 1e-2
 # end-to-end caps against the oracle's own codes, with (1) and (2) holding: share of elements outside the
 # tolerance, and the worst |got - ref| / (atol + rtol |ref|).  One e4m3 step (1/8 relative at most) on a handful
-# of a row's I elements moves an output by a few atol at most; measured <= 0.2 % and <= 4.
-MAX_OUTSIDE = 5e-3
-MAX_WORST = 12.0
+# of a row's I elements moves an output by a few atol at most; measured at full layer size: 0.03 % of the per-slot
+# outputs, 0.18-0.27 % of the weighted sums, worst 3.2-4.8.
+MAX_OUTSIDE = 4e-3
+MAX_WORST = 8.0
 MAX_COS_DIFF = 3e-5
+# share of the re-quantised SwiGLU codes that must equal the oracle's (measured 0.9983-0.9986 at full layer size)
+MIN_CODES_IDENTICAL = 0.995
 
 
 def outside_fraction(got: torch.Tensor, ref: torch.Tensor) -> float:
@@ -63,7 +66,10 @@ def assert_codes_within_one_step(oracle, hq_dev, hs_dev, hq_ref, hs_ref, what: s
     ok = (v_dev - v_ref).abs() <= oracle.e4m3_step(hq_ref) + 0.0625
     assert ok.all(), f"{what}: {int((~ok).sum())} re-quantised codes are more than one e4m3 step off"
     same = (hq_dev == hq_ref).float().mean().item() if hq_dev.numel() else 1.0
-    assert same >= 0.99, f"{what}: only {same:.4f} of the re-quantised codes match"
+    # a sample of a few hundred codes may hold a handful of boundary cases: four codes of grace on top of the share
+    differing = int((hq_dev != hq_ref).sum())
+    assert differing <= (1.0 - MIN_CODES_IDENTICAL) * hq_dev.numel() + 4, \
+        f"{what}: only {same:.4f} of the {hq_dev.numel()} re-quantised codes match"
     return same
 
 

@@ -36,7 +36,7 @@ def test_binding_table_covers_the_header(pkg):
 
 def test_version_and_arch(pkg):
     from torch_tpu_amd._lib import lib
-    assert lib.moe_hip_version() >= 100
+    assert lib.moe_hip_version() >= 200      # 200: tile-blocked weights
     assert lib.moe_hip_arch() == b"gfx950"
     assert lib.moe_hip_strerror(0) == b"ok"
     assert b"NULL" in lib.moe_hip_strerror(-1)

@@ -314,3 +314,22 @@ def test_mlp_w8a8_quant_forward(pkg, oracle, dev, M, H, I):
                                torch.cat([sg, su], 0).float(), pad(wd, Hp, Ip), sd.float())[:, :H]
     assert normalised_outside(got, ref) <= MAX_OUTSIDE
     assert oracle.cal_diff(ref, got)[0] < 1e-4
+
+
+def test_w8a16_beyond_its_range_raises_instead_of_switching_arithmetic(pkg, dev):
+    """set_expert_numerics('w8a16') covers reduction lengths up to 16384.  Beyond that the dense ops (and the expert op)
+    raise; they never fall through to the FP8-activation arithmetic the caller did not select."""
+    M, K, N = 4, 16384 + 128, 32
+    w = torch.zeros(N, K, dtype=torch.float8_e4m3fn, device=dev)
+    s = torch.ones(N // 128 + 1, K // 128, dtype=torch.bfloat16, device=dev)
+    x = torch.zeros(M, K, dtype=torch.bfloat16, device=dev)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    pkg.set_expert_numerics("w8a16")
+    try:
+        with pytest.raises(RuntimeError, match="up to 16384"):
+            torch.ops.my_ops.mm_w8a16_dq_forward(x, w, s, out, 128)
+    finally:
+        pkg.set_expert_numerics("w8a8")
+    torch.ops.my_ops.mm_w8a16_dq_forward(x, w, s, out, 128)        # the default arithmetic takes the shape
+    torch.cuda.synchronize()
+    assert float(out.float().abs().max()) == 0.0

@@ -194,15 +194,16 @@ def test_large_batch_addresses(pkg, oracle, dev):
 
 
 def test_read_probe_reads_any_size_and_rejects_bad_arguments(pkg, dev):
-    """moe_hbm_read_probe (bench.py's yardstick): runs on sizes that its piece size does not divide, leaves the buffer
-    alone, and refuses sizes that are not multiples of 16 bytes."""
+    """bench.py's yardstick (bench_hbm_read_probe, a library of its own beside the product's): runs on sizes that its
+    piece size does not divide, leaves the buffer alone, and refuses sizes that are not multiples of 16 bytes."""
+    import bench
     buf = torch.arange(3 * 1000 * 16 + 16, dtype=torch.uint8, device=dev)
     before = buf.clone()
     for piece in (16, 4096, 1 << 20, 1 << 30):
-        pkg.hbm_read_probe(buf, piece)
+        bench.hbm_read_probe(buf, piece)
     torch.cuda.synchronize()
     assert torch.equal(buf, before)
     with pytest.raises(RuntimeError):
-        pkg.hbm_read_probe(buf[:24])
+        bench.hbm_read_probe(buf[:24])
     with pytest.raises(RuntimeError):
-        pkg.hbm_read_probe(buf, 24)
+        bench.hbm_read_probe(buf, 24)

@@ -112,3 +112,71 @@ def test_decode_deepseek_shape_full_size(pkg, oracle, dev, checks, ds_layer, T):
                           shared=shared)
     torch.cuda.synchronize()
     assert torch.equal(again.view(torch.int16), out.view(torch.int16))
+
+
+def _router_logits_close(x, wr, logits):
+    exact = x.double().cpu() @ wr.double().cpu().t()
+    err = (logits.double().cpu() - exact).abs()
+    bound = exact.abs() * 2.0 ** -8 + 1e-4 * x.double().cpu().norm(dim=1, keepdim=True) * wr.double().cpu().norm(dim=1)[None]
+    assert bool((err <= bound).all()), float((err - bound).max())
+
+
+def _timed_softmax_step(pkg, oracle, checks, dev, T, Hh, Ii, Ee, Kk, bias, pick, what, tile):
+    """One call of the layer entry point as the benchmark times it (router product, softmax routing, permutation,
+    quantisation, both grouped GEMMs, weighted sum) at the workload's full size: logits against an fp64 product,
+    ids / weights exactly given the device's logits, permutation exactly, and sampled tokens of the batch's OWN
+    output through the strict steps of oracle/parity_checks.py."""
+    say(what, "timed path, T =", T, "tile rows", pkg.tile_rows(T, Kk, Ee))
+    assert pkg.tile_rows(T, Kk, Ee) == tile
+    layer = (*pkg.synthetic_weights(Ee, 2 * Ii, Hh, dev, 1), *pkg.synthetic_weights(Ee, Hh, Ii, dev, 2))
+    g = torch.Generator(device=dev).manual_seed(5)
+    wr = (torch.randn(Ee, Hh, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    gx = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn(T, Hh, generator=gx, device=dev).to(torch.bfloat16)
+    mode = "softmax" if bias is None else "softmax_logit_bias"
+    out, logits, w, ids = pkg.layer_fp8(x, wr, *layer, Kk, mode, bias=bias, renorm=True, return_routing=True)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    _router_logits_close(x, wr, logits)
+    lg = logits.float().cpu() if bias is None else logits.float().cpu() + bias.cpu()
+    w_ref, ids_ref = oracle.route_softmax_topk(lg, Kk, True)
+    assert torch.equal(ids.cpu(), ids_ref), "routing ids differ from the oracle's on the device's logits"
+    assert torch.allclose(w.cpu(), w_ref, rtol=1e-5, atol=1e-7)
+    ss, off, s2r = pkg.moe_permute(ids, Ee)
+    ss_ref, off_ref, s2r_ref = oracle.permute_counting_sort(ids_ref, Ee)
+    assert torch.equal(ss.cpu(), ss_ref) and torch.equal(off.cpu(), off_ref) and torch.equal(s2r.cpu(), s2r_ref)
+    # the staged entry point on the same routing: same bits
+    out2 = pkg.fused_experts_fp8(x, *layer, ids, w)
+    y = pkg.fused_experts_fp8(x, *layer, ids)
+    torch.cuda.synchronize()
+    assert torch.equal(out2.view(torch.int16), out.view(torch.int16))
+    pick = pick.to(dev)
+    rep = checks.check_sample(pkg, oracle, x[pick].contiguous(), ids[pick].contiguous(), layer,
+                              w_s=w[pick].contiguous(), y_big=y[pick].contiguous(), out_big=out[pick].contiguous(),
+                              what=what)
+    say("   ", rep)
+    return off_ref
+
+
+def test_timed_prefill_path_mixtral_shape(pkg, oracle, dev, checks):
+    """The Mixtral-8x7B-shaped step the benchmark reports under other_shapes (T=4096, E=8, top-2, 1024 rows per expert)."""
+    _timed_softmax_step(pkg, oracle, checks, dev, 4096, 4096, 14336, 8, 2, None,
+                        torch.tensor([0, 7, 1900, 3333, 4095]), "C2 T=4096", 192)
+    torch.cuda.empty_cache()
+
+
+def test_timed_prefill_path_skewed_load(pkg, oracle, dev, checks):
+    """The Qwen3-30B-A3B-shaped step under the skewed load (T=16384, E=128, top-8; popularity ~ rank^-1.2 through a bias
+    on the logits, 13 experts switched off): experts with thousands of rows next to experts with a handful and none."""
+    Ee = 128
+    g = torch.Generator(device=dev).manual_seed(5)
+    torch.randn(Ee, 2048, generator=g, device=dev)              # the router weight's draw comes first, as in the benchmark
+    rank = torch.randperm(Ee, generator=g, device=dev).float() + 1
+    bias = -1.2 * torch.log(rank)
+    dead = torch.randperm(Ee, generator=g, device=dev)[:13]
+    bias[dead] = -1e9
+    off = _timed_softmax_step(pkg, oracle, checks, dev, 16384, 2048, 768, Ee, 8, bias,
+                              torch.tensor([0, 5000, 11111, 12345, 16383]), "C5 T=16384", 192)
+    counts = off[1:] - off[:-1]
+    assert int((counts[dead.cpu()] == 0).all()) and int((counts == 0).sum()) >= 13 and int(counts.max()) > 4000
+    torch.cuda.empty_cache()

@@ -208,12 +208,13 @@ def test_softmax_router_whose_bias_is_part_of_the_logits(pkg, oracle, dev, T):
     moe = pkg.FusedMoE(wr, *ld, top_k=K, mode="softmax", bias=biasd)
     assert moe._one_call(T) and moe.layer_mode() == "softmax_logit_bias"
     assert torch.equal(moe(x).view(torch.int16), out.view(torch.int16))
-    wm, im = moe.route(x)                                              # its staged road: torch.matmul logits + bias
+    wm, im = moe.route(x)                                              # its staged road: the router product and the selection, call by call
     assert not bool(torch.isin(im.cpu().long(), off).any())
 
 
 @pytest.mark.parametrize("T,H,E", [(1, 128, 1), (5, 7168, 256), (64, 256, 16), (65, 384, 100), (700, 7168, 256),
-                                   (4096, 2048, 128), (130, 9216, 37)])
+                                   (4096, 2048, 128), (130, 9216, 37), (3, 512, 257), (200, 1024, 384), (70, 256, 1024),
+                                   (300, 384, 1000)])
 def test_router_logits_kernel(pkg, dev, T, H, E):
     say("router logits", T, H, E)
     g = torch.Generator().manual_seed(T + H + E)
@@ -262,12 +263,12 @@ def test_layer_entry_point_rejects_what_it_does_not_cover(pkg, oracle, dev):
     H, I = 256, 128
     g = torch.Generator().manual_seed(1)
     assert pkg.layer_eligible(33, 16, 8) and pkg.layer_eligible(4096, 256, 8)
-    assert not pkg.layer_eligible(1, 257, 8) and not pkg.layer_eligible(1, 4, 8)
+    assert pkg.layer_eligible(1, 1024, 8) and not pkg.layer_eligible(1, 1025, 8) and not pkg.layer_eligible(1, 4, 8)
     lib = pkg._lib.lib
-    # more than 256 experts: refused on the shape alone, before anything is launched (the pointers are never used)
-    assert lib.moe_layer_fp8(None, 1, 1, H, 1, None, 300, 8, 0, 1, 1, 1, 1.0, 1, 1, 1, 1, I, None, None, None, None,
+    # more than 1024 experts: refused on the shape alone, before anything is launched (the pointers are never used)
+    assert lib.moe_layer_fp8(None, 1, 1, H, 1, None, 1300, 8, 0, 1, 1, 1, 1.0, 1, 1, 1, 1, I, None, None, None, None,
                              0, 1, None, None, None, 256, 1 << 30) == -2
-    assert lib.moe_layer_fp8_workspace_bytes(1, H, I, 300, 8, 0) == 0
+    assert lib.moe_layer_fp8_workspace_bytes(1, H, I, 1300, 8, 0) == 0
     E, K = 16, 8
     ld = pkg.pack_layer(*(t.to(dev) for t in oracle.make_layer(E, H, I, seed=1)))
     wr = (torch.randn(E, H, generator=g) * 0.05).to(torch.bfloat16).to(dev)
@@ -351,3 +352,89 @@ def test_checkpoint_converter_feeds_the_kernels(pkg, oracle, dev, checks):
     ss, off, s2r = torch.ops.my_ops.moe_permute(ids, E)
     ss_ref, off_ref, s2r_ref = oracle.permute_counting_sort(ids.cpu(), E)
     assert torch.equal(ss.cpu(), ss_ref) and torch.equal(off.cpu(), off_ref) and torch.equal(s2r.cpu(), s2r_ref)
+
+
+def test_checkpoint_converter_pads_ragged_sizes_and_names_the_device_it_needs(pkg, oracle, dev):
+    """A checkpoint whose H and I are no multiples of 128 (partial blocks at the edges, ceil(n/128) scales): the
+    converter pads codes to whole blocks like the reference-layout packer does, and the layer runs on activations
+    padded the same way; asked to tile-block host tensors it says what it needs."""
+    say("checkpoint converter, ragged sizes")
+    E, H, I, K, T = 4, 328, 200, 2, 9
+    Hp, Ip = 384, 256
+    g = torch.Generator().manual_seed(5)
+    state, pre = {}, "m."
+    dense = {}
+    for e in range(E):
+        for proj, (n, k) in (("gate_proj", (I, H)), ("up_proj", (I, H)), ("down_proj", (H, I))):
+            wfull = torch.zeros(-(-n // 128) * 128, -(-k // 128) * 128)
+            wfull[:n, :k] = torch.randn(n, k, generator=g) * 0.05
+            q, sc = oracle.quant_weight_block128(wfull)
+            state[f"{pre}experts.{e}.{proj}.weight"], state[f"{pre}experts.{e}.{proj}.weight_scale_inv"] = q[:n, :k].contiguous(), sc
+            dense[(e, proj)] = (q, sc)
+    state[pre + "gate.weight"] = (torch.randn(E, H, generator=g) * 0.05).to(torch.bfloat16)
+    with pytest.raises(RuntimeError, match="device="):
+        pkg.convert_hf_moe_layer(state, pre, E)
+    conv = pkg.convert_hf_moe_layer(state, pre, E, device=dev)
+    assert tuple(conv["w13"].shape) == (E, 2 * Ip, Hp) and tuple(conv["w2"].shape) == (E, Hp, Ip)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    xp = torch.nn.functional.pad(x, (0, Hp - H)).to(dev)
+    ids, w = torch.tensor([[e % E, (e + 1) % E] for e in range(T)], dtype=torch.int32), torch.full((T, K), 0.5)
+    out = pkg.fused_experts_fp8(xp, conv["w13"], conv["w13_scale"], conv["w2"], conv["w2_scale"], ids.to(dev), w.to(dev))
+    torch.cuda.synchronize()
+    layer = (torch.cat([torch.stack([dense[(e, "gate_proj")][0] for e in range(E)]),
+                        torch.stack([dense[(e, "up_proj")][0] for e in range(E)])], 1),
+             torch.cat([torch.stack([dense[(e, "gate_proj")][1] for e in range(E)]),
+                        torch.stack([dense[(e, "up_proj")][1] for e in range(E)])], 1),
+             torch.stack([dense[(e, "down_proj")][0] for e in range(E)]),
+             torch.stack([dense[(e, "down_proj")][1] for e in range(E)]))
+    ref = oracle.moe_w8a8_fp32(xp.cpu(), ids, w, *layer)
+    got = out.float().cpu()
+    assert float(got[:, H:].abs().max()) == 0.0            # the padding columns of the output are zero
+    scale = ref.abs().max().item()
+    assert ((got - ref).abs() <= 1e-2 * scale + 2e-2 * ref.abs()).float().mean() >= 0.995
+
+
+@pytest.mark.parametrize("T,E,K,mode,G,TG", [(1, 384, 8, "sigmoid", 8, 4), (9, 512, 6, "softmax", 1, 1),
+                                             (40, 1024, 8, "sigmoid", 16, 5), (300, 320, 4, "softmax_logit_bias", 1, 1)])
+def test_layer_entry_point_with_more_than_256_experts(pkg, oracle, dev, checks, T, E, K, mode, G, TG):
+    """Layers with more than 256 experts (up to 1024) run behind the same entry point: the router product in blocks of
+    256 experts, routing from the partial sums, the permutation.  Logits against an fp64 product; ids and weights equal
+    the stand-alone routing entry point's on the same logits and the oracle's; the output equals the staged entry
+    point's on the same routing, bit for bit; a sample of tokens through the strict steps."""
+    say("layer with", E, "experts, T =", T, mode)
+    H, I = 512, 128
+    ld = pkg.pack_layer(*(t.to(dev) for t in oracle.make_layer(E, H, I, seed=E)))
+    g = torch.Generator().manual_seed(E + T)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+    wr = (torch.randn(E, H, generator=g) * 0.05).to(torch.bfloat16).to(dev)
+    bias = None if mode == "softmax" else (torch.randn(E, generator=g) * 0.1).to(dev)
+    scale = 2.5 if mode == "sigmoid" else 1.0
+    out, logits, w, ids = pkg.layer_fp8(x, wr, *ld, K, mode, bias=bias, n_groups=G, topk_groups=TG, renorm=True, scale=scale,
+                                        return_routing=True)
+    torch.cuda.synchronize()
+    exact = x.double().cpu() @ wr.double().cpu().t()
+    err = (logits.double().cpu() - exact).abs()
+    bound = exact.abs() * 2.0 ** -8 + 1e-4 * x.double().cpu().norm(dim=1, keepdim=True) * wr.double().cpu().norm(dim=1)[None]
+    assert bool((err <= bound).all())
+    assert torch.equal(logits.view(torch.int16), pkg.router_logits(x, wr).view(torch.int16))
+    w1, ids1 = pkg.moe_route(logits, K, mode, bias=bias, n_groups=G, topk_groups=TG, renorm=True, scale=scale)
+    assert torch.equal(ids, ids1) and torch.equal(w, w1)
+    if mode == "sigmoid":
+        scores = pkg.moe_route(logits, K, mode, bias=bias, n_groups=G, topk_groups=TG, renorm=True, scale=scale,
+                               return_scores=True)[2].cpu()
+        w_ref, ids_ref = oracle.select_sigmoid_grouped(scores, bias.cpu(), K, G, TG, scale, True)
+    else:
+        lg = logits.float().cpu() + (bias.cpu() if mode == "softmax_logit_bias" else 0.0)
+        w_ref, ids_ref = oracle.route_softmax_topk(lg, K, True)
+    assert torch.equal(ids.cpu(), ids_ref) and torch.allclose(w.cpu(), w_ref, rtol=1e-5, atol=1e-7)
+    staged = pkg.fused_experts_fp8(x, *ld, ids, w)
+    assert torch.equal(out.view(torch.int16), staged.view(torch.int16))
+    moe = pkg.FusedMoE(wr, *ld, top_k=K, mode="softmax" if mode == "softmax_logit_bias" else mode, bias=bias, n_groups=G,
+                       topk_groups=TG, renorm=True, scale=scale)
+    assert torch.equal(moe(x).view(torch.int16), out.view(torch.int16))
+    wm, im = moe.route(x)                                  # the module's staged road: the same kernels, call by call
+    assert torch.equal(im, ids) and torch.equal(wm, w)
+    pick = torch.arange(min(T, 6), device=dev)
+    rep = checks.check_sample(pkg, oracle, x[pick].contiguous(), ids[pick].contiguous(), ld, w_s=w[pick].contiguous(),
+                              out_big=out[pick].contiguous(), what=f"E={E}")
+    say("   ", rep)

@@ -329,7 +329,7 @@ def check_experts(pkg, oracle, dev, x, layer, ids, w, shared=None):
     # fp32 sums' absolute error) 1.4e-4 of the group maximum = 1/16 in units of the scale
     assert ((v_dev - v_ref).abs() <= oracle.e4m3_step(hq_r) + 0.0625).all(), "a code is more than one step off"
     same = (hq_dev == hq_r).float().mean().item()
-    assert same >= 0.99, f"only {same:.4f} of the re-quantised codes match"
+    assert int((hq_dev != hq_r).sum()) <= 0.005 * hq_dev.numel() + 4, f"only {same:.4f} of the re-quantised codes match"
 
     # ---- (2) second GEMM on the device's own codes: strict, every element
     y_mid = oracle.experts_w8a8_fp32(x, ids, *layer, mid=(hq_dev.reshape(T, K, I), hs_dev.reshape(T, K, -1)))
@@ -487,6 +487,59 @@ def test_my_ops_drop_in_reference_layout(pkg, oracle, dev, checks):
     got16 = out.float().cpu()
     assert oracle.cos_sim(ref_bf16.numpy(), got16.numpy()) > 0.99
     assert oracle.cal_diff(ref_bf16, got16)[0] < 1e-4
+
+
+def test_my_ops_registered_from_cpp_keeps_one_packed_copy_per_weight_set(pkg, oracle, dev):
+    """The reference's op names come from the C++ extension (TORCH_LIBRARY, function pointers: inferred schemas with
+    unnamed arguments).  The packed copy of a weight set belongs to the sources' storages: fresh Python wrappers of the
+    same storages (`.data`, views made per call) find it again, an in-place change or new tensors do not; both output
+    forms equal the staged entry point on weights packed by hand, bit for bit."""
+    say("my_ops C++ registration and its packed-copy table")
+    ops = torch.ops.my_ops
+    assert ops.fused_moe_fused_experts.default._schema.arguments[0].name == "_0"
+    T, H, I, E, K = 5, 512, 256, 8, 2
+    g = torch.Generator().manual_seed(77)
+    gate, up, down = ((torch.randn(E, I, H, generator=g) * 0.1).to(torch.float8_e4m3fn).to(dev) for _ in range(3))
+    gs, us, ds = ((torch.rand(E, I // 128, H // 128, generator=g) * 0.1 + 0.01).to(torch.bfloat16).to(dev) for _ in range(3))
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+    ids, w = distinct_ids(T, E, K, seed=3)
+    ids, w16 = ids.to(dev), w.to(torch.bfloat16).to(dev)
+    tail = [None, None, None, 128, E, K, False, 1, 1, None, None, None, False]
+    pkg.invalidate_weight_cache()
+    assert ops._packed_weight_sets() == 0
+    out = torch.empty(T, K, H, dtype=torch.bfloat16, device=dev)
+    ops.fused_moe_fused_experts(out, x, None, None, gate, up, down, gs, us, ds, ids, w16, *tail)
+    assert ops._packed_weight_sets() == 1
+    for _ in range(3):          # new wrapper objects around the same storages: no second copy
+        out2 = torch.empty_like(out)
+        ops.fused_moe_fused_experts(out2, x, None, None, gate.data, up.view(E, I, H), down[:], gs.data, us.data, ds.data,
+                                    ids, w16, *tail)
+        assert ops._packed_weight_sets() == 1
+        assert torch.equal(out2.view(torch.int16), out.view(torch.int16))
+    packed = pkg.pack_expert_weights(gate, up, down, gs, us, ds)
+    want = pkg.fused_experts_fp8(x, *packed, ids)
+    assert torch.equal(want.view(torch.int16), out.view(torch.int16))
+    # the weighted form, routing weights in bf16 as the reference's callers hold them
+    red = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    ops.fused_moe_fused_experts(red, x, None, None, gate, up, down, gs, us, ds, ids, w16, *tail)
+    want_red = pkg.fused_experts_fp8(x, *packed, ids, w16.float())
+    assert torch.equal(red.view(torch.int16), want_red.view(torch.int16))
+    # a recorded in-place change re-packs; so do new tensors
+    gs.mul_(2.0)
+    ops.fused_moe_fused_experts(out2, x, None, None, gate, up, down, gs, us, ds, ids, w16, *tail)
+    assert ops._packed_weight_sets() == 2
+    want2 = pkg.fused_experts_fp8(x, *pkg.pack_expert_weights(gate, up, down, gs, us, ds), ids)
+    assert torch.equal(out2.view(torch.int16), want2.view(torch.int16))
+    del gate
+    gate2 = (torch.randn(E, I, H, generator=g) * 0.1).to(torch.float8_e4m3fn).to(dev)
+    ops.fused_moe_fused_experts(out2, x, None, None, gate2, up, down, gs, us, ds, ids, w16, *tail)
+    torch.cuda.synchronize()
+    assert ops._packed_weight_sets() == 1          # the entries whose gate storage is gone were dropped on the way
+    pkg.invalidate_weight_cache()
+    assert ops._packed_weight_sets() == 0
+    with pytest.raises(RuntimeError, match="do not match"):
+        ops.fused_moe_fused_experts(out, x, None, None, gate2, up, down, gs, us, ds, ids, w16, None, None, None, 128, E + 1,
+                                    K, False, 1, 1, None, None, None, False)
 
 
 @pytest.mark.parametrize("block", [64, 256])

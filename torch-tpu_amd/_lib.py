@@ -10,6 +10,8 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libmoe_hip.so")
 
+MIN_VERSION = 200        # MOE_HIP_VERSION of include/moe_hip.h: weights are handed over tile-blocked
+
 # name -> (restype, argtypes); the single source for both binding and the symbol test
 SIGNATURES = {
     "moe_hip_version": (c_int, []),
@@ -45,7 +47,7 @@ SIGNATURES = {
                                      c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_size_t]),
     "moe_hip_init": (c_int, []),
-    "moe_hbm_read_probe": (c_int, [c_void_p, c_void_p, c_size_t, c_size_t, c_void_p]),
+    "moe_static_scratch_address": (c_int, [ctypes.POINTER(c_void_p)]),
     "moe_layer_fp8_static": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                      c_int, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                      c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
@@ -75,6 +77,9 @@ def _load():
         fn = getattr(lib, name)          # AttributeError if the symbol is absent
         fn.restype = res
         fn.argtypes = args
+    if lib.moe_hip_version() < MIN_VERSION:
+        raise ImportError(f"{LIB_PATH} is version {lib.moe_hip_version()}, this package needs >= {MIN_VERSION} "
+                          "(the weight layout of the GEMM entry points changed): rebuild it")
     return lib
 
 

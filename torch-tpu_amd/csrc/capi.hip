@@ -122,8 +122,9 @@ struct LayerWs {
   size_t bytes;
 };
 
-// up to this many slots (T * K) one workgroup can permute, and the two-launch decode front end applies
-static bool decode_size(int T, int K) { return (long)T * K <= kChunk; }
+// the two-launch decode front end: up to kChunk slots (T * K), which one workgroup can permute, and up to 256 experts,
+// which one workgroup can rank; every other problem takes the matrix-core router product, routing and permutation launches
+static bool decode_size(int T, int K, int E) { return (long)T * K <= kChunk && E <= 256; }
 
 static LayerWs layer_layout(void *base, int T, int H, int I, int E, int K, int I_sh) {
   LayerWs d{};
@@ -138,7 +139,7 @@ static LayerWs layer_layout(void *base, int T, int H, int I, int E, int K, int I
   d.weights = (float *)take((size_t)T * K * 4);
   d.ids = (int32_t *)take((size_t)T * K * 4);
   d.arrivals = (int *)take(4);
-  if (!decode_size(T, K)) d.partial = (float *)take(router_front_partial_bytes(T, H, E));
+  if (!decode_size(T, K, E)) d.partial = (float *)take(router_front_partial_bytes(T, H, E));
   d.bytes = off;
   return d;
 }
@@ -152,7 +153,8 @@ static bool dims_in_range(int T, int H, int I, int K) {
 
 }  // namespace moe
 
-extern "C" int moe_hip_version(void) { return 100; }
+// 200: the GEMM entry points read their weights tile-blocked (moe_pack_weights); 100 read them row-major
+extern "C" int moe_hip_version(void) { return 200; }
 extern "C" const char *moe_hip_arch(void) { return "gfx950"; }
 
 extern "C" const char *moe_hip_strerror(int code) {
@@ -215,7 +217,7 @@ extern "C" int moe_fused_experts_fp8(void *stream, const void *x_bf16, int T, in
 }
 
 extern "C" size_t moe_layer_fp8_workspace_bytes(int T, int H, int I, int E, int K, int I_shared) {
-  if (T < 0 || H < 1 || I < 1 || E < 1 || E > 256 || K < 1 || I_shared < 0 || H % moe::kBlock) return 0;
+  if (T < 0 || H < 1 || I < 1 || E < 1 || E > MOE_MAX_EXPERTS || K < 1 || I_shared < 0 || H % moe::kBlock) return 0;
   return moe::layer_layout(nullptr, T, H, I, E, K, I_shared).bytes;
 }
 
@@ -229,7 +231,7 @@ static int layer_fp8_run(void *stream, const void *x_bf16, int T, int H, const v
                          size_t workspace_bytes) {
   if (!router_w_bf16 || !w13 || !w13_scale || !w2 || !w2_scale || !workspace) return MOE_E_NULL;
   if (T != 0 && (!x_bf16 || !out_bf16)) return MOE_E_NULL;
-  if (T < 0 || H < 1 || I < 1 || E < 1 || E > 256 || K < 1 || K > MOE_MAX_TOPK || K > E) return MOE_E_SHAPE;
+  if (T < 0 || H < 1 || I < 1 || E < 1 || E > MOE_MAX_EXPERTS || K < 1 || K > MOE_MAX_TOPK || K > E) return MOE_E_SHAPE;
   if ((long)T * K > (1l << 30)) return MOE_E_SHAPE;
   if (!dims_in_range(T, H, I, K)) return MOE_E_SHAPE;
   if (mode != MOE_ROUTE_SOFTMAX && mode != MOE_ROUTE_SIGMOID && mode != MOE_ROUTE_SOFTMAX_LOGIT_BIAS) return MOE_E_MODE;
@@ -253,7 +255,7 @@ static int layer_fp8_run(void *stream, const void *x_bf16, int T, int H, const v
   float *weights = weights_out ? weights_out : d.weights;
   int32_t *ids = ids_out ? ids_out : d.ids;
   int rc;
-  if (decode_size(T, K)) {
+  if (decode_size(T, K, E)) {
     // two launches: router logits + activation quantisation, then routing + permutation
     rc = decode_prep_launch(st, (const uint16_t *)x_bf16, T, H, (const uint16_t *)router_w_bf16, router_bias, E, K, mode,
                             n_groups, topk_groups, renorm, scale, logits_out_bf16 ? (uint16_t *)logits_out_bf16 : d.logits,
@@ -330,6 +332,11 @@ extern "C" int moe_hip_init(void) {
   return moe::static_scratch(&p);
 }
 
+extern "C" int moe_static_scratch_address(void **address) {
+  if (!address) return MOE_E_NULL;
+  return moe::static_scratch(address);
+}
+
 extern "C" int moe_layer_fp8_static(void *stream, const void *x_bf16, int T, int H, const void *router_w_bf16,
                                     const float *router_bias, int E, int K, int mode, int n_groups, int topk_groups,
                                     int renorm, float scale, const uint8_t *w13, const float *w13_scale,
@@ -338,7 +345,8 @@ extern "C" int moe_layer_fp8_static(void *stream, const void *x_bf16, int T, int
                                     const float *shared_w2_scale, int I_shared, void *out_bf16, void *logits_out_bf16,
                                     float *weights_out, int32_t *ids_out) {
   using namespace moe;
-  if (T < 0 || H < 1 || I < 1 || E < 1 || E > 256 || K < 1 || K > MOE_MAX_TOPK || K > E || I_shared < 0) return MOE_E_SHAPE;
+  if (T < 0 || H < 1 || I < 1 || E < 1 || E > MOE_MAX_EXPERTS || K < 1 || K > MOE_MAX_TOPK || K > E || I_shared < 0)
+    return MOE_E_SHAPE;
   if (H % kBlock || I % kBlock) return MOE_E_ALIGN;
   const int I_sh = shared_w13 ? I_shared : 0;
   // the problem must fit the array: refused here, before anything is launched
@@ -353,7 +361,7 @@ extern "C" int moe_layer_fp8_static(void *stream, const void *x_bf16, int T, int
 
 // The router product on its own: logits [T, E] bf16 = x [T, H] . Wr [E, H]^T (fp32 sums, rounded once).
 extern "C" size_t moe_router_logits_workspace_bytes(int T, int H, int E) {
-  if (T < 0 || H < 1 || E < 1 || E > 256 || H % moe::kBlock) return 0;
+  if (T < 0 || H < 1 || E < 1 || E > MOE_MAX_EXPERTS || H % moe::kBlock) return 0;
   return moe::align_up(moe::router_front_partial_bytes(T, H, E) + 1, 256);
 }
 
@@ -362,7 +370,7 @@ extern "C" int moe_router_logits(void *stream, const void *x_bf16, int T, int H,
   using namespace moe;
   if (!router_w_bf16 || !workspace) return MOE_E_NULL;
   if (T != 0 && (!x_bf16 || !logits_bf16)) return MOE_E_NULL;
-  if (T < 0 || H < 1 || E < 1 || E > 256) return MOE_E_SHAPE;
+  if (T < 0 || H < 1 || E < 1 || E > MOE_MAX_EXPERTS) return MOE_E_SHAPE;
   if (H % kBlock) return MOE_E_ALIGN;
   if (((uintptr_t)workspace % 256) || ((uintptr_t)x_bf16 % 16) || ((uintptr_t)router_w_bf16 % 16)) return MOE_E_ALIGN;
   if (workspace_bytes < moe_router_logits_workspace_bytes(T, H, E)) return MOE_E_WORKSPACE;

@@ -1,9 +1,10 @@
-// A measuring aid, not part of the path: what a pure read of device memory reaches on this GPU, with the
-// decomposition the grouped GEMMs use for their weights - one workgroup of eight wavefronts streams one contiguous
-// piece, 16 bytes per lane and load, eight loads of a lane in flight.  bench.py reports it next to the nominal HBM
-// peak so that a kernel's fraction of the peak can be read against what a kernel that does nothing else reaches.
+// A measuring aid of the benchmark, NOT part of the product library: built into a library of its own
+// (libmoe_bench_probe.so) that only bench.py loads, and declared in no public header.  What a pure read of device
+// memory reaches on this GPU, with the decomposition the grouped GEMMs use for their weights - one workgroup of
+// eight wavefronts streams one contiguous piece, 16 bytes per lane and load, eight loads of a lane in flight.
+// bench.py reports it next to the nominal HBM peak so that a kernel's fraction of the peak can be read against what
+// a kernel that does nothing else reaches.  Returns 0, a negative argument error, or a positive hipError_t.
 #include "moe_common.h"
-#include "../../include/moe_hip.h"
 
 namespace moe {
 
@@ -28,14 +29,14 @@ __global__ __launch_bounds__(512) void hbm_read_probe_kernel(const v4i *__restri
 
 }  // namespace moe
 
-extern "C" int moe_hbm_read_probe(void *stream, const void *buf, size_t bytes, size_t bytes_per_workgroup, void *sink) {
+extern "C" int bench_hbm_read_probe(void *stream, const void *buf, size_t bytes, size_t bytes_per_workgroup, void *sink) {
   using namespace moe;
-  if (!buf || !sink) return MOE_E_NULL;
-  if (((uintptr_t)buf % 16) || ((uintptr_t)sink % 4)) return MOE_E_ALIGN;
-  if (bytes < 16 || bytes % 16 || bytes_per_workgroup < 16 || bytes_per_workgroup % 16) return MOE_E_SHAPE;
+  if (!buf || !sink) return -1;
+  if (((uintptr_t)buf % 16) || ((uintptr_t)sink % 4)) return -3;
+  if (bytes < 16 || bytes % 16 || bytes_per_workgroup < 16 || bytes_per_workgroup % 16) return -2;
   const size_t n_vec = bytes / 16, per = bytes_per_workgroup / 16;
   const size_t blocks = (n_vec + per - 1) / per;
-  if (blocks > 0x7fffffffull) return MOE_E_SHAPE;
+  if (blocks > 0x7fffffffull) return -2;
   hbm_read_probe_kernel<<<(unsigned)blocks, 512, 0, (hipStream_t)stream>>>((const v4i *)buf, n_vec, per, (int *)sink);
   return (int)hipGetLastError();
 }

@@ -341,13 +341,13 @@ int sum_slices_launch(hipStream_t st, const float *partial, int n_slices, int T,
   return (int)hipGetLastError();
 }
 
-// routing straight from the partial sums of the router product (E <= 256: four scores per lane)
+// routing straight from the partial sums of the router product
 // x / H / xq / xs: the activations [T, H] bf16 are quantised in the same launch (xq e4m3fn [T, H], xs fp32 with
 // pitch scale_pitch(H / 128)); x null: routing only.
 int route_from_partials_launch(hipStream_t st, const float *partial, int n_slices, const float *bias, int T, int E, int K,
                                int mode, int n_groups, int topk_groups, int renorm, float scale, float *weights_out,
                                int32_t *ids_out, const uint16_t *x, int H, uint8_t *xq, float *xs) {
-  if (E > 256 || n_slices < 1) return MOE_E_SHAPE;
+  if (n_slices < 1 || n_slices > 8) return MOE_E_SHAPE;
   if (mode != MOE_ROUTE_SOFTMAX && mode != MOE_ROUTE_SIGMOID && mode != MOE_ROUTE_SOFTMAX_LOGIT_BIAS) return MOE_E_MODE;
   const int rc = check_route_shape(T, E, K, n_groups, topk_groups);
   if (rc) return rc;
@@ -365,12 +365,15 @@ int route_from_partials_launch(hipStream_t st, const float *partial, int n_slice
   }
   if (blocks > 0x7fffffffl) return MOE_E_SHAPE;
   dim3 grid((unsigned)blocks), block(256);
-  if (E <= 64)
-    route_topk_kernel<1><<<grid, block, 0, st>>>(partial, 0, bias, T, E, K, mode, n_groups, topk_groups, renorm, scale, weights_out, ids_out, nullptr, n_slices, ride);
-  else if (E <= 128)
-    route_topk_kernel<2><<<grid, block, 0, st>>>(partial, 0, bias, T, E, K, mode, n_groups, topk_groups, renorm, scale, weights_out, ids_out, nullptr, n_slices, ride);
-  else
-    route_topk_kernel<4><<<grid, block, 0, st>>>(partial, 0, bias, T, E, K, mode, n_groups, topk_groups, renorm, scale, weights_out, ids_out, nullptr, n_slices, ride);
+#define MOE_LAUNCH_ROUTE_PARTIALS(P)                                                                               \
+  route_topk_kernel<P><<<grid, block, 0, st>>>(partial, 0, bias, T, E, K, mode, n_groups, topk_groups, renorm, scale, \
+                                               weights_out, ids_out, nullptr, n_slices, ride)
+  if (E <= 64) MOE_LAUNCH_ROUTE_PARTIALS(1);
+  else if (E <= 128) MOE_LAUNCH_ROUTE_PARTIALS(2);
+  else if (E <= 256) MOE_LAUNCH_ROUTE_PARTIALS(4);
+  else if (E <= 512) MOE_LAUNCH_ROUTE_PARTIALS(8);
+  else MOE_LAUNCH_ROUTE_PARTIALS(16);
+#undef MOE_LAUNCH_ROUTE_PARTIALS
   return (int)hipGetLastError();
 }
 

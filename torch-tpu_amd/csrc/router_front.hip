@@ -1,10 +1,10 @@
-// Router logits for batches beyond the decode size: logits[T, E] = x[T, H] . Wr[E, H]^T in bf16 on the matrix
-// cores, E <= 256.
+// Router logits for batches beyond the decode size (and for any batch of a layer with more than 256 experts):
+// logits[T, E] = x[T, H] . Wr[E, H]^T in bf16 on the matrix cores, E <= 1024 in blocks of 256 experts.
 //
 // The product is short and wide (a few thousand tokens by at most 256 experts over a long reduction), so the
 // reduction is cut into slices: workgroup (block of 128 tokens, slice) leaves its fp32 partial sums, and the routing
 // kernel that follows adds the slices in a fixed order, rounds to bf16 (what a bf16 matmul leaves) and routes.
-// Four wavefronts; wavefront w owns experts 64w .. 64w+63 for all 128 tokens (8 x 4 tiles of 16 x 16: with fewer
+// Four wavefronts; wavefront w owns experts 64w .. 64w+63 of the workgroup's block of 256 for all 128 tokens (8 x 4 tiles of 16 x 16: with fewer
 // tokens per workgroup the router rows, re-read by every token block, saturate the L2 -> LDS path before the matrix
 // pipe).  A step is 64 reduction elements = 128 bytes of a row = two v_mfma_f32_16x16x32_bf16 per tile pair.  Both
 // operands travel L2 -> LDS with direct loads, two steps ahead, through three stages: the token tile (shared, one
@@ -31,12 +31,15 @@ __device__ __forceinline__ uint32_t rf_lds_offset(const void *p) { return (uint3
 
 __global__ __launch_bounds__(256) void router_logits_splitk_kernel(const uint8_t *__restrict__ x,
                                                                    const uint8_t *__restrict__ wr, int T, int H, int E,
-                                                                   int n_slices, int blocks_per_slice,
+                                                                   int n_slices, int blocks_per_slice, int n_eblocks,
                                                                    float *__restrict__ partial) {
   __shared__ RfSmem sm;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int li = lane & 15, lg = lane >> 4;
-  const int slice = blockIdx.x % n_slices, m0 = (blockIdx.x / n_slices) * kRfTokens;
+  // workgroup id = ((token block) * n_eblocks + expert block) * n_slices + slice: the workgroups that share a token
+  // block, and then an expert block, are neighbours in launch order
+  const int slice = blockIdx.x % n_slices, eb = (blockIdx.x / n_slices) % n_eblocks, e0 = eb * 256;
+  const int m0 = (blockIdx.x / (n_slices * n_eblocks)) * kRfTokens;
   const int nblk = H >> 7;
   const int b0 = slice * blocks_per_slice, b1 = min(nblk, b0 + blocks_per_slice);
   const int n_steps = 2 * (b1 - b0);                      // steps of 64 elements
@@ -53,7 +56,7 @@ __global__ __launch_bounds__(256) void router_logits_splitk_kernel(const uint8_t
 #pragma unroll
   for (int u = 0; u < NX; u++) x_src[u] = (uint32_t)min(m0 + 8 * (NX * wave + u) + sub, T - 1) * (uint32_t)row_bytes + chunk * 16;
 #pragma unroll
-  for (int u = 0; u < 8; u++) w_src[u] = (uint32_t)min(64 * wave + 8 * u + sub, E - 1) * (uint32_t)row_bytes + chunk * 16;
+  for (int u = 0; u < 8; u++) w_src[u] = (uint32_t)min(e0 + 64 * wave + 8 * u + sub, E - 1) * (uint32_t)row_bytes + chunk * 16;
   const uint32_t x_lds = __builtin_amdgcn_readfirstlane(rf_lds_offset(&sm.x[0][0])) + (NX * wave) * 1024;
   const uint32_t w_lds = __builtin_amdgcn_readfirstlane(rf_lds_offset(&sm.w[0][0])) + (8 * wave) * 1024;
   auto request = [&](int step) {
@@ -107,7 +110,7 @@ __global__ __launch_bounds__(256) void router_logits_splitk_kernel(const uint8_t
                                                               __builtin_bit_cast(v8bf_t, wb[j][h]), acc[i][j], 0, 0, 0);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  // c[r] of tile (i, j): token m0 + 16 i + 4 (l / 16) + r, expert 64 w + 16 j + l % 16
+  // c[r] of tile (i, j): token m0 + 16 i + 4 (l / 16) + r, expert e0 + 64 w + 16 j + l % 16
   float *const out = partial + (size_t)slice * T * E;
 #pragma unroll
   for (int i = 0; i < kRfMT; i++)
@@ -116,15 +119,15 @@ __global__ __launch_bounds__(256) void router_logits_splitk_kernel(const uint8_t
       const int tok = m0 + 16 * i + 4 * lg + r;
 #pragma unroll
       for (int j = 0; j < 4; j++) {
-        const int e = 64 * wave + 16 * j + li;
+        const int e = e0 + 64 * wave + 16 * j + li;
         if (tok < T && e < E) out[(size_t)tok * E + e] = acc[i][j][r];
       }
     }
 }
 
 // how the reduction is cut: enough workgroups for every compute unit, slices of whole 128-column blocks
-void router_front_plan(int T, int H, int *n_slices, int *blocks_per_slice) {
-  const int mblocks = (T + kRfTokens - 1) / kRfTokens, nblk = H / kBlock;
+void router_front_plan(int T, int H, int E, int *n_slices, int *blocks_per_slice) {
+  const int mblocks = (T + kRfTokens - 1) / kRfTokens * ((E + 255) / 256), nblk = H / kBlock;
   int s = (512 + mblocks - 1) / mblocks;
   if (s < 1) s = 1;
   if (s > 8) s = 8;
@@ -137,18 +140,22 @@ void router_front_plan(int T, int H, int *n_slices, int *blocks_per_slice) {
 size_t router_front_partial_bytes(int T, int H, int E) {
   int s, per;
   if (T < 1) return 0;
-  router_front_plan(T, H, &s, &per);
+  router_front_plan(T, H, E, &s, &per);
   return (size_t)s * T * E * 4;
 }
 
 // x [T, H] bf16, wr [E, H] bf16 -> partial [n_slices][T][E] fp32.  The caller has checked pointers and alignment.
 int router_front_launch(hipStream_t st, const void *x, int T, int H, const void *wr, int E, float *partial, int *n_slices_out) {
-  if (T < 1 || E < 1 || E > 256 || H % kBlock) return MOE_E_SHAPE;
-  if ((double)T * H * 2 >= 2147483648.0) return MOE_E_SHAPE;       // per-lane source offsets are 32-bit
+  if (T < 1 || E < 1 || E > MOE_MAX_EXPERTS || H % kBlock) return MOE_E_SHAPE;
+  // per-lane source offsets are 32-bit
+  if ((double)T * H * 2 >= 2147483648.0 || (double)E * H * 2 >= 2147483648.0) return MOE_E_SHAPE;
   int s, per;
-  router_front_plan(T, H, &s, &per);
-  const long blocks = (long)((T + kRfTokens - 1) / kRfTokens) * s;
-  router_logits_splitk_kernel<<<(unsigned)blocks, 256, 0, st>>>((const uint8_t *)x, (const uint8_t *)wr, T, H, E, s, per, partial);
+  router_front_plan(T, H, E, &s, &per);
+  const int n_eblocks = (E + 255) / 256;
+  const long blocks = (long)((T + kRfTokens - 1) / kRfTokens) * n_eblocks * s;
+  if (blocks > 0x7fffffffl) return MOE_E_SHAPE;
+  router_logits_splitk_kernel<<<(unsigned)blocks, 256, 0, st>>>((const uint8_t *)x, (const uint8_t *)wr, T, H, E, s, per,
+                                                                n_eblocks, partial);
   *n_slices_out = s;
   return (int)hipGetLastError();
 }

@@ -94,20 +94,31 @@ def convert_hf_moe_layer(state: dict, prefix: str, num_experts: int, device=None
         t = state[prefix + name]
         return t.to(device) if device is not None else t
 
+    if tile_block and device is None and not state[prefix + "gate.weight"].is_cuda:
+        raise RuntimeError("convert_hf_moe_layer: tile-blocking the weight bytes runs on the GPU - pass device='cuda' "
+                           "(or tile_block=False for the stacked row-major tensors on the host)")
+
     def stack(proj, suffix):
         return torch.stack([get(f"experts.{e}.{proj}.{suffix}") for e in range(num_experts)])
 
-    w13 = torch.cat([stack("gate_proj", "weight"), stack("up_proj", "weight")], dim=1).contiguous()
-    w13_scale = torch.cat([stack("gate_proj", "weight_scale_inv"), stack("up_proj", "weight_scale_inv")],
-                          dim=1).to(torch.float32).contiguous()
-    w2 = stack("down_proj", "weight").contiguous()
-    w2_scale = stack("down_proj", "weight_scale_inv").to(torch.float32).contiguous()
-    for t in (w13, w2):
+    # I or H that 128 does not divide: zero codes up to whole 128-blocks in both dimensions, as stack_expert_weights
+    # does for the reference's argument form (the scale tensors already hold ceil(n/128) blocks)
+    def whole(t):
+        n, k = t.shape[-2:]
+        return _pad_to(t, -(-n // 128) * 128, -(-k // 128) * 128)
+
+    gate, up, down = stack("gate_proj", "weight"), stack("up_proj", "weight"), stack("down_proj", "weight")
+    for t in (gate, up, down):
         if t.dtype != torch.float8_e4m3fn:
             raise RuntimeError("expert weights must be float8_e4m3fn (convert bf16 checkpoints with quant_weight_block128)")
+    w13 = torch.cat([whole(gate), whole(up)], dim=1).contiguous()
+    w13_scale = torch.cat([stack("gate_proj", "weight_scale_inv"), stack("up_proj", "weight_scale_inv")],
+                          dim=1).to(torch.float32).contiguous()
+    w2 = whole(down).contiguous()
+    w2_scale = stack("down_proj", "weight_scale_inv").to(torch.float32).contiguous()
     shared = None
     if prefix + "shared_experts.gate_proj.weight" in state:
-        sg, su, sd = (get(f"shared_experts.{p}.weight") for p in ("gate_proj", "up_proj", "down_proj"))
+        sg, su, sd = (whole(get(f"shared_experts.{p}.weight")) for p in ("gate_proj", "up_proj", "down_proj"))
         sgs, sus, sds = (get(f"shared_experts.{p}.weight_scale_inv") for p in ("gate_proj", "up_proj", "down_proj"))
         shared = (torch.cat([sg, su], 0)[None].contiguous(), torch.cat([sgs, sus], 0)[None].to(torch.float32).contiguous(),
                   sd[None].contiguous(), sds[None].to(torch.float32).contiguous())
@@ -133,7 +144,9 @@ class FusedMoE:
     def __init__(self, router_weight, w13, w13_scale, w2, w2_scale, top_k, mode="softmax", bias=None,
                  n_groups=1, topk_groups=1, renorm=True, scale=1.0, shared=None):
         # w13 / w2 (and the shared expert's) are tile-blocked: ops.pack_weights / pack_expert_weights / convert_hf_moe_layer
-        self.router_weight = router_weight          # [E, H] bf16
+        # [E, H]; the logits are a bf16 product (fp32 sums, rounded once) as in the reference's recipe
+        # (python/regression/test_llm/test_torch_ops.py:440), so a router weight kept in fp32 is rounded once, here
+        self.router_weight = router_weight if router_weight.dtype == torch.bfloat16 else router_weight.to(torch.bfloat16)
         self.w13, self.w13_scale, self.w2, self.w2_scale = w13, w13_scale, w2, w2_scale
         self.top_k, self.mode, self.bias = top_k, mode, bias
         self.n_groups, self.topk_groups, self.renorm, self.scale = n_groups, topk_groups, renorm, scale
@@ -150,11 +163,10 @@ class FusedMoE:
         return self._ws
 
     def route(self, x):
-        logits = torch.matmul(x, self.router_weight.t())           # bf16; the routing kernel widens it
-        bias = self.bias
-        if self.mode == "softmax" and bias is not None:
-            logits, bias = logits + bias, None          # a softmax router's bias is part of the logits
-        return ops.moe_route(logits, self.top_k, self.mode, bias, self.n_groups, self.topk_groups,
+        """The staged road: the router product and the selection as two calls (the kernels the one-call entry point
+        runs for batches beyond the decode size) -> (weights fp32 [T,K], ids int32 [T,K])."""
+        logits = ops.router_logits(x, self.router_weight)
+        return ops.moe_route(logits, self.top_k, self.layer_mode(), self.bias, self.n_groups, self.topk_groups,
                              self.renorm, self.scale)
 
     def experts(self, x, weights, ids, out=None):
@@ -162,7 +174,7 @@ class FusedMoE:
                                      shared=self.shared, workspace=self._workspace(x.shape[0]))
 
     def _one_call(self, T):
-        return ops.layer_eligible(T, self.w13.shape[0], self.top_k) and self.router_weight.dtype == torch.bfloat16
+        return ops.layer_eligible(T, self.w13.shape[0], self.top_k)
 
     def layer_mode(self):
         """The routing mode handed to the one-call entry point: a softmax router's bias is part of the logits."""

@@ -1,38 +1,43 @@
-"""Registers the reference's operator names in the `my_ops` namespace, so that callers written
-against torch-tpu (`torch.ops.my_ops.fused_moe_fused_experts(...)`, positional arguments, caller
-allocated outputs) run unchanged on a ROCm device.
+"""The `my_ops` operator namespace of the reference on a ROCm device, so that callers written against torch-tpu
+(`torch.ops.my_ops.fused_moe_fused_experts(...)`, positional arguments, caller allocated outputs) run unchanged.
 
-Schemas follow the reference's C++ declarations (torch_tpu/csrc/ops/my_ops/ops.hpp:610-676,
-716-722; registered at myOps.cpp:73-77).
+The reference's own MoE ops - fused_moe_fused_experts, fused_moe_fused_experts_v2, noaux_tc_topk,
+fused_moe_grouped_topk - are registered from C++ as the reference registers them (`TORCH_LIBRARY(my_ops, m)` with
+function pointers, torch_tpu/csrc/ops/my_ops/myOps.cpp:29-80; signatures torch_tpu/csrc/ops/my_ops/ops.hpp:610-676,
+716-722): csrc/my_ops.cpp -> libmy_ops_torch.so, which forwards the common call straight to the C ABI.  This module
+loads that library, adds the ops the reference keeps elsewhere or leaves to its callers (the dense W8A16 / W8A8
+layers, the router recipe, the index building, the weight re-layout) as a fragment of the same namespace, and
+implements the rarer forms of the expert op (bf16 weights, other block sizes, ragged sizes, the W8A16 arithmetic)
+that the C++ op hands over to `my_ops::_fused_experts_general`.
 """
 from __future__ import annotations
 
-import weakref
+import os
 
 import torch
+from torch.multiprocessing.reductions import StorageWeakRef
 
 from . import ops
 from .layer import _pad_to, pack_expert_weights
 
-_lib = torch.library.Library("my_ops", "DEF")
+_SHIM = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libmy_ops_torch.so")
+if not os.path.exists(_SHIM):
+    raise ImportError(f"{_SHIM} is missing: build it with `python {os.path.join(os.path.dirname(_SHIM), 'build.py')}` "
+                      "(g++ against the torch headers). There is no fallback registration.")
+torch.ops.load_library(_SHIM)
 
-_EXPERTS_HEAD = ("Tensor(a!) output, Tensor input, Tensor? output_sample, Tensor? input_sample, "
+_lib = torch.library.Library("my_ops", "FRAGMENT")
+
+_EXPERTS_ARGS = ("Tensor output, Tensor input, Tensor? output_sample, Tensor? input_sample, "
                  "Tensor gate_weights, Tensor up_weights, Tensor down_weights, "
                  "Tensor? gate_scales, Tensor? up_scales, Tensor? down_scales, "
                  "Tensor select_experts, Tensor routing_weights, Tensor? num_select_experts, "
-                 "Tensor? select_experts_middle, Tensor? routing_weights_middle, ")
-_EXPERTS_TAIL = ("int blocksize, int num_experts, int num_experts_per_tok, bool use_grouped_topk, "
+                 "Tensor? select_experts_middle, Tensor? routing_weights_middle, "
+                 "int blocksize, int num_experts, int num_experts_per_tok, bool use_grouped_topk, "
                  "int num_expert_group, int topk_group, Tensor? silu, Tensor? sigmoid, Tensor? m0, "
-                 "bool save_mid_res) -> Tensor(a!)")
-
-_lib.define("fused_moe_fused_experts(" + _EXPERTS_HEAD + _EXPERTS_TAIL)
-_lib.define("fused_moe_fused_experts_v2(" + _EXPERTS_HEAD + "Tensor? gather_buffer, Tensor? scatter_buffer, "
-            + _EXPERTS_TAIL)
-_lib.define("noaux_tc_topk(Tensor(a!) values, Tensor(b!) indices, Tensor scores, int n_groups, int topk_groups, "
-            "int top_k) -> Tensor(a!)")
-_lib.define("fused_moe_grouped_topk(Tensor topk_experts_res, Tensor topk_weights_res_bf16, Tensor left_bf16, "
-            "Tensor right_bf16, Tensor topk_weights_res, Tensor left, Tensor right, Tensor max, Tensor matmul_res, "
-            "Tensor softmax_res) -> Tensor")
+                 "bool save_mid_res) -> Tensor")
+# the forms of fused_moe_fused_experts that the C++ op does not run itself (same arguments, same result)
+_lib.define("_fused_experts_general(" + _EXPERTS_ARGS)
 
 # What the reference leaves to its callers or to closed code, as ops of the same namespace: the router recipe
 # (python/regression/test_llm/test_torch_ops.py:440-456), the index building of the expert kernel
@@ -66,6 +71,7 @@ def set_expert_numerics(mode: str) -> None:
     if mode not in ("w8a8", "w8a16"):
         raise ValueError("mode must be 'w8a8' or 'w8a16'")
     _numerics = mode
+    torch.ops.my_ops._set_expert_numerics(0 if mode == "w8a8" else 1)      # the C++ op runs the default mode only
 
 
 def _dequant_bf16(w, s, blocksize=128):
@@ -79,38 +85,47 @@ class _DerivedCache:
     """Tensors derived from a caller's weight tensors (packed / de-quantised copies), kept for as long as the
     sources live.
 
-    An entry belongs to the source tensor OBJECTS: it holds weak references to them, is found through their ids, is
-    valid only while every reference still resolves to the very tensor handed in and address, version counter, shape,
-    stride, dtype and device are what they were, and is dropped by a finaliser the moment one of the sources is
-    freed - so new weights that land on a recycled address never meet an old copy, and a model with many layers keeps
-    one entry per layer (nothing is evicted by count).  An in-place write through `.data` does not move the version
-    counter and cannot be seen from here: call `invalidate_weight_cache()` after such an update (or pack explicitly
-    with pack_expert_weights and call torch_tpu_amd.fused_experts_fp8 / FusedMoE).  The derived copy doubles the weight
-    memory unless the caller drops the originals."""
+    An entry belongs to the STORAGES of the source tensors, not to the Python objects that wrap them (callers
+    re-create those freely: `param.data`, a view made per call, tensors re-wrapped by a framework): it is found through
+    storage, offset, shape, stride, dtype and device of every source, is valid while every storage is alive and the
+    version counters are what they were, and is dropped - the next time the table is touched - once a storage has
+    been freed.  The table holds weak references to the storages, so a freed storage's identity cannot be taken over
+    by a new one while its entry exists: new weights never meet an old copy, whatever address they land on, and a
+    model with many layers keeps one entry per layer (nothing is evicted by count).  An in-place write through
+    `.data` does not move the version counter and cannot be seen from here: call `invalidate_weight_cache()` after
+    such an update (or pack explicitly with pack_expert_weights and call torch_tpu_amd.fused_experts_fp8 /
+    FusedMoE).  The derived copy doubles the weight memory unless the caller drops the originals."""
 
     def __init__(self):
         self._entries = {}
 
     @staticmethod
-    def _signature(tensors):
-        return tuple((t.data_ptr(), t._version, tuple(t.shape), tuple(t.stride()), t.dtype, t.device) for t in tensors)
+    def _identity(t):
+        return (t.untyped_storage()._cdata, t.storage_offset(), tuple(t.shape), tuple(t.stride()), t.dtype, t.device)
+
+    def _purge(self):
+        dead = [k for k, (refs, _, _) in self._entries.items() if any(r.expired() for r in refs)]
+        for k in dead:
+            del self._entries[k]
 
     def get(self, tensors, tag, make):
-        key = (tag,) + tuple(id(t) for t in tensors)
+        key = (tag,) + tuple(self._identity(t) for t in tensors)
+        versions = tuple(t._version for t in tensors)
         entry = self._entries.get(key)
         if entry is not None:
-            refs, sig, value = entry
-            if all(r() is t for r, t in zip(refs, tensors)) and sig == self._signature(tensors):
+            refs, seen, value = entry
+            if seen == versions and not any(r.expired() for r in refs):
                 return value
+        self._purge()
         value = make()
-        drop = lambda _ref, k=key, d=self._entries: d.pop(k, None)
-        self._entries[key] = ([weakref.ref(t, drop) for t in tensors], self._signature(tensors), value)
+        self._entries[key] = ([StorageWeakRef(t.untyped_storage()) for t in tensors], versions, value)
         return value
 
     def clear(self):
         self._entries.clear()
 
     def __len__(self):
+        self._purge()
         return len(self._entries)
 
 
@@ -121,6 +136,7 @@ def invalidate_weight_cache() -> None:
     """Forget every packed / de-quantised copy made for the drop-in ops (needed after weights were overwritten in place
     through `.data`, which no version counter records)."""
     _weights.clear()
+    torch.ops.my_ops._invalidate_weight_cache()
 
 
 def _dense_packed(key_tensors, make, tag="dense"):
@@ -249,10 +265,19 @@ def _padded_io(output, input, Hp, run):
     return output
 
 
+def _w8a16_in_range(*reduction_lengths):
+    """The W8A16 kernels keep a token row's step offsets in 16 bits of bf16 elements: reduction lengths up to 16384.
+    Beyond that the selected arithmetic is not available, and no other arithmetic is substituted silently."""
+    if any(n > 16384 for n in reduction_lengths):
+        raise RuntimeError(f"set_expert_numerics('w8a16') covers reduction lengths up to 16384, got {max(reduction_lengths)}; "
+                           "use the default 'w8a8' arithmetic for this layer")
+
+
 def _run_packed(output, input, w13, w13s, w2, w2s, select_experts, rw):
     T, H = input.shape
     E, I2, _ = w13.shape
     if _numerics == "w8a16":
+        _w8a16_in_range(H, I2 // 2)
         ws = _workspace(input.device, ops.fused_experts_bf16_workspace_bytes(T, H, I2 // 2, E, select_experts.shape[1]))
         ops.fused_experts_w8a16(input, w13, w13s, w2, w2s, select_experts, rw, out=output, workspace=ws)
         return output
@@ -270,23 +295,6 @@ def _run_bf16(output, input, w13, w2, select_experts, routing_weights):
     return output
 
 
-def _fused_experts_v2(output, input, output_sample, input_sample, gate_weights, up_weights, down_weights,
-                      gate_scales, up_scales, down_scales, select_experts, routing_weights, num_select_experts,
-                      select_experts_middle, routing_weights_middle, gather_buffer, scatter_buffer, blocksize,
-                      num_experts, num_experts_per_tok, use_grouped_topk, num_expert_group, topk_group, silu, sigmoid,
-                      m0, save_mid_res):
-    # the scratch tensors of the reference's second implementation are accepted and left untouched
-    return _fused_experts(output, input, output_sample, input_sample, gate_weights, up_weights, down_weights,
-                          gate_scales, up_scales, down_scales, select_experts, routing_weights, num_select_experts,
-                          select_experts_middle, routing_weights_middle, blocksize, num_experts, num_experts_per_tok,
-                          use_grouped_topk, num_expert_group, topk_group, silu, sigmoid, m0, save_mid_res)
-
-
-def _grouped_topk(*args):
-    raise RuntimeError("fused_moe_grouped_topk: the reference's fused router is closed-source, untested and "
-                       "undocumented; use noaux_tc_topk or torch_tpu_amd.moe_route instead")
-
-
 def _moe_route(x, router_weight, bias, mode, top_k, n_group, topk_group, scale, renorm):
     """Router of one layer: logits = x . router_weight^T (bf16, fp32 sums rounded once), then top-k selection and
     weights -> (fp32 weights [T, top_k], int32 ids [T, top_k]).  mode "softmax" | "sigmoid"; bias [E] fp32 takes part in
@@ -294,15 +302,20 @@ def _moe_route(x, router_weight, bias, mode, top_k, n_group, topk_group, scale, 
     if x.dim() != 2 or router_weight.dim() != 2 or x.shape[1] != router_weight.shape[1]:
         raise RuntimeError("x must be [T, H] and router_weight [E, H]")
     E, H = router_weight.shape
-    if x.dtype == torch.bfloat16 and router_weight.dtype == torch.bfloat16 and E <= 256 and H % 128 == 0:
-        ws = _workspace(x.device, ops.router_logits_workspace_bytes(x.shape[0], H, E))
-        logits = ops.router_logits(x.contiguous(), router_weight.contiguous(), workspace=ws)
-    else:
-        logits = torch.matmul(x, router_weight.t()).contiguous()
-        if logits.dtype not in (torch.float32, torch.bfloat16):
-            logits = logits.float()
+    # The product runs in bf16 on the matrix cores (what the reference's recipe computes, test_torch_ops.py:440): a
+    # router weight held in another dtype, or a hidden size that 128 does not divide, is brought into that form once
+    # per weight tensor (zero columns add nothing), the activations per call.
+    Hp = -(-H // 128) * 128
+    if router_weight.dtype != torch.bfloat16 or Hp != H or not router_weight.is_contiguous():
+        (router_weight,) = _dense_packed(
+            (router_weight,), lambda: (torch.nn.functional.pad(router_weight.to(torch.bfloat16), (0, Hp - H)).contiguous(),),
+            "router")
+    if x.dtype != torch.bfloat16 or Hp != H or not x.is_contiguous():
+        x = torch.nn.functional.pad(x.to(torch.bfloat16), (0, Hp - H)).contiguous()
+    ws = _workspace(x.device, ops.router_logits_workspace_bytes(x.shape[0], Hp, E))
+    logits = ops.router_logits(x, router_weight, workspace=ws)
     if mode == "softmax" and bias is not None:
-        logits, bias = (logits.float() + bias), None
+        mode = "softmax_logit_bias"            # a softmax router's bias is part of the logits; the kernel adds it
     return ops.moe_route(logits, top_k, mode, bias, n_group, topk_group, renorm, scale)
 
 
@@ -404,7 +417,8 @@ def _mlp_forward(input, gate_weight, up_weight, down_weight, gate_scale, up_scal
                  ops.pack_weights(_pad_to(as_t(down_weight), Ip, Hp).t().contiguous()),
                  _scales_128(as_t(down_scale), blocksize, I, H).t().contiguous()),
         f"mlp{blocksize}{orient}")
-    if numerics == "w8a16" and Hp <= 16384 and Ip <= 16384:
+    if numerics == "w8a16":
+        _w8a16_in_range(Hp, Ip)
         # the reference's own arithmetic: one expert that every row selects, weights de-quantised in registers
         ids = _zero_ids(input.device, M)
         ws = _workspace(input.device, ops.fused_experts_bf16_workspace_bytes(M, Hp, Ip, 1, 1))
@@ -442,20 +456,18 @@ def _mm_w8a16_dq_forward(input, weight, scale, output, blocksize):
         return done()
     w, ws = _dense_packed((weight, scale), lambda: (ops.pack_weights(_pad_to(weight, Np, Kp).contiguous()),
                                                      _scales_128(scale, blocksize, N, K)), f"mm{blocksize}")
-    if _numerics == "w8a16" and Kp <= 16384:
+    if _numerics == "w8a16":
+        _w8a16_in_range(Kp)
         ops.mm_w8a16(x, w, ws, out=out)
         return done()
     ops.mm_fp8(x, w, ws, out=out, workspace=_workspace(input.device, ops.mm_workspace_bytes(M, Kp, Np)))
     return done()
 
 
-_lib.impl("fused_moe_fused_experts", _fused_experts, "CompositeExplicitAutograd")
+_lib.impl("_fused_experts_general", _fused_experts, "CompositeExplicitAutograd")
 _lib.impl("mlp_w8a16_dq_forward", _mlp_w8a16_dq_forward, "CompositeExplicitAutograd")
 _lib.impl("mlp_w8a8_quant_forward", _mlp_w8a8_quant_forward, "CompositeExplicitAutograd")
 _lib.impl("mm_w8a16_dq_forward", _mm_w8a16_dq_forward, "CompositeExplicitAutograd")
-_lib.impl("fused_moe_fused_experts_v2", _fused_experts_v2, "CompositeExplicitAutograd")
-_lib.impl("noaux_tc_topk", ops.noaux_tc_topk, "CompositeExplicitAutograd")
-_lib.impl("fused_moe_grouped_topk", _grouped_topk, "CompositeExplicitAutograd")
 _lib.impl("moe_route", _moe_route, "CompositeExplicitAutograd")
 _lib.impl("moe_permute", _moe_permute, "CompositeExplicitAutograd")
 _lib.impl("moe_pack_weights", _moe_pack_weights, "CompositeExplicitAutograd")

@@ -170,19 +170,6 @@ def unpack_weights(w):
     return _repack(w, lib.moe_unpack_weights, "unpack_weights")
 
 
-def hbm_read_probe(buf, bytes_per_workgroup: int = 1835008):
-    """Launches one pure read of `buf` (any contiguous GPU tensor whose byte size is a multiple of 16) on the current
-    stream: one workgroup of eight wavefronts per contiguous piece of `bytes_per_workgroup` (default: one weight strip of
-    the DeepSeek-V3 layer's first GEMM, 256 rows x 7168 bytes).  A measuring aid for bench.py; returns nothing."""
-    _need(isinstance(buf, torch.Tensor) and buf.is_cuda and buf.is_contiguous(), "buf must be a contiguous GPU tensor")
-    nbytes = buf.numel() * buf.element_size()
-    _need(nbytes >= 16 and nbytes % 16 == 0 and bytes_per_workgroup >= 16 and bytes_per_workgroup % 16 == 0,
-          "sizes must be multiples of 16 bytes")
-    sink = torch.empty(1, dtype=torch.int32, device=buf.device)
-    rc = lib.moe_hbm_read_probe(_stream(), buf.data_ptr(), nbytes, bytes_per_workgroup, sink.data_ptr())
-    check(rc, "moe_hbm_read_probe")
-
-
 def pack_layer(w13, w13_scale, w2, w2_scale):
     """(w13, w13_scale, w2, w2_scale) with row-major weights on the GPU -> the same with tile-blocked weights."""
     return pack_weights(w13), w13_scale, pack_weights(w2), w2_scale
@@ -255,16 +242,16 @@ def fused_experts_fp8(x, w13, w13_scale, w2, w2_scale, ids, routing_weights=None
 
 
 def layer_eligible(T: int, E: int, K: int) -> bool:
-    """Shapes the one-call entry point takes (layer_fp8): any batch, up to 256 experts."""
-    return T >= 0 and 1 <= K <= E <= 256
+    """Shapes the one-call entry point takes (layer_fp8): any batch, up to 1024 experts."""
+    return T >= 0 and 1 <= K <= E <= 1024
 
 
 def router_logits(x, router_weight, out=None, workspace=None):
-    """logits [T,E] bf16 = x [T,H] bf16 . router_weight [E,H]^T bf16 (fp32 sums, rounded once), E <= 256."""
+    """logits [T,E] bf16 = x [T,H] bf16 . router_weight [E,H]^T bf16 (fp32 sums, rounded once), E <= 1024."""
     _need(x.dim() == 2 and router_weight.dim() == 2 and x.shape[1] == router_weight.shape[1], "x must be [T,H], router_weight [E,H]")
     T, H = x.shape
     E = router_weight.shape[0]
-    _need(E <= 256 and H % 128 == 0, "router_logits takes E <= 256 and H a multiple of 128")
+    _need(E <= 1024 and H % 128 == 0, "router_logits takes E <= 1024 and H a multiple of 128")
     if out is None:
         out = torch.empty(T, E, dtype=torch.bfloat16, device=x.device)
     _need(tuple(out.shape) == (T, E), "out must be [T, E]")
@@ -286,7 +273,7 @@ def layer_workspace_bytes(T, H, I, E, K, I_shared=0) -> int:
 def layer_fp8(x, router_weight, w13, w13_scale, w2, w2_scale, top_k: int, mode: str = "softmax", bias=None,
                      n_groups: int = 1, topk_groups: int = 1, renorm: bool = True, scale: float = 1.0, shared=None,
                      out=None, workspace=None, return_routing: bool = False, static_scratch: bool = False):
-    """Router and experts of one layer in one call (E <= 256).
+    """Router and experts of one layer in one call (E <= 1024).
 
     x [T,H] bf16, router_weight [E,H] bf16, the expert weights as in fused_experts_fp8.  Returns out [T,H] bf16,
     or (out, logits bf16 [T,E], weights fp32 [T,k], ids int32 [T,k]) with return_routing.
@@ -298,7 +285,7 @@ def layer_fp8(x, router_weight, w13, w13_scale, w2, w2_scale, top_k: int, mode: 
     T, H = x.shape
     E, I2, H2 = w13.shape
     I = I2 // 2
-    _need(layer_eligible(T, E, top_k), "layer_fp8 takes E <= 256 and top_k <= E")
+    _need(layer_eligible(T, E, top_k), "layer_fp8 takes E <= 1024 and top_k <= E")
     _need(H2 == H and tuple(w2.shape) == (E, H, I) and tuple(router_weight.shape) == (E, H), "weight shapes do not match x")
     _need(H % 128 == 0 and I % 128 == 0, "H and I must be multiples of 128")
     _need(tuple(w13_scale.shape) == (E, I2 // 128, H // 128), "w13_scale must be [E, 2I/128, H/128]")
