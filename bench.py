@@ -135,6 +135,78 @@ def event_time(fn, iters, warmup=2):
     return e0.elapsed_time(e1) / iters * 1e-3
 
 
+def _sysfs_power_files():
+    import glob
+    base = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*"))
+    if not base:
+        return None
+    hw = base[0]
+    dev_dir = os.path.dirname(os.path.dirname(hw))
+    files = dict(power=os.path.join(hw, "power1_input"), cap=os.path.join(hw, "power1_cap"),
+                 sclk=os.path.join(dev_dir, "pp_dpm_sclk"))
+    return files if all(os.path.exists(f) for f in files.values()) else None
+
+
+def power_sample(fn, seconds=1.0):
+    """Package power and shader clock while `fn` is launched back to back for `seconds`: the driver's own sysfs counters
+    (hwmon power1_input / power1_cap in microwatts, the level of pp_dpm_sclk marked current), polled from a host thread.
+    None when the counters cannot be read.  Why it is here: under the grouped GEMMs the package sits at its power cap
+    and the shader clock falls to what the cap leaves, so a launch takes the time its energy takes at that power - a
+    bound next to the memory and matrix roofs that no schedule of the same work gets around."""
+    import threading
+    files = _sysfs_power_files()
+    if files is None:
+        return None
+
+    def read(path):
+        with open(path) as f:
+            return f.read()
+
+    def sclk_now():
+        for line in read(files["sclk"]).splitlines():
+            if line.rstrip().endswith("*"):
+                return float(line.split(":")[1].lower().replace("mhz", "").replace("*", "").strip())
+        return None
+
+    for _ in range(10):
+        fn()
+    torch.cuda.synchronize()
+    watts, clocks, stop = [], [], [False]
+
+    def poll():
+        while not stop[0]:
+            try:
+                watts.append(float(read(files["power"])) / 1e6)
+                c = sclk_now()
+                if c is not None:
+                    clocks.append(c)
+            except (OSError, ValueError):
+                pass
+            time.sleep(0.05)
+
+    th = threading.Thread(target=poll)
+    th.start()
+    t0, n = time.perf_counter(), 0
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
+        n += 20
+    dt = time.perf_counter() - t0
+    stop[0] = True
+    th.join()
+    # the first readings still average over the time before the load
+    w, c = watts[len(watts) // 3:], clocks[len(clocks) // 3:]
+    if not w:
+        return None
+    try:
+        cap = float(read(files["cap"])) / 1e6
+    except (OSError, ValueError):
+        cap = None
+    return dict(watts=sum(w) / len(w), cap_watts=cap, sclk_mhz=sum(c) / len(c) if c else None, ms_per_launch=dt / n * 1e3,
+                samples=len(w))
+
+
 def bench_prefill(pkg, moe, cfg, dev, steps, warmup):
     T, H, I, E, K = cfg["T"], cfg["H"], cfg["I"], cfg["E"], cfg["K"]
     g = torch.Generator(device=dev).manual_seed(11)
@@ -187,6 +259,9 @@ def bench_prefill(pkg, moe, cfg, dev, steps, warmup):
     probe_gbs = probe_buf.numel() / kp / 1e9
     # the same bytes read by short-lived workgroups of 8 KB each that sweep the buffer front to back
     kf = event_time(lambda: hbm_read_probe(probe_buf, 8192), max(3, steps), warmup=3)
+    # package power and shader clock under each of them (sysfs counters, a second of back-to-back launches each)
+    power = dict(first_gemm=power_sample(gemm1), second_gemm=power_sample(gemm2),
+                 read_probe=power_sample(lambda: hbm_read_probe(probe_buf, probe_piece)), step=power_sample(step))
     touched = int((off[1:] > off[:-1]).sum().item())
     # algorithmic traffic of one launch of the first GEMM: each touched expert's W13 (+scales) once,
     # quantised activations once, re-quantised SwiGLU output once
@@ -211,7 +286,7 @@ def bench_prefill(pkg, moe, cfg, dev, steps, warmup):
                 hbm_gbs=b1 / k1 / 1e9, hbm_frac=b1 / k1 / 1e9 / PEAK_HBM_GBS,
                 second_gemm=dict(launch_ms=k2 * 1e3, mfma_tflops=f2 / k2 / 1e12, hbm_gbs=b2 / k2 / 1e9,
                                  hbm_frac=b2 / k2 / 1e9 / PEAK_HBM_GBS),
-                experts_touched=touched,
+                experts_touched=touched, power=power,
                 read_probe=dict(gbs=probe_gbs, frac_of_peak=probe_gbs / PEAK_HBM_GBS, bytes=probe_buf.numel(),
                                 bytes_per_workgroup=probe_piece, gbs_short_workgroups=probe_buf.numel() / kf / 1e9,
                                 note="a kernel that only reads (bench_hbm_read_probe in libmoe_bench_probe.so), same workgroup "

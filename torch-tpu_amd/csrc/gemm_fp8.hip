@@ -74,7 +74,8 @@ struct GemmArgs {
   int total_blocks;             // launched workgroups (multiple of 8)
   int E;                        // experts (tile_prefix[E] = number of row tiles)
   int fixed_expert;             // >= 0: dense mode, every row belongs to this expert and A row p = p
-  int max_mtiles;               // entries allocated in tile_expert
+  int max_mtiles;               // entries allocated in tile_expert (row tiles of the list's height)
+  int split;                    // row tiles of this kernel per row tile of the list (1, or 2: half tiles)
   // optional shared expert riding in the same launch (same N / Kd as the routed experts): its
   // row tiles follow the routed ones; rows are the tokens in order
   const uint8_t *sh_aq;         // its activations ([sh_rows, Kd]; the token tensor for the first GEMM)
@@ -165,7 +166,8 @@ __device__ __forceinline__ void mma_bf16(v4f (&acc)[WT], const v8i (&w)[WT], con
 // BF16   un-quantised mode: both operands are bf16 (a 128-byte step is 64 elements = two
 //        v_mfma_f32_16x16x32_bf16 accumulating in place), no scales, bf16 intermediate
 template <int MT, int NW, int DEPTH, bool GATED, bool WREG, bool BF16 = false, int TPS = 16, bool DQ = false>
-__global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a) {
+// Four wavefronts with the weights in registers: two such workgroups share a compute unit (256 registers a lane each)
+__global__ __launch_bounds__(64 * NW, (WREG && NW == 4) ? 2 : 1) void grouped_gemm_kernel(const GemmArgs a) {
   static_assert(!DQ || BF16, "de-quantised weights feed the bf16 matrix instructions");
   static_assert(TPS % NW == 0 && (TPS == 16 || (!GATED && !WREG && TPS <= 8)), "narrow strips: second GEMM, operands through LDS");
   constexpr int BM = 16 * MT;
@@ -186,7 +188,9 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
   // has its own L2, works on a contiguous range of the real tiles (their number is only known
   // on the device): neighbours in that range share the token tile and, for experts with more
   // than one row tile, the weight strip.
-  const int n_routed = a.fixed_expert >= 0 ? (a.rows_a + BM - 1) / BM : min(a.tile_prefix[a.E], a.max_mtiles);
+  // The tile list may be coarser than this kernel's row tile (a.split of its tiles per list entry, 192 = 2 x 96): an
+  // entry's tiles follow one another, the ones past the expert's last row exit right away.
+  const int n_routed = a.fixed_expert >= 0 ? (a.rows_a + BM - 1) / BM : min(a.tile_prefix[a.E], a.max_mtiles) * a.split;
   const int n_mtiles = n_routed + (a.sh_rows + BM - 1) / BM;
   // Each XCD takes an equal share of the shared expert's work items (full tiles: the heaviest, so
   // they go first) and then an equal, contiguous share of the routed ones.
@@ -217,12 +221,12 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
     e = a.fixed_expert; first_mtile = 0; n_mt = n_routed;
   } else {
     // one 32-byte record holds everything about the expert this tile belongs to
-    const v4i d0 = *(const v4i *)(a.tile_desc + (size_t)g0 * 8);
-    const v4i d1 = *(const v4i *)(a.tile_desc + (size_t)g0 * 8 + 4);
+    const v4i d0 = *(const v4i *)(a.tile_desc + (size_t)(g0 / a.split) * 8);
+    const v4i d1 = *(const v4i *)(a.tile_desc + (size_t)(g0 / a.split) * 8 + 4);
     e = d0[0];
     if (e < 0 || e >= a.E) return;
-    first_mtile = d0[1];
-    n_mt = min(d0[1] + d0[2], a.max_mtiles) - first_mtile;
+    first_mtile = d0[1] * a.split;
+    n_mt = (min(d0[1] + d0[2], a.max_mtiles) - d0[1]) * a.split;
     e_row0 = d0[3];
     e_rows = d1[0];
   }
@@ -814,19 +818,36 @@ __global__ __launch_bounds__(64 * NW) void grouped_gemm_kernel(const GemmArgs a)
 
 // Launch shape per tile height.  Eight wavefronts (two per SIMD, two weight tiles each) keep
 // more loads in flight for the bandwidth-bound shapes.
+// tile_m: row tile of the tile list (grouped mode) or of this launch (dense mode); routed_tiles: entries of the list
+// (an upper bound known on the host) or row tiles of the dense matrix; mean_rows: rows per expert on average.
 template <bool GATED, bool BF16 = false, bool DQ = false>
-static int launch_gemm(hipStream_t st, GemmArgs &a, int tile_m, int max_mtiles) {
+static int launch_gemm(hipStream_t st, GemmArgs &a, int tile_m, int routed_tiles, double mean_rows) {
   // the kernel keeps one weight-block scale per 128-step in LDS and forms per-lane operand offsets in 32 bits
   if (a.Kd < 128 || a.Kd % 128 || (a.Kd >> 7) > kMaxKB) return MOE_E_SHAPE;
   if ((double)a.rows_a * a.Kd >= 2147483648.0 || (double)a.sh_rows * a.Kd >= 2147483648.0) return MOE_E_SHAPE;
+  // Half tiles: experts with many rows (the launch is bound by the matrix pipes, not by the weight stream) and a
+  // short reduction - a work item's start and end are then as long as its loop.  The 192-row entries of the tile list
+  // are walked as two 96-row tiles each by workgroups of four wavefronts with four weight tiles each (the token
+  // operand is read from LDS once per four matrix instructions instead of two), two workgroups per compute unit, so
+  // that one's start and end hide behind the other's loop.  Measured, Qwen3-shaped layer under the skewed load
+  // (T=16384; 16 and 6 steps): first GEMM 0.522 -> 0.458 ms, second 0.366 -> 0.347; Mixtral shape (32 and 112 steps):
+  // 1.02 -> 1.06 and 0.486 -> 0.579 ms - each row tile re-reads its weight strip from L2, which a long reduction
+  // does not forgive; DeepSeek shape (128 rows per expert, bound by the weight stream): 1.40 -> 1.73 ms.
+  int km = tile_m;                                   // this launch's row tile
+  a.split = 1;
+  if (a.fixed_expert < 0 && tile_m == 192 && (a.Kd >> 7) <= kHalfTileMaxSteps && mean_rows >= 320.0) {
+    km = 96;
+    a.split = 2;
+  }
+  const long row_tiles = (long)routed_tiles * a.split + (a.sh_rows + km - 1) / km;
   // Second GEMM with small row tiles: strips of 64 output columns instead of 256 - four times the workgroups,
   // three of them resident per compute unit, so that one's start and end hide behind the others' streams (and a
   // batch with few experts still reaches every compute unit: a workgroup alone streams at most ~37 GB/s).  The
   // order of every sum is the same.  With 64-row tiles it only pays while the wide strips would leave units idle.
-  const bool narrow = !GATED && (tile_m <= 32 || (tile_m == 64 && (long)max_mtiles * ((a.N + 255) / 256) < 192));
+  const bool narrow = !GATED && (km <= 32 || (km == 64 && row_tiles * ((a.N + 255) / 256) < 192));
   a.n_strips = GATED ? a.N / 128 : narrow ? (a.N + 63) / 64 : (a.N + 255) / 256;
-  a.max_mtiles = max_mtiles - (a.sh_rows + tile_m - 1) / tile_m;
-  long total = (long)max_mtiles * a.n_strips;
+  a.max_mtiles = routed_tiles;
+  long total = row_tiles * a.n_strips;
   total = (total + 7) / 8 * 8 + 16;                  // the per-XCD split rounds two shares up
   if (total <= 0 || total > 0x7fffffffl) return MOE_E_SHAPE;
   a.total_blocks = (int)total;
@@ -837,7 +858,7 @@ static int launch_gemm(hipStream_t st, GemmArgs &a, int tile_m, int max_mtiles) 
   if constexpr (!GATED) {
     if (narrow) {
 #define MOE_GEMM_NARROW(MT, D) grouped_gemm_kernel<MT, 4, D, false, false, BF16, 4, DQ><<<grid, dim3(256), 0, st>>>(a)
-      switch (tile_m) {
+      switch (km) {
         case 16: MOE_GEMM_NARROW(1, 3); break;
         case 32: MOE_GEMM_NARROW(2, 3); break;
         default: MOE_GEMM_NARROW(4, 2); break;
@@ -846,10 +867,11 @@ static int launch_gemm(hipStream_t st, GemmArgs &a, int tile_m, int max_mtiles) 
       return (int)hipGetLastError();
     }
   }
-  switch (tile_m) {
+  switch (km) {
     case 16: MOE_GEMM(1, 8, 3, false); break;
     case 32: MOE_GEMM(2, 8, 3, false); break;
     case 64: MOE_GEMM(4, 8, 2, false); break;
+    case 96: MOE_GEMM(6, 4, 2, true); break;
     case 128: MOE_GEMM(8, 8, 2, true); break;
     case 192: MOE_GEMM(12, 8, 2, true); break;
     default: return MOE_E_SHAPE;
@@ -882,11 +904,14 @@ int gemm1_launch(hipStream_t st, const uint8_t *xq, const float *xs, int T, int 
   a.hq = hq; a.hs = hs; a.y = nullptr;
   a.as_pitch = scale_pitch(H / kBlock); a.hs_pitch = scale_pitch(I / kBlock);
   a.Kd = bf16 ? 2 * H : H; a.N = I; a.n_rows_w = 2 * I; a.rows_a = T; a.topk = K; a.E = E; a.fixed_expert = fixed_expert;
-  const int tile_m = choose_tile_m(T, K, E);
-  const int max_mtiles = fixed_expert >= 0 ? (T + tile_m - 1) / tile_m : pw->max_tiles;
-  if (numerics == kNumericsW8A16) return launch_gemm<true, true, true>(st, a, tile_m, max_mtiles + (a.sh_rows + tile_m - 1) / tile_m);
-  if (bf16) return launch_gemm<true, true>(st, a, tile_m, max_mtiles + (a.sh_rows + tile_m - 1) / tile_m);
-  return launch_gemm<true>(st, a, tile_m, max_mtiles + (a.sh_rows + tile_m - 1) / tile_m);
+  // the dense layers (rows in order, nothing shared with a permutation) size their row tile from the problem at hand
+  const bool dense = fixed_expert >= 0 && T > 128 && !sh_w13;
+  const int tile_m = dense ? choose_dense_tile_m(T, I / kBlock, a.Kd >> 7) : choose_tile_m(T, K, E);
+  const int routed_tiles = fixed_expert >= 0 ? (T + tile_m - 1) / tile_m : pw->max_tiles;
+  const double mean_rows = (double)T * K / E;
+  if (numerics == kNumericsW8A16) return launch_gemm<true, true, true>(st, a, tile_m, routed_tiles, mean_rows);
+  if (bf16) return launch_gemm<true, true>(st, a, tile_m, routed_tiles, mean_rows);
+  return launch_gemm<true>(st, a, tile_m, routed_tiles, mean_rows);
 }
 
 int gemm2_launch(hipStream_t st, const uint8_t *hq, const float *hs, int rows_a, int T, int H, const uint8_t *w2,
@@ -903,11 +928,13 @@ int gemm2_launch(hipStream_t st, const uint8_t *hq, const float *hs, int rows_a,
   a.hq = nullptr; a.hs = nullptr; a.y = y;
   a.as_pitch = scale_pitch(I / kBlock); a.hs_pitch = 0;
   a.Kd = bf16 ? 2 * I : I; a.N = H; a.n_rows_w = H; a.rows_a = rows_a; a.topk = K; a.E = E; a.fixed_expert = fixed_expert;
-  const int tile_m = choose_tile_m(T, K, E);
-  const int max_mtiles = fixed_expert >= 0 ? (rows_a + tile_m - 1) / tile_m : pw->max_tiles;
-  if (numerics == kNumericsW8A16) return launch_gemm<false, true, true>(st, a, tile_m, max_mtiles + (a.sh_rows + tile_m - 1) / tile_m);
-  if (bf16) return launch_gemm<false, true>(st, a, tile_m, max_mtiles + (a.sh_rows + tile_m - 1) / tile_m);
-  return launch_gemm<false>(st, a, tile_m, max_mtiles + (a.sh_rows + tile_m - 1) / tile_m);
+  const bool dense = fixed_expert >= 0 && rows_a > 128 && !sh_w2;
+  const int tile_m = dense ? choose_dense_tile_m(rows_a, (H + 255) / 256, a.Kd >> 7) : choose_tile_m(T, K, E);
+  const int routed_tiles = fixed_expert >= 0 ? (rows_a + tile_m - 1) / tile_m : pw->max_tiles;
+  const double mean_rows = (double)rows_a / E;
+  if (numerics == kNumericsW8A16) return launch_gemm<false, true, true>(st, a, tile_m, routed_tiles, mean_rows);
+  if (bf16) return launch_gemm<false, true>(st, a, tile_m, routed_tiles, mean_rows);
+  return launch_gemm<false>(st, a, tile_m, routed_tiles, mean_rows);
 }
 
 }  // namespace moe

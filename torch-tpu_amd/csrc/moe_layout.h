@@ -40,6 +40,33 @@ static inline int choose_tile_m(int T, int K, int E) {
   return mean > 104.0 ? 192 : 128;
 }
 
+// Row tile of the dense layers (one "expert" owns every row; M > 128 rows, `items_per_row_tile` strips of the output,
+// `steps` 128-steps of the reduction).  Nothing is read from HBM more than once here and the matrix fits the caches,
+// so what counts is how the work items fill the 256 compute units and what one item costs: a model instead of a
+// table - rounds of work items x (steps x (cost of a step, which grows with the tile's m-tiles) + the item's fixed
+// start and end).  Shader cycles measured with the operands coming from L2: a step costs about 300 + 150 per m-tile,
+// start and end of an item about 20 000; the 96-row kernel runs two workgroups per unit (512 items per round), one
+// hiding the other's start and end, which pays while the reduction is short (kHalfTileMaxSteps).
+// Example: 4096 x 7168 -> 1536 (6 strips of 256 columns): 192 rows = 132 items, half the units idle, 56 steps x 2100
+// cycles; 128 rows = 192 items x 56 x 1500, a third less.
+constexpr int kHalfTileMaxSteps = 20;
+static inline int choose_dense_tile_m(long rows, int items_per_row_tile, int steps) {
+  int best = 192;
+  double best_cost = 0.0;
+  const int tiles[4] = {192, 128, 96, 64};
+  for (int i = 0; i < 4; i++) {
+    const int tm = tiles[i];
+    if (tm == 96 && steps > kHalfTileMaxSteps) continue;
+    const long items = (rows + tm - 1) / tm * (long)items_per_row_tile;
+    const long per_round = tm == 96 ? 512 : 256;
+    const long rounds = (items + per_round - 1) / per_round;
+    const double item = (double)steps * (300.0 + 150.0 * (tm / 16)) + (tm == 96 ? 10000.0 : 20000.0);
+    const double cost = (double)rounds * item * (tm == 96 ? 2.0 : 1.0);      // two resident workgroups share a unit
+    if (i == 0 || cost < best_cost * 0.97) { best = tm; best_cost = cost; }     // near-ties go to the taller tile
+  }
+  return best;
+}
+
 struct PermuteWs {
   int32_t *chunk_counts;   // [n_chunks, E]
   int32_t *tile_prefix;    // [E + 1] first tile of each expert; [E] = number of tiles
