@@ -135,6 +135,25 @@ def event_time(fn, iters, warmup=2):
     return e0.elapsed_time(e1) / iters * 1e-3
 
 
+_MFMA_PROBE = None
+
+
+def mfma_probe(workgroups, iters, out):
+    """Launches the matrix-instruction yardstick of libmoe_bench_probe.so (FP8 matrix instructions on register operands
+    and nothing else); returns the operations one launch performs."""
+    global _MFMA_PROBE
+    import ctypes
+    if _MFMA_PROBE is None:
+        _MFMA_PROBE = ctypes.CDLL(os.path.join(ROOT, "torch-tpu_amd", "libmoe_bench_probe.so")).bench_mfma_probe
+        _MFMA_PROBE.restype = ctypes.c_int
+        _MFMA_PROBE.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    assert out.numel() >= workgroups * 512 and out.dtype == torch.float32
+    rc = _MFMA_PROBE(torch.cuda.current_stream(out.device).cuda_stream, workgroups, iters, out.data_ptr())
+    if rc != 0:
+        raise RuntimeError(f"bench_mfma_probe: code {rc}")
+    return workgroups * 8 * iters * 8 * 2.0 * 16 * 16 * 128
+
+
 def _sysfs_power_files():
     import glob
     base = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*"))
@@ -207,6 +226,29 @@ def power_sample(fn, seconds=1.0):
                 samples=len(w))
 
 
+def power_roof(power, nbytes, flops, probe_bytes):
+    """The roof the package power cap sets for one launch that must move `nbytes` through HBM and perform `flops` FP8
+    matrix operations: energy of the two at the rates measured in this very run (watts above idle per TB/s under the
+    read probe, per PFLOP/s under the matrix-instruction probe) over the power the cap leaves above idle.  A launch
+    cannot take less time than that whatever its schedule; what it takes beyond is the energy of everything else it
+    does (operand traffic through L2 and LDS, vector instructions) plus time it is not limited by power at all."""
+    need = ("read_probe", "matrix_instructions_only", "first_gemm")
+    if power is None or any(power.get(k) is None for k in need) or "idle_watts" not in power:
+        return None
+    idle, cap = power["idle_watts"], power["first_gemm"]["cap_watts"]
+    if not cap or cap <= idle:
+        return None
+    probe_tbs = probe_bytes / (power["read_probe"]["ms_per_launch"] * 1e-3) / 1e12
+    w_per_tbs = (power["read_probe"]["watts"] - idle) / probe_tbs
+    w_per_pflops = (power["matrix_instructions_only"]["watts"] - idle) / (power["matrix_instructions_only"]["tflops"] / 1e3)
+    joules = nbytes / 1e12 * w_per_tbs + flops / 1e15 * w_per_pflops
+    return dict(idle_watts=idle, cap_watts=cap, watts_per_tb_per_s=w_per_tbs, watts_per_pflop_per_s=w_per_pflops,
+                joules_hbm=nbytes / 1e12 * w_per_tbs, joules_matrix=flops / 1e15 * w_per_pflops,
+                floor_ms=joules / (cap - idle) * 1e3,
+                measured_ms=power["first_gemm"]["ms_per_launch"], measured_watts=power["first_gemm"]["watts"],
+                note="first grouped GEMM: the time its HBM bytes and matrix operations alone take at the package power cap")
+
+
 def bench_prefill(pkg, moe, cfg, dev, steps, warmup):
     T, H, I, E, K = cfg["T"], cfg["H"], cfg["I"], cfg["E"], cfg["K"]
     g = torch.Generator(device=dev).manual_seed(11)
@@ -262,6 +304,23 @@ def bench_prefill(pkg, moe, cfg, dev, steps, warmup):
     # package power and shader clock under each of them (sysfs counters, a second of back-to-back launches each)
     power = dict(first_gemm=power_sample(gemm1), second_gemm=power_sample(gemm2),
                  read_probe=power_sample(lambda: hbm_read_probe(probe_buf, probe_piece)), step=power_sample(step))
+    # and under nothing but FP8 matrix instructions: the matrix roof of this GPU under its power cap
+    mfma_out = torch.empty(1024 * 512, dtype=torch.float32, device=dev)
+    mfma_ops = mfma_probe(1024, 2000, mfma_out)
+    power["matrix_instructions_only"] = power_sample(lambda: mfma_probe(1024, 2000, mfma_out))
+    if power["matrix_instructions_only"] is not None:
+        power["matrix_instructions_only"]["tflops"] = mfma_ops / (power["matrix_instructions_only"]["ms_per_launch"] * 1e-3) / 1e12
+    # with the GPU left alone for two seconds: what the package draws whatever runs
+    torch.cuda.synchronize()
+    time.sleep(2.0)
+    files = _sysfs_power_files()
+    if files is not None and power["read_probe"] is not None and power["matrix_instructions_only"] is not None:
+        idle = []
+        for _ in range(10):
+            with open(files["power"]) as f:
+                idle.append(float(f.read()) / 1e6)
+            time.sleep(0.05)
+        power["idle_watts"] = sum(idle) / len(idle)
     touched = int((off[1:] > off[:-1]).sum().item())
     # algorithmic traffic of one launch of the first GEMM: each touched expert's W13 (+scales) once,
     # quantised activations once, re-quantised SwiGLU output once
@@ -286,7 +345,7 @@ def bench_prefill(pkg, moe, cfg, dev, steps, warmup):
                 hbm_gbs=b1 / k1 / 1e9, hbm_frac=b1 / k1 / 1e9 / PEAK_HBM_GBS,
                 second_gemm=dict(launch_ms=k2 * 1e3, mfma_tflops=f2 / k2 / 1e12, hbm_gbs=b2 / k2 / 1e9,
                                  hbm_frac=b2 / k2 / 1e9 / PEAK_HBM_GBS),
-                experts_touched=touched, power=power,
+                experts_touched=touched, power=power, power_roof=power_roof(power, b1, f1, probe_buf.numel()),
                 read_probe=dict(gbs=probe_gbs, frac_of_peak=probe_gbs / PEAK_HBM_GBS, bytes=probe_buf.numel(),
                                 bytes_per_workgroup=probe_piece, gbs_short_workgroups=probe_buf.numel() / kf / 1e9,
                                 note="a kernel that only reads (bench_hbm_read_probe in libmoe_bench_probe.so), same workgroup "
