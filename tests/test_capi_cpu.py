@@ -121,6 +121,10 @@ def test_my_ops_are_registered_with_reference_arity(pkg):
     assert len(ops.moe_route.default._schema.arguments) == 9
     assert len(ops.moe_permute.default._schema.arguments) == 2
     assert len(ops.moe_pack_weights.default._schema.arguments) == 6
+    # the reference's own names come from the C++ extension (function-pointer registration: unnamed arguments)
+    assert ops.fused_moe_fused_experts.default._schema.arguments[0].name == "_0"
+    assert len(ops.enable_profile.default._schema.arguments) == 2           # ops.hpp:688-691
+    assert len(ops.disable_profile.default._schema.arguments) == 0
     with pytest.raises(RuntimeError, match="closed-source"):
         ops.fused_moe_grouped_topk(*[torch.zeros(1)] * 10)
     z = torch.zeros(1, 1, 128, dtype=torch.bfloat16)
@@ -264,3 +268,20 @@ def test_bench_hands_on_the_offline_traffic_only_for_the_profiled_sources():
         assert got is None and "stale" in why
     other, why2 = bench.offline_traffic((1, 2, 3, 4, 5))
     assert other is None and "another workload" in why2
+
+
+def test_host_side_layout_arithmetic_under_address_and_undefined_behaviour_sanitizers(tmp_path):
+    """The library's host-only arithmetic (workspace layout, tile heights, the bound on the tile list) built on its
+    own with g++ -fsanitize=address,undefined and run here: every piece of the layout is written through, every
+    bound is checked on extreme loads (tests/host_layout_check.cpp)."""
+    import shutil
+    import subprocess
+    if shutil.which("g++") is None:
+        pytest.skip("no g++")
+    exe = tmp_path / "host_layout_check"
+    src = os.path.join(ROOT, "tests", "host_layout_check.cpp")
+    r = subprocess.run(["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
+                        "-static-libasan", src, "-o", str(exe)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert r.returncode == 0, r.stdout[-3000:]
+    r = subprocess.run([str(exe)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+    assert r.returncode == 0 and "host layout checks passed" in r.stdout, r.stdout[-3000:]

@@ -537,6 +537,16 @@ def test_my_ops_registered_from_cpp_keeps_one_packed_copy_per_weight_set(pkg, or
     assert ops._packed_weight_sets() == 1          # the entries whose gate storage is gone were dropped on the way
     pkg.invalidate_weight_cache()
     assert ops._packed_weight_sets() == 0
+    # enable_profile / disable_profile (torch_tpu/csrc/ops/my_ops/profile.cpp:12-44): GPU time per op between the two
+    ops.enable_profile(2, 0)                     # at most two calls recorded, nothing printed
+    for _ in range(3):
+        ops.fused_moe_fused_experts(out2, x, None, None, gate2, up, down, gs, us, ds, ids, w16, *tail)
+    ops.disable_profile()
+    report = ops._profile_report()
+    line = [l for l in report.splitlines() if l.startswith("fused_moe_fused_experts,")]
+    assert len(line) == 1 and int(line[0].split(",")[1]) == 2 and float(line[0].split(",")[2]) > 0.0, report
+    ops.fused_moe_fused_experts(out2, x, None, None, gate2, up, down, gs, us, ds, ids, w16, *tail)      # off again
+    pkg.invalidate_weight_cache()
     with pytest.raises(RuntimeError, match="do not match"):
         ops.fused_moe_fused_experts(out, x, None, None, gate2, up, down, gs, us, ds, ids, w16, None, None, None, 128, E + 1,
                                     K, False, 1, 1, None, None, None, False)

@@ -41,7 +41,7 @@ def build_shim(verbose=True):
            f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
            "-I" + os.path.join(tdir, "include"), "-I" + os.path.join(tdir, "include", "torch", "csrc", "api", "include"),
            "-I/opt/rocm/include", os.path.join(CSRC, SHIM_SOURCE), "-o", SHIM_LIB,
-           "-L" + os.path.join(tdir, "lib"), "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-L" + HERE, "-lmoe_hip",
+           "-L" + os.path.join(tdir, "lib"), "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-lamdhip64", "-L" + HERE, "-lmoe_hip",
            "-Wl,-rpath,$ORIGIN"]
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:

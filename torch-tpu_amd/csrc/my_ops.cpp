@@ -13,11 +13,15 @@
 #include <ATen/ATen.h>
 #include <ATen/core/dispatch/Dispatcher.h>
 #include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime_api.h>
 #include <torch/library.h>
 
+#include <cstdio>
 #include <map>
 #include <mutex>
 #include <optional>
+#include <sstream>
+#include <string>
 #include <vector>
 
 #include "../../include/moe_hip.h"
@@ -123,6 +127,40 @@ Tensor &scratch(std::map<std::pair<int, void *>, Tensor> &table, const Tensor &l
   return t;
 }
 
+// ---- enable_profile / disable_profile (torch_tpu/csrc/ops/my_ops/profile.cpp:12-44) --------------------------------
+// While enabled, every op of this file brackets its work on the stream with a pair of events; disable_profile waits
+// for them and reports GPU time per op (count, total, mean, min, max).  At most `max_record_num` calls are recorded.
+struct ProfileRecord {
+  const char *op;
+  hipEvent_t start, stop;
+};
+bool g_profiling = false;
+int64_t g_profile_max = 0, g_profile_mode = 0;
+std::vector<ProfileRecord> g_profile;
+std::string g_profile_report;
+
+struct ProfileScope {
+  hipEvent_t stop = nullptr;
+  void *stream = nullptr;
+  // call with g_mutex held
+  ProfileScope(const char *op, void *st) {
+    if (!g_profiling || (int64_t)g_profile.size() >= g_profile_max) return;
+    ProfileRecord r{op, nullptr, nullptr};
+    if (hipEventCreate(&r.start) != hipSuccess) return;
+    if (hipEventCreate(&r.stop) != hipSuccess) {
+      (void)hipEventDestroy(r.start);
+      return;
+    }
+    (void)hipEventRecord(r.start, (hipStream_t)st);
+    stop = r.stop;
+    stream = st;
+    g_profile.push_back(r);
+  }
+  ~ProfileScope() {
+    if (stop) (void)hipEventRecord(stop, (hipStream_t)stream);
+  }
+};
+
 Tensor call_general(const char *name, std::vector<c10::IValue> stack) {
   auto op = c10::Dispatcher::singleton().findSchema({name, ""});
   TORCH_CHECK(op.has_value(), name, " is not defined: this form of the op is implemented by the Python package "
@@ -193,6 +231,7 @@ Tensor fused_moe_fused_experts(const Tensor &output, const Tensor &input, const 
 
   std::lock_guard<std::mutex> lock(g_mutex);
   void *st = stream_of(input);
+  ProfileScope prof("fused_moe_fused_experts", st);
   const PackedEntry &w = packed_weights(gate_weights, up_weights, down_weights, *gate_scales, *up_scales, *down_scales);
   const float *rw = nullptr;
   if (out_mode) {
@@ -254,6 +293,8 @@ Tensor noaux_tc_topk(const Tensor &values, const Tensor &indices, const Tensor &
               "scores must be float32 or bfloat16");
   for (const Tensor *t : {&values, &indices, &scores})
     TORCH_CHECK(t->is_cuda() && t->is_contiguous(), "tensors must be contiguous and on the GPU");
+  std::lock_guard<std::mutex> lock(g_mutex);
+  ProfileScope prof("noaux_tc_topk", stream_of(scores));
   check_rc(moe_noaux_tc_topk(stream_of(scores), scores.data_ptr(),
                              scores.scalar_type() == at::kFloat ? MOE_DTYPE_F32 : MOE_DTYPE_BF16, (int)T, (int)E,
                              (int)n_groups, (int)topk_groups, (int)top_k, values.data_ptr(), indices.data_ptr<int32_t>()),
@@ -266,6 +307,54 @@ Tensor fused_moe_grouped_topk(const Tensor &, const Tensor &, const Tensor &, co
                               const Tensor &, const Tensor &, const Tensor &, const Tensor &, const Tensor &) {
   TORCH_CHECK(false, "fused_moe_grouped_topk: the reference's fused router is closed-source, untested and undocumented; "
               "use noaux_tc_topk or torch_tpu_amd.moe_route instead");
+}
+
+void enable_profile(std::optional<int64_t> max_record_num, std::optional<int64_t> mode) {
+  std::lock_guard<std::mutex> lock(g_mutex);
+  for (auto &r : g_profile) {
+    (void)hipEventDestroy(r.start);
+    (void)hipEventDestroy(r.stop);
+  }
+  g_profile.clear();
+  g_profile_max = max_record_num.value_or(40960);          // the reference's defaults (profile.cpp:17-18)
+  g_profile_mode = mode.value_or(1);
+  TORCH_CHECK(g_profile_max >= 0, "max_record_num must not be negative");
+  g_profiling = true;
+}
+
+void disable_profile() {
+  std::lock_guard<std::mutex> lock(g_mutex);
+  g_profiling = false;
+  struct Sum {
+    int64_t n = 0;
+    double total = 0, lo = 1e300, hi = 0;
+  };
+  std::map<std::string, Sum> per_op;
+  for (auto &r : g_profile) {
+    float ms = 0.f;
+    if (hipEventSynchronize(r.stop) == hipSuccess && hipEventElapsedTime(&ms, r.start, r.stop) == hipSuccess) {
+      Sum &s = per_op[r.op];
+      s.n++;
+      s.total += ms * 1e3;
+      s.lo = std::min(s.lo, (double)ms * 1e3);
+      s.hi = std::max(s.hi, (double)ms * 1e3);
+    }
+    (void)hipEventDestroy(r.start);
+    (void)hipEventDestroy(r.stop);
+  }
+  g_profile.clear();
+  std::ostringstream os;
+  os << "my_ops profile: op, calls, total us, mean us, min us, max us\n";
+  for (auto &kv : per_op)
+    os << kv.first << ", " << kv.second.n << ", " << kv.second.total << ", " << kv.second.total / kv.second.n << ", "
+       << kv.second.lo << ", " << kv.second.hi << "\n";
+  g_profile_report = os.str();
+  if (g_profile_mode != 0) std::fputs(g_profile_report.c_str(), stdout);
+}
+
+std::string _profile_report() {
+  std::lock_guard<std::mutex> lock(g_mutex);
+  return g_profile_report;
 }
 
 // housekeeping for the Python package: the arithmetic switch and the packed-copy table
@@ -290,6 +379,9 @@ TORCH_LIBRARY(my_ops, m) {
   m.def("fused_moe_fused_experts", fused_moe_fused_experts);
   m.def("fused_moe_fused_experts_v2", fused_moe_fused_experts_v2);
   m.def("noaux_tc_topk", noaux_tc_topk);
+  m.def("enable_profile", enable_profile);
+  m.def("disable_profile", disable_profile);
+  m.def("_profile_report", _profile_report);
   m.def("_set_expert_numerics", _set_expert_numerics);
   m.def("_invalidate_weight_cache", _invalidate_weight_cache);
   m.def("_packed_weight_sets", _packed_weight_sets);
