@@ -412,7 +412,8 @@ def bench_decode(pkg, moe, cfg, dev, steps, warmup, batches=(1, 8, 32)):
                         hbm_frac=avg_bytes / sec / 1e9 / PEAK_HBM_GBS, experts_touched_avg=sum(touched) / len(touched),
                         algorithmic_bytes=avg_bytes, launch_mode="hip_graph" if use_graph else "eager",
                         ms_per_step_eager=sec_eager * 1e3,
-                        ms_per_step_hip_graph=None if sec_graph is None else sec_graph * 1e3))
+                        ms_per_step_hip_graph=None if sec_graph is None else sec_graph * 1e3,
+                        power=power_sample(step, 1.0)))       # package power and shader clock under this step
     return res
 
 
