@@ -285,3 +285,24 @@ def test_host_side_layout_arithmetic_under_address_and_undefined_behaviour_sanit
     assert r.returncode == 0, r.stdout[-3000:]
     r = subprocess.run([str(exe)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
     assert r.returncode == 0 and "host layout checks passed" in r.stdout, r.stdout[-3000:]
+
+
+def test_bench_refuses_more_than_one_gpu_and_its_power_roof_is_plain_arithmetic():
+    """bench.py measures one GPU: `--gpus 2` exits with a message before anything touches a device.  The roof the power
+    cap sets is energy over power: checked on hand numbers."""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], stdout=subprocess.PIPE,
+                       stderr=subprocess.PIPE, text=True, timeout=300)
+    assert r.returncode == 2 and "ONE GPU" in r.stderr
+    sys.path.insert(0, ROOT)
+    import bench
+    power = dict(read_probe=dict(watts=1100.0, ms_per_launch=1.0), first_gemm=dict(watts=1400.0, cap_watts=1400.0, ms_per_launch=1.5),
+                 matrix_instructions_only=dict(watts=1300.0, tflops=4000.0), idle_watts=300.0)
+    # probe: 6e12 bytes/s at 800 W above idle; matrix probe: 4 PFLOP/s at 1000 W above idle
+    roof = bench.power_roof(power, nbytes=6.0e9, flops=2.0e12, probe_bytes=6.0e9)
+    assert abs(roof["watts_per_tb_per_s"] - 800.0 / 6.0) < 1e-9 and abs(roof["watts_per_pflop_per_s"] - 250.0) < 1e-9
+    assert abs(roof["joules_hbm"] - 0.8) < 1e-9 and abs(roof["joules_matrix"] - 0.5) < 1e-9
+    assert abs(roof["floor_ms"] - 1.3 / 1100.0 * 1e3) < 1e-9
+    assert bench.power_roof(dict(power, idle_watts=1500.0), 1, 1, 1) is None           # a cap below idle: no roof
+    assert bench.power_roof(dict(power, read_probe=None), 1, 1, 1) is None             # counters unreadable

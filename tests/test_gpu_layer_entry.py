@@ -438,3 +438,27 @@ def test_layer_entry_point_with_more_than_256_experts(pkg, oracle, dev, checks, 
     rep = checks.check_sample(pkg, oracle, x[pick].contiguous(), ids[pick].contiguous(), ld, w_s=w[pick].contiguous(),
                               out_big=out[pick].contiguous(), what=f"E={E}")
     say("   ", rep)
+
+
+def test_module_form_holds_its_weights_as_buffers(pkg, oracle, dev):
+    """FusedMoEModule: the nn.Module shape the reference's tests give their wrapper (test_moe.py:143-160).  Its buffers
+    travel through state_dict / load_state_dict, and forward equals the plain class bit for bit."""
+    say("nn.Module form")
+    T, H, I, E, K = 20, 512, 256, 16, 4
+    ld = pkg.pack_layer(*(t.to(dev) for t in oracle.make_layer(E, H, I, seed=3)))
+    sh = pkg.pack_layer(*(t.to(dev) for t in oracle.make_layer(1, H, I, seed=4)))
+    g = torch.Generator().manual_seed(8)
+    wr = (torch.randn(E, H, generator=g) * 0.05).to(dev)                          # fp32: rounded to bf16 once
+    bias = (torch.randn(E, generator=g) * 0.1).to(dev)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+    mod = pkg.FusedMoEModule(wr, *ld, top_k=K, mode="sigmoid", bias=bias, n_groups=4, topk_groups=2, scale=2.5, shared=sh)
+    ref = pkg.FusedMoE(wr, *ld, top_k=K, mode="sigmoid", bias=bias, n_groups=4, topk_groups=2, scale=2.5, shared=sh)
+    out = mod(x)
+    assert torch.equal(out.view(torch.int16), ref(x).view(torch.int16))
+    state = mod.state_dict()
+    assert {"router_weight", "w13", "w13_scale", "w2", "w2_scale", "bias", "shared_w13", "shared_w2"} <= set(state)
+    other = pkg.FusedMoEModule(torch.zeros_like(wr), *(torch.zeros_like(t) for t in ld), top_k=K, mode="sigmoid",
+                               bias=torch.zeros_like(bias), n_groups=4, topk_groups=2, scale=2.5,
+                               shared=tuple(torch.zeros_like(t) for t in sh))
+    other.load_state_dict(state)
+    assert torch.equal(other(x).view(torch.int16), out.view(torch.int16))

@@ -188,3 +188,36 @@ class FusedMoE:
                                         self.scale, shared=self.shared, out=out, workspace=self._workspace(T, True))
         weights, ids = self.route(x)
         return self.experts(x, weights, ids, out)
+
+
+class FusedMoEModule(torch.nn.Module):
+    """FusedMoE as a torch.nn.Module, the shape the reference's tests give their wrapper around the op
+    (python/regression/test_llm/test_moe.py:143-160): the packed weights are buffers (so `.to(device)`, `state_dict()` and
+    `load_state_dict()` see them), `forward(x)` = router -> experts (+ shared expert) -> [T, H] bf16.  Inference only."""
+
+    def __init__(self, router_weight, w13, w13_scale, w2, w2_scale, top_k, mode="softmax", bias=None, n_groups=1,
+                 topk_groups=1, renorm=True, scale=1.0, shared=None):
+        super().__init__()
+        self.register_buffer("router_weight", router_weight if router_weight.dtype == torch.bfloat16
+                             else router_weight.to(torch.bfloat16))
+        for name, t in (("w13", w13), ("w13_scale", w13_scale), ("w2", w2), ("w2_scale", w2_scale)):
+            self.register_buffer(name, t)
+        self.register_buffer("bias", bias)
+        for i, name in enumerate(("shared_w13", "shared_w13_scale", "shared_w2", "shared_w2_scale")):
+            self.register_buffer(name, None if shared is None else shared[i])
+        self.top_k, self.mode = top_k, mode
+        self.n_groups, self.topk_groups, self.renorm, self.scale = n_groups, topk_groups, renorm, scale
+        self._impl = None
+
+    def _moe(self):
+        m = self._impl
+        if m is None or m.w13.data_ptr() != self.w13.data_ptr():          # built late: `.to(device)` replaces the buffers
+            shared = None if self.shared_w13 is None else (self.shared_w13, self.shared_w13_scale, self.shared_w2,
+                                                           self.shared_w2_scale)
+            m = self._impl = FusedMoE(self.router_weight, self.w13, self.w13_scale, self.w2, self.w2_scale, self.top_k,
+                                      self.mode, self.bias, self.n_groups, self.topk_groups, self.renorm, self.scale, shared)
+        return m
+
+    @torch.no_grad()
+    def forward(self, x):
+        return self._moe()(x)
