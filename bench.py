@@ -661,9 +661,15 @@ def main():
                           step_hbm_frac=step_bytes / sec / 1e9 / PEAK_HBM_GBS,
                           first_gemm_alone_ms=roof["launch_ms"], second_gemm_alone_ms=roof["second_gemm"]["launch_ms"],
                           rest_ms=sec * 1e3 - roof["launch_ms"] - roof["second_gemm"]["launch_ms"],
+                          power_floor_ms=None if not roof.get("power_roof") else
+                          (step_bytes / 1e12 * roof["power_roof"]["watts_per_tb_per_s"]
+                           + flops / 1e15 * roof["power_roof"]["watts_per_pflop_per_s"])
+                          / (roof["power_roof"]["cap_watts"] - roof["power_roof"]["idle_watts"]) * 1e3,
                           note="the GEMM figures are the routed experts' launches on their own; inside the step the same "
                                "launches also carry the shared expert's tiles; rest = router product, routing + activation "
-                               "quantisation, permutation, weighted sum and the shared expert's share")
+                               "quantisation, permutation, weighted sum and the shared expert's share; power_floor_ms = the "
+                               "time the step's unavoidable bytes and matrix operations alone take at the package power cap "
+                               "(coefficients of roofline.power_roof)")
     if decode is not None:
         result["decode"] = decode
         result["dense"] = bench_dense(pkg, dev, args.steps, args.warmup)
