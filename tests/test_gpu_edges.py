@@ -207,3 +207,38 @@ def test_read_probe_reads_any_size_and_rejects_bad_arguments(pkg, dev):
         bench.hbm_read_probe(buf[:24])
     with pytest.raises(RuntimeError):
         bench.hbm_read_probe(buf, 24)
+
+
+@pytest.mark.parametrize("counts", [[1, 97, 193, 1209], [96, 192, 288, 1000], [95, 191, 2, 1400], [0, 383, 385, 900]])
+def test_half_tiles_at_the_edges_of_their_tiles(pkg, oracle, dev, checks, counts):
+    """Experts with many rows and a short reduction run the 96-row half tiles on a 192-row tile list: expert row counts
+    that end exactly at, one before and one after the halves' and the list tiles' edges (and an expert without a row),
+    every token against the oracle through the strict steps, and the batch's rows equal to the same tokens run alone."""
+    say("half tiles, rows per expert", counts)
+    E, K, H, I = len(counts), 1, 256, 256
+    T = sum(counts)
+    assert T * K / E >= 320 and H // 128 <= 20 and pkg.tile_rows(T, K, E) == 192      # the launcher's rule for half tiles
+    ids = torch.cat([torch.full((n,), e, dtype=torch.int32) for e, n in enumerate(counts)])
+    g = torch.Generator().manual_seed(sum(counts))
+    ids = ids[torch.randperm(T, generator=g)].reshape(T, 1).contiguous()
+    w = torch.rand(T, 1, generator=g) + 0.5
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    ld = pkg.pack_layer(*(t.to(dev) for t in oracle.make_layer(E, H, I, seed=7)))
+    xd, idd, wd = x.to(dev), ids.to(dev), w.to(dev)
+    y = pkg.fused_experts_fp8(xd, *ld, idd)
+    out = pkg.fused_experts_fp8(xd, *ld, idd, wd)
+    torch.cuda.synchronize()
+    assert torch.isfinite(y.float()).all()
+    # first and last rows of every expert (in permuted order those sit at the tiles' edges)
+    order = torch.argsort(ids[:, 0], stable=True)
+    edges = []
+    pos = 0
+    for n in counts:
+        for r in (0, 95, 96, 97, 191, 192, 193, n - 1):
+            if 0 <= r < n:
+                edges.append(int(order[pos + r]))
+        pos += n
+    pick = torch.tensor(sorted(set(edges)), device=dev)
+    rep = checks.check_sample(pkg, oracle, xd[pick].contiguous(), idd[pick].contiguous(), ld, w_s=wd[pick].contiguous(),
+                              y_big=y[pick].contiguous(), out_big=out[pick].contiguous(), what="half tiles")
+    say("   ", rep)
