@@ -7,7 +7,8 @@
 namespace moe {
 
 int permute_launch(hipStream_t st, const int32_t *ids, int T, int K, int E, int tile_m, int32_t *sorted_slot,
-                   int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &ws);
+                   int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &ws, uint16_t *zero_rows = nullptr,
+                   int row_len = 0);
 int gemm1_launch(hipStream_t st, const uint8_t *xq, const float *xs, int T, int H, const uint8_t *w13,
                  const float *w13s, int I, int E, int K, const int32_t *sorted_slot, const int32_t *expert_offsets,
                  const PermuteWs *pw, int fixed_expert, uint8_t *hq, float *hs, const uint8_t *sh_w13,
@@ -22,7 +23,6 @@ int decode_prep_launch(hipStream_t st, const uint16_t *x, int T, int H, const ui
                        int32_t *ids, int *arrivals, uint8_t *xq, float *xs, int tile_m, int32_t *sorted_slot,
                        int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &pw);
 
-int zero_dropped_rows_launch(hipStream_t st, const int32_t *slot_to_row, int TK, int H, uint16_t *y);
 int weighted_reduce_launch(hipStream_t st, const uint16_t *y, const float *w, const uint16_t *shared_y,
                            const int32_t *slot_to_row, int T, int K, int H, uint16_t *out);
 size_t router_front_partial_bytes(int T, int H, int E);
@@ -97,8 +97,9 @@ static int run_experts(void *stream, const FusedWs &w, const PermuteWs &pw, int 
   rc = gemm2_launch(st, w.hq, w.hs, T * K, T, H, w2, w2_scale, I, E, K, w.sorted_slot, w.expert_offsets, &pw, -1, y,
                     w.sh_hq, w.sh_hs, T, fuse_shared ? shared_w2 : nullptr, shared_w2_scale, w.sh_y);
   if (rc) return rc;
-  // slots whose expert id lies outside [0, E) have no row: zero rows in the per-slot form, no term in the sum
-  if (out_mode == 0) return zero_dropped_rows_launch(st, w.slot_to_row, T * K, H, y);
+  // slots whose expert id lies outside [0, E) have no row: zero rows in the per-slot form (cleared by the permutation
+  // launch), no term in the sum
+  if (out_mode == 0) return MOE_OK;
   if (has_shared && !fuse_shared) {
     rc = gemm1_launch(st, w.xq, w.xs, T, H, shared_w13, shared_w13_scale, I_sh, 1, 1, nullptr, nullptr, nullptr, 0,
                       w.sh_hq, w.sh_hs, nullptr, nullptr, nullptr, nullptr);
@@ -208,7 +209,9 @@ extern "C" int moe_fused_experts_fp8(void *stream, const void *x_bf16, int T, in
 
   hipStream_t st = (hipStream_t)stream;
   PermuteWs pw = permute_ws_layout(w.permute, T, K, E);
-  int rc = permute_launch(st, ids, T, K, E, choose_tile_m(T, K, E), w.sorted_slot, w.expert_offsets, w.slot_to_row, pw);
+  // per-slot output form: the rows of slots without an expert are cleared by the permutation (nothing else writes them)
+  int rc = permute_launch(st, ids, T, K, E, choose_tile_m(T, K, E), w.sorted_slot, w.expert_offsets, w.slot_to_row, pw,
+                          out_mode == 0 ? (uint16_t *)out_bf16 : nullptr, H);
   if (rc) return rc;
   rc = moe_act_quant(stream, x_bf16, T, H, w.xq, w.xs);
   if (rc) return rc;
@@ -571,7 +574,8 @@ static int experts_a16_run(void *stream, const void *x_bf16, int T, int H, const
   if (T == 0) return MOE_OK;
   hipStream_t st = (hipStream_t)stream;
   PermuteWs pw = permute_ws_layout(w.permute, T, K, E);
-  int rc = permute_launch(st, ids, T, K, E, choose_tile_m(T, K, E), w.sorted_slot, w.expert_offsets, w.slot_to_row, pw);
+  int rc = permute_launch(st, ids, T, K, E, choose_tile_m(T, K, E), w.sorted_slot, w.expert_offsets, w.slot_to_row, pw,
+                          out_mode == 0 ? (uint16_t *)out_bf16 : nullptr, H);
   if (rc) return rc;
   rc = gemm1_launch(st, (const uint8_t *)x_bf16, nullptr, T, H, (const uint8_t *)w13, w13_scale, I, E, K, w.sorted_slot,
                     w.expert_offsets, &pw, -1, (uint8_t *)w.h, nullptr, nullptr, nullptr, nullptr, nullptr, numerics);
@@ -580,7 +584,7 @@ static int experts_a16_run(void *stream, const void *x_bf16, int T, int H, const
   rc = gemm2_launch(st, (const uint8_t *)w.h, nullptr, T * K, T, H, (const uint8_t *)w2, w2_scale, I, E, K,
                     w.sorted_slot, w.expert_offsets, &pw, -1, y, nullptr, nullptr, 0, nullptr, nullptr, nullptr, numerics);
   if (rc) return rc;
-  if (out_mode == 0) return zero_dropped_rows_launch(st, w.slot_to_row, T * K, H, y);
+  if (out_mode == 0) return MOE_OK;        // the rows of slots without an expert were cleared by the permutation launch
   return weighted_reduce_launch(st, y, routing_weights, nullptr, w.slot_to_row, T, K, H, (uint16_t *)out_bf16);
 }
 }  // namespace moe

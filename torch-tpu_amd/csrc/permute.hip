@@ -36,6 +36,14 @@ __device__ __forceinline__ void match_rank(int v, bool valid, int lane, int &ran
   }
 }
 
+// The per-slot output row of a slot without an expert is zero: its one thread clears it (such slots are rare - a rank of
+// an expert-parallel group sees them for the experts it does not hold).  rows null: nothing to clear.
+__device__ __forceinline__ void zero_slot_row(uint16_t *__restrict__ rows, int row_len, int slot) {
+  if (rows == nullptr) return;
+  v4i *row = (v4i *)(rows + (size_t)slot * row_len);
+  for (int i = 0; i < row_len / 8; i++) row[i] = (v4i){0, 0, 0, 0};
+}
+
 __global__ __launch_bounds__(64) void permute_count_kernel(const int32_t *__restrict__ ids, int TK, int E,
                                                            int32_t *__restrict__ chunk_counts) {
   __shared__ int hist[MOE_MAX_EXPERTS];
@@ -163,7 +171,8 @@ __global__ __launch_bounds__(kChunk) void permute_scatter_kernel(const int32_t *
                                                                  const int32_t *__restrict__ chunk_counts,
                                                                  const int32_t *__restrict__ expert_offsets,
                                                                  int32_t *__restrict__ sorted_slot,
-                                                                 int32_t *__restrict__ slot_to_row) {
+                                                                 int32_t *__restrict__ slot_to_row,
+                                                                 uint16_t *__restrict__ zero_rows, int row_len) {
   constexpr int NWV = kChunk / 64;
   __shared__ int base[MOE_MAX_EXPERTS];
   __shared__ int wcount[NWV][MOE_MAX_EXPERTS];
@@ -189,6 +198,7 @@ __global__ __launch_bounds__(kChunk) void permute_scatter_kernel(const int32_t *
   }
   if (valid && row < TK) sorted_slot[row] = s;
   if (s < TK) slot_to_row[s] = row;
+  if (s < TK && row < 0) zero_slot_row(zero_rows, row_len, s);
 }
 
 __global__ __launch_bounds__(kChunk) void permute_small_kernel(const int32_t *__restrict__ ids, int TK, int E, int tile_m,
@@ -197,26 +207,31 @@ __global__ __launch_bounds__(kChunk) void permute_small_kernel(const int32_t *__
                                                               int32_t *__restrict__ slot_to_row,
                                                               int32_t *__restrict__ tile_prefix,
                                                               int32_t *__restrict__ tile_expert,
-                                                              int32_t *__restrict__ tile_desc) {
+                                                              int32_t *__restrict__ tile_desc,
+                                                              uint16_t *__restrict__ zero_rows, int row_len) {
   __shared__ PermuteSmallSmem sm;
   const int s = threadIdx.x;
-  permute_small_block(sm, (s < TK) ? ids[s] : -1, TK, E, tile_m, max_tiles, sorted_slot, expert_offsets, slot_to_row,
-                      tile_prefix, tile_expert, tile_desc);
+  const int v = (s < TK) ? ids[s] : -1;
+  permute_small_block(sm, v, TK, E, tile_m, max_tiles, sorted_slot, expert_offsets, slot_to_row, tile_prefix, tile_expert,
+                      tile_desc);
+  if (s < TK && (v < 0 || v >= E)) zero_slot_row(zero_rows, row_len, s);
 }
 
+// zero_rows (may be null): a [T*K, row_len] bf16 tensor in slot order whose rows of slots WITHOUT an expert (id outside
+// [0, E)) are cleared here - the per-slot output form: nothing else ever writes those rows
 int permute_launch(hipStream_t st, const int32_t *ids, int T, int K, int E, int tile_m, int32_t *sorted_slot,
-                   int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &ws) {
+                   int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &ws, uint16_t *zero_rows, int row_len) {
   const int TK = T * K;
   if (TK <= kChunk) {
     permute_small_kernel<<<1, kChunk, 0, st>>>(ids, TK, E, tile_m, ws.max_tiles, sorted_slot, expert_offsets, slot_to_row,
-                                           ws.tile_prefix, ws.tile_expert, ws.tile_desc);
+                                           ws.tile_prefix, ws.tile_expert, ws.tile_desc, zero_rows, row_len);
     return (int)hipGetLastError();
   }
   permute_count_kernel<<<ws.n_chunks, 64, 0, st>>>(ids, TK, E, ws.chunk_counts);
   permute_scan_kernel<<<1, 1024, 0, st>>>(ws.chunk_counts, ws.n_chunks, E, tile_m, ws.max_tiles, expert_offsets,
                                           ws.tile_prefix, ws.tile_expert, ws.tile_desc);
   permute_scatter_kernel<<<ws.n_chunks, kChunk, 0, st>>>(ids, TK, E, ws.chunk_counts, expert_offsets, sorted_slot,
-                                                     slot_to_row);
+                                                     slot_to_row, zero_rows, row_len);
   return (int)hipGetLastError();
 }
 
@@ -240,5 +255,5 @@ extern "C" int moe_permute(void *stream, const int32_t *ids, int T, int K, int E
   if ((uintptr_t)workspace % 4) return MOE_E_ALIGN;
   PermuteWs ws = permute_ws_layout(workspace, T, K, E);
   return permute_launch((hipStream_t)stream, ids, T, K, E, choose_tile_m(T, K, E), sorted_slot, expert_offsets,
-                        slot_to_row, ws);
+                        slot_to_row, ws, nullptr, 0);
 }

@@ -72,16 +72,6 @@ __global__ __launch_bounds__(256) void weighted_reduce_kernel(const uint16_t *__
   else *(v4i *)(out + (size_t)t * H + c) = o;
 }
 
-// [T, K, H] output form: the rows of slots without an expert (id outside [0, E)) are zero.  One thread per slot; the
-// rare thread that finds such a slot clears its row.
-__global__ __launch_bounds__(256) void zero_dropped_rows_kernel(const int32_t *__restrict__ slot_to_row, int TK, int H,
-                                                                uint16_t *__restrict__ y) {
-  const int s = blockIdx.x * 256 + threadIdx.x;
-  if (s >= TK || slot_to_row[s] >= 0) return;
-  v4i *row = (v4i *)(y + (size_t)s * H);
-  for (int i = 0; i < H / 8; i++) row[i] = (v4i){0, 0, 0, 0};
-}
-
 // Weight bytes between row-major order and the tile-blocked order the GEMMs read.  Tile-blocked: the matrix is cut
 // into tiles of 16 rows and steps of 128 bytes; the 2 KB of a (tile, step) pair are contiguous, tiles in row order,
 // a tile's steps one after the other, and inside the 2 KB: half h (0/1), then lane l (0..63), 16 bytes each =
@@ -113,12 +103,6 @@ static int repack_launch(hipStream_t st, const void *src, int64_t rows, int row_
   if (blocks > 0x7fffffffull) return MOE_E_SHAPE;
   repack_weights_kernel<<<(unsigned)blocks, 256, 0, st>>>((const v4i *)src, (v4i *)dst, n_units, row_bytes / kBlock,
                                                           row_bytes / 16, to_blocked);
-  return (int)hipGetLastError();
-}
-
-int zero_dropped_rows_launch(hipStream_t st, const int32_t *slot_to_row, int TK, int H, uint16_t *y) {
-  if (TK < 1) return MOE_OK;
-  zero_dropped_rows_kernel<<<(TK + 255) / 256, 256, 0, st>>>(slot_to_row, TK, H, y);
   return (int)hipGetLastError();
 }
 
