@@ -9,6 +9,9 @@ namespace moe {
 int permute_launch(hipStream_t st, const int32_t *ids, int T, int K, int E, int tile_m, int32_t *sorted_slot,
                    int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &ws, uint16_t *zero_rows = nullptr,
                    int row_len = 0);
+int permute_quant_small_launch(hipStream_t st, const int32_t *ids, int T, int K, int E, int tile_m, int32_t *sorted_slot,
+                               int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &ws, uint16_t *zero_rows,
+                               int row_len, const uint16_t *x, int H, uint8_t *xq, float *xs);
 int gemm1_launch(hipStream_t st, const uint8_t *xq, const float *xs, int T, int H, const uint8_t *w13,
                  const float *w13s, int I, int E, int K, const int32_t *sorted_slot, const int32_t *expert_offsets,
                  const PermuteWs *pw, int fixed_expert, uint8_t *hq, float *hs, const uint8_t *sh_w13,
@@ -210,11 +213,20 @@ extern "C" int moe_fused_experts_fp8(void *stream, const void *x_bf16, int T, in
   hipStream_t st = (hipStream_t)stream;
   PermuteWs pw = permute_ws_layout(w.permute, T, K, E);
   // per-slot output form: the rows of slots without an expert are cleared by the permutation (nothing else writes them)
-  int rc = permute_launch(st, ids, T, K, E, choose_tile_m(T, K, E), w.sorted_slot, w.expert_offsets, w.slot_to_row, pw,
-                          out_mode == 0 ? (uint16_t *)out_bf16 : nullptr, H);
-  if (rc) return rc;
-  rc = moe_act_quant(stream, x_bf16, T, H, w.xq, w.xs);
-  if (rc) return rc;
+  uint16_t *const zero_rows = out_mode == 0 ? (uint16_t *)out_bf16 : nullptr;
+  int rc;
+  if ((long)T * K <= kChunk) {
+    // decode sizes: permutation and activation quantisation share one launch
+    rc = permute_quant_small_launch(st, ids, T, K, E, choose_tile_m(T, K, E), w.sorted_slot, w.expert_offsets,
+                                    w.slot_to_row, pw, zero_rows, H, (const uint16_t *)x_bf16, H, w.xq, w.xs);
+    if (rc) return rc;
+  } else {
+    rc = permute_launch(st, ids, T, K, E, choose_tile_m(T, K, E), w.sorted_slot, w.expert_offsets, w.slot_to_row, pw,
+                        zero_rows, H);
+    if (rc) return rc;
+    rc = moe_act_quant(stream, x_bf16, T, H, w.xq, w.xs);
+    if (rc) return rc;
+  }
   return run_experts(stream, w, pw, T, H, w13, w13_scale, w2, w2_scale, I, E, K, routing_weights, shared_w13,
                      shared_w13_scale, shared_w2, shared_w2_scale, I_sh, out_bf16, out_mode);
 }

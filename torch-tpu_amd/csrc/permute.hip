@@ -13,6 +13,7 @@
 #include "moe_common.h"
 #include "moe_layout.h"
 #include "permute_small.h"
+#include "act_quant.h"
 #include "../../include/moe_hip.h"
 
 namespace moe {
@@ -215,6 +216,40 @@ __global__ __launch_bounds__(kChunk) void permute_small_kernel(const int32_t *__
   permute_small_block(sm, v, TK, E, tile_m, max_tiles, sorted_slot, expert_offsets, slot_to_row, tile_prefix, tile_expert,
                       tile_desc);
   if (s < TK && (v < 0 || v >= E)) zero_slot_row(zero_rows, row_len, s);
+}
+
+// The same with the activation quantisation in the launch: workgroup 0 permutes, the workgroups after it quantise x
+// (16 lanes per 128-column group).  At this size either is one short dependent chain; side by side they cost one launch.
+__global__ __launch_bounds__(kChunk) void permute_small_quant_kernel(
+    const int32_t *__restrict__ ids, int TK, int E, int tile_m, int max_tiles, int32_t *__restrict__ sorted_slot,
+    int32_t *__restrict__ expert_offsets, int32_t *__restrict__ slot_to_row, int32_t *__restrict__ tile_prefix,
+    int32_t *__restrict__ tile_expert, int32_t *__restrict__ tile_desc, uint16_t *__restrict__ zero_rows, int row_len,
+    const uint16_t *__restrict__ x, size_t n_groups, int groups_per_row, int pitch, uint8_t *__restrict__ xq,
+    float *__restrict__ xs) {
+  if (blockIdx.x > 0) {
+    act_quant_thread(x, n_groups, groups_per_row, pitch, xq, xs, (size_t)(blockIdx.x - 1) * kChunk + threadIdx.x);
+    return;
+  }
+  __shared__ PermuteSmallSmem sm;
+  const int s = threadIdx.x;
+  const int v = (s < TK) ? ids[s] : -1;
+  permute_small_block(sm, v, TK, E, tile_m, max_tiles, sorted_slot, expert_offsets, slot_to_row, tile_prefix, tile_expert,
+                      tile_desc);
+  if (s < TK && (v < 0 || v >= E)) zero_slot_row(zero_rows, row_len, s);
+}
+
+// Permutation of at most kChunk slots and quantisation of x [T, H] bf16 -> xq e4m3fn [T, H], xs fp32 (pitch
+// scale_pitch(H / 128)) in one launch.  The caller has checked T * K <= kChunk, H % 128 == 0 and the pointers.
+int permute_quant_small_launch(hipStream_t st, const int32_t *ids, int T, int K, int E, int tile_m, int32_t *sorted_slot,
+                               int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &ws, uint16_t *zero_rows,
+                               int row_len, const uint16_t *x, int H, uint8_t *xq, float *xs) {
+  const size_t groups = (size_t)T * (H / kBlock);
+  const unsigned quant_blocks = (unsigned)((groups * 16 + kChunk - 1) / kChunk);
+  permute_small_quant_kernel<<<1 + quant_blocks, kChunk, 0, st>>>(ids, T * K, E, tile_m, ws.max_tiles, sorted_slot,
+                                                                  expert_offsets, slot_to_row, ws.tile_prefix,
+                                                                  ws.tile_expert, ws.tile_desc, zero_rows, row_len, x,
+                                                                  groups, H / kBlock, scale_pitch(H / kBlock), xq, xs);
+  return (int)hipGetLastError();
 }
 
 // zero_rows (may be null): a [T*K, row_len] bf16 tensor in slot order whose rows of slots WITHOUT an expert (id outside
