@@ -298,6 +298,18 @@ int moe_layer_fp8(void *stream, const void *x_bf16, int T, int H,
                          void *workspace, size_t workspace_bytes);
 
 /*
+ * Batches of 512 tokens and more with a shared expert of the routed experts' width: moe_layer_fp8 runs the shared
+ * expert's first GEMM, which needs nothing of the routing, on a stream of the library's own beside the router
+ * product, routing and permutation launches (short chains that leave most of the chip idle), fenced by events on
+ * both sides, so that to the caller the call is still work on its one stream; the results are the same bit for bit.
+ * The side stream and its two events are created per (device, caller's stream) at the first call that uses them.
+ * Not used while the caller's stream is being captured into a graph.  No counterpart in the reference (its device
+ * runtime schedules the whole op).  moe_set_shared_overlap(0) switches it off, (1) on (the default); returns the
+ * previous setting.
+ */
+int moe_set_shared_overlap(int enabled);
+
+/*
  * moe_layer_fp8 for callers that cannot allocate device memory or hand over a workspace: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference (its ops take
  * every scratch tensor from the caller, fusedMoE.cpp:237-318).  Same arguments, same kernels and the same

@@ -43,13 +43,18 @@ int main() {
         unsigned char *base = buf.data() + (32 - (uintptr_t)buf.data() % 32) % 32;
         PermuteWs p = permute_ws_layout(base, T, K, E);
         CHECK((unsigned char *)p.chunk_counts == base);
-        CHECK(p.tile_prefix == p.chunk_counts + (size_t)p.n_chunks * E);
+        // the table, the per-expert totals and the arrival counter are one run of integers (cleared in one go)
+        CHECK(p.expert_count == p.chunk_counts + (size_t)p.n_chunks * E);
+        CHECK(p.arrivals == p.expert_count + E);
+        CHECK(p.tile_prefix == p.arrivals + 1);
         CHECK(p.tile_expert == p.tile_prefix + E + 1);
         CHECK((uintptr_t)p.tile_desc % 32 == 0 && p.tile_desc >= p.tile_expert + p.max_tiles);
         CHECK((unsigned char *)(p.tile_desc + (size_t)8 * p.max_tiles) <= base + bytes);
         CHECK(p.max_tiles == mt);
         // touch every byte the layout hands out (the sanitizer watches the vector's bounds)
         for (int i = 0; i < p.n_chunks * E; i++) p.chunk_counts[i] = i;
+        for (int i = 0; i < E; i++) p.expert_count[i] = i;
+        *p.arrivals = 0;
         for (int i = 0; i <= E; i++) p.tile_prefix[i] = i;
         for (int i = 0; i < p.max_tiles; i++) p.tile_expert[i] = i;
         for (long i = 0; i < 8l * p.max_tiles; i++) p.tile_desc[i] = (int)i;

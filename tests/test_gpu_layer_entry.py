@@ -258,6 +258,54 @@ def test_layer_entry_point_in_a_hip_graph(pkg, oracle, dev):
             assert torch.equal(moe(x).view(torch.int16), ref.view(torch.int16))     # eager work between replays
 
 
+def test_shared_expert_beside_the_front_end_changes_no_bit(pkg, oracle, dev):
+    """Batches of 512 tokens and more: the shared expert's first GEMM runs on a stream of the library's own beside the
+    router product, routing and permutation.  Same bits as with that switched off, on the default stream and on a
+    stream of the caller's, call after call into one workspace, and inside a graph capture (where the side stream is
+    not used)."""
+    say("shared expert beside the front end")
+    T, H, I, E, K = 777, 1024, 256, 32, 4
+    ld = pkg.pack_layer(*(t.to(dev) for t in oracle.make_layer(E, H, I, seed=11)))
+    shared = _shared(pkg, oracle, H, I, 12, dev)
+    g = torch.Generator().manual_seed(11)
+    wr = (torch.randn(E, H, generator=g) * 0.05).to(torch.bfloat16).to(dev)
+    xs = [torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev) for _ in range(3)]
+    kw = dict(shared=shared, n_groups=4, topk_groups=2, renorm=True, scale=2.5)
+    was = pkg.set_shared_overlap(False)
+    try:
+        assert was is True
+        plain = [pkg.layer_fp8(x, wr, *ld, K, "sigmoid", **kw).clone() for x in xs]
+        assert pkg.set_shared_overlap(True) is False
+        ws = torch.empty(pkg.layer_workspace_bytes(T, H, I, E, K, I), dtype=torch.uint8, device=dev)
+        for rep in range(3):
+            for x, ref in zip(xs, plain):
+                got = pkg.layer_fp8(x, wr, *ld, K, "sigmoid", workspace=ws, **kw)
+                assert torch.equal(got.view(torch.int16), ref.view(torch.int16)), rep
+        torch.cuda.synchronize()
+        own = torch.cuda.Stream()
+        own.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(own):
+            ws2 = torch.empty_like(ws)
+            got = [pkg.layer_fp8(x, wr, *ld, K, "sigmoid", workspace=ws2, **kw) for x in xs]
+        torch.cuda.current_stream().wait_stream(own)
+        for a, ref in zip(got, plain):
+            assert torch.equal(a.view(torch.int16), ref.view(torch.int16))
+        # under capture the call stays on the captured stream
+        x_static, out_static = xs[0].clone(), torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            pkg.layer_fp8(x_static, wr, *ld, K, "sigmoid", out=out_static, workspace=ws, **kw)
+        for rep in range(2):
+            for x, ref in zip(xs, plain):
+                x_static.copy_(x)
+                graph.replay()
+                torch.cuda.synchronize()
+                assert torch.equal(out_static.view(torch.int16), ref.view(torch.int16)), rep
+                assert torch.equal(pkg.layer_fp8(x, wr, *ld, K, "sigmoid", **kw).view(torch.int16), ref.view(torch.int16))
+    finally:
+        pkg.set_shared_overlap(True)
+
+
 def test_layer_entry_point_rejects_what_it_does_not_cover(pkg, oracle, dev):
     say("layer entry errors")
     H, I = 256, 128

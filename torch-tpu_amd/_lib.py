@@ -46,6 +46,7 @@ SIGNATURES = {
                                      c_int, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                      c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_size_t]),
+    "moe_set_shared_overlap": (c_int, [c_int]),
     "moe_hip_init": (c_int, []),
     "moe_static_scratch_address": (c_int, [ctypes.POINTER(c_void_p)]),
     "moe_layer_fp8_static": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,

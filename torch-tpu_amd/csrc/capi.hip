@@ -1,5 +1,6 @@
 // The whole-path entry point and the library's housekeeping calls.
 #include <atomic>
+#include <mutex>
 #include "moe_common.h"
 #include "moe_layout.h"
 #include "../../include/moe_hip.h"
@@ -8,7 +9,7 @@ namespace moe {
 
 int permute_launch(hipStream_t st, const int32_t *ids, int T, int K, int E, int tile_m, int32_t *sorted_slot,
                    int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &ws, uint16_t *zero_rows = nullptr,
-                   int row_len = 0);
+                   int row_len = 0, bool counted = false);
 int permute_quant_small_launch(hipStream_t st, const int32_t *ids, int T, int K, int E, int tile_m, int32_t *sorted_slot,
                                int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &ws, uint16_t *zero_rows,
                                int row_len, const uint16_t *x, int H, uint8_t *xq, float *xs);
@@ -29,11 +30,13 @@ int decode_prep_launch(hipStream_t st, const uint16_t *x, int T, int H, const ui
 int weighted_reduce_launch(hipStream_t st, const uint16_t *y, const float *w, const uint16_t *shared_y,
                            const int32_t *slot_to_row, int T, int K, int H, uint16_t *out);
 size_t router_front_partial_bytes(int T, int H, int E);
-int router_front_launch(hipStream_t st, const void *x, int T, int H, const void *wr, int E, float *partial, int *n_slices_out);
+int router_front_launch(hipStream_t st, const void *x, int T, int H, const void *wr, int E, float *partial, int *n_slices_out,
+                        int32_t *zero = nullptr, int n_zero = 0);
 int sum_slices_launch(hipStream_t st, const float *partial, int n_slices, int T, int E, uint16_t *logits);
 int route_from_partials_launch(hipStream_t st, const float *partial, int n_slices, const float *bias, int T, int E, int K,
                                int mode, int n_groups, int topk_groups, int renorm, float scale, float *weights_out,
-                               int32_t *ids_out, const uint16_t *x, int H, uint8_t *xq, float *xs);
+                               int32_t *ids_out, const uint16_t *x, int H, uint8_t *xq, float *xs,
+                               int32_t *chunk_counts = nullptr);
 
 size_t dense_small_partial_bytes(int M, int K, int N, bool keep_partial);
 int dense_small_launch(hipStream_t st, const uint8_t *xq, const float *xs, int M, int K, const uint8_t *w, const float *ws,
@@ -83,18 +86,75 @@ static FusedWs fused_layout(void *base, int T, int H, int I, int E, int K, int I
   return w;
 }
 
+// ---- the shared expert's first GEMM beside the front end ----
+// The shared expert's first GEMM needs the quantised activations and nothing of the routing.  The router product,
+// the routing and the three permutation launches are short chains that leave most of the chip idle, so for batches
+// beyond the decode size moe_layer_fp8 runs the quantisation and that GEMM on a stream of its own while the caller's
+// stream goes through the front end: an event on the caller's stream lets the side stream start, the caller's stream
+// waits for the quantised activations before the first grouped GEMM and for the shared expert's first GEMM before
+// the second (which carries the shared expert's tiles as before).  The router product comes first on the caller's
+// stream: its workgroups need most of a compute unit's LDS, which a GEMM workgroup would not leave them.
+// To the caller the call is still work on its one stream.  One side stream and one pair of events per (device,
+// caller's stream), created at the first call that uses them and kept until the process ends; streams of the default
+// priority, no implicit synchronisation with the null stream.  Not used while the caller's stream is being captured
+// into a graph, nor by the entry point that allocates nothing.
+struct SideLane {
+  int device;
+  hipStream_t main, side;
+  hipEvent_t fork, quantised, join;
+};
+constexpr int kMaxSideLanes = 32;
+static std::mutex g_side_mutex;
+static SideLane g_side[kMaxSideLanes];
+static int g_n_side = 0;
+static std::atomic<int> g_overlap_enabled{1};
+constexpr int kOverlapMinTokens = 512;       // below, the front end is too short to hide anything behind
+
+static const SideLane *side_lane(hipStream_t st) {
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(st, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+  std::lock_guard<std::mutex> lock(g_side_mutex);
+  for (int i = 0; i < g_n_side; i++)
+    if (g_side[i].device == dev && g_side[i].main == st) return &g_side[i];
+  if (g_n_side == kMaxSideLanes) return nullptr;       // more caller streams than lanes: those go without
+  SideLane l{dev, st, nullptr, nullptr, nullptr, nullptr};
+  if (hipStreamCreateWithFlags(&l.side, hipStreamNonBlocking) != hipSuccess) return nullptr;
+  if (hipEventCreateWithFlags(&l.fork, hipEventDisableTiming) != hipSuccess ||
+      hipEventCreateWithFlags(&l.quantised, hipEventDisableTiming) != hipSuccess ||
+      hipEventCreateWithFlags(&l.join, hipEventDisableTiming) != hipSuccess) {
+    if (l.fork) (void)hipEventDestroy(l.fork);
+    if (l.quantised) (void)hipEventDestroy(l.quantised);
+    (void)hipStreamDestroy(l.side);
+    return nullptr;
+  }
+  g_side[g_n_side] = l;
+  return &g_side[g_n_side++];
+}
+
 // The grouped GEMMs and the weighted sum, once the permutation and the quantised activations are in the workspace.
+// join: the shared expert's first GEMM has been launched elsewhere and this event marks its end.
 static int run_experts(void *stream, const FusedWs &w, const PermuteWs &pw, int T, int H, const uint8_t *w13,
                        const float *w13_scale, const uint8_t *w2, const float *w2_scale, int I, int E, int K,
                        const float *routing_weights, const uint8_t *shared_w13, const float *shared_w13_scale,
-                       const uint8_t *shared_w2, const float *shared_w2_scale, int I_sh, void *out_bf16, int out_mode) {
+                       const uint8_t *shared_w2, const float *shared_w2_scale, int I_sh, void *out_bf16, int out_mode,
+                       hipEvent_t join = nullptr) {
   hipStream_t st = (hipStream_t)stream;
   const bool has_shared = shared_w13 != nullptr;
   // a shared expert of the routed experts' width rides in the routed launches (its tiles fill the
   // machine together with theirs); any other width gets launches of its own
   const bool fuse_shared = has_shared && I_sh == I;
   int rc = gemm1_launch(st, w.xq, w.xs, T, H, w13, w13_scale, I, E, K, w.sorted_slot, w.expert_offsets, &pw, -1, w.hq, w.hs,
-                        fuse_shared ? shared_w13 : nullptr, shared_w13_scale, w.sh_hq, w.sh_hs);
+                        fuse_shared && !join ? shared_w13 : nullptr, shared_w13_scale, w.sh_hq, w.sh_hs);
+  if (join) {
+    // also after a failed launch: nothing of this call may outlive the caller's stream on the side stream
+    const int rc_wait = (int)hipStreamWaitEvent(st, join, 0);
+    if (rc == MOE_OK) rc = rc_wait;
+  }
   if (rc) return rc;
   uint16_t *y = out_mode == 0 ? (uint16_t *)out_bf16 : w.y;
   rc = gemm2_launch(st, w.hq, w.hs, T * K, T, H, w2, w2_scale, I, E, K, w.sorted_slot, w.expert_offsets, &pw, -1, y,
@@ -243,7 +303,7 @@ static int layer_fp8_run(void *stream, const void *x_bf16, int T, int H, const v
                          const float *w2_scale, int I, const uint8_t *shared_w13, const float *shared_w13_scale,
                          const uint8_t *shared_w2, const float *shared_w2_scale, int I_shared, void *out_bf16,
                          void *logits_out_bf16, float *weights_out, int32_t *ids_out, void *workspace,
-                         size_t workspace_bytes) {
+                         size_t workspace_bytes, bool may_use_side_stream) {
   if (!router_w_bf16 || !w13 || !w13_scale || !w2 || !w2_scale || !workspace) return MOE_E_NULL;
   if (T != 0 && (!x_bf16 || !out_bf16)) return MOE_E_NULL;
   if (T < 0 || H < 1 || I < 1 || E < 1 || E > MOE_MAX_EXPERTS || K < 1 || K > MOE_MAX_TOPK || K > E) return MOE_E_SHAPE;
@@ -270,6 +330,7 @@ static int layer_fp8_run(void *stream, const void *x_bf16, int T, int H, const v
   float *weights = weights_out ? weights_out : d.weights;
   int32_t *ids = ids_out ? ids_out : d.ids;
   int rc;
+  hipEvent_t join = nullptr;
   if (decode_size(T, K, E)) {
     // two launches: router logits + activation quantisation, then routing + permutation
     rc = decode_prep_launch(st, (const uint16_t *)x_bf16, T, H, (const uint16_t *)router_w_bf16, router_bias, E, K, mode,
@@ -278,23 +339,59 @@ static int layer_fp8_run(void *stream, const void *x_bf16, int T, int H, const v
                             w.slot_to_row, pw);
     if (rc) return rc;
   } else {
-    // the router product on the matrix cores, its reduction cut into slices; the routing kernel adds the slices
+    // a shared expert of the routed experts' width: its first GEMM runs beside the front end
+    const SideLane *lane = nullptr;
+    if (may_use_side_stream && has_shared && I_sh == I && T >= kOverlapMinTokens && g_overlap_enabled.load())
+      lane = side_lane(st);
+    // the router product on the matrix cores, its reduction cut into slices; the routing kernel adds the slices.
+    // More than kChunk slots: the routing kernel also counts the slots per (chunk, expert) - the permutation's first
+    // pass - into a table the router product's launch has cleared (table, per-expert totals and arrival counter are
+    // one run of integers).
     int n_slices = 0;
-    rc = router_front_launch(st, x_bf16, T, H, router_w_bf16, E, d.partial, &n_slices);
-    if (rc) return rc;
-    if (logits_out_bf16) {
-      rc = sum_slices_launch(st, d.partial, n_slices, T, E, (uint16_t *)logits_out_bf16);
+    const bool counted = (long)T * K > kChunk && (size_t)pw.n_chunks * E < ((size_t)1 << 30);
+    int32_t *const zero = counted ? pw.chunk_counts : nullptr;
+    const int n_zero = counted ? (int)(pw.arrivals + 1 - pw.chunk_counts) : 0;
+    if (lane) {
+      rc = (int)hipEventRecord(lane->fork, st);
       if (rc) return rc;
+      rc = router_front_launch(st, x_bf16, T, H, router_w_bf16, E, d.partial, &n_slices, zero, n_zero);
+      if (rc) return rc;
+      rc = (int)hipStreamWaitEvent(lane->side, lane->fork, 0);
+      if (rc) return rc;
+      rc = moe_act_quant(lane->side, x_bf16, T, H, w.xq, w.xs);
+      if (rc == MOE_OK) rc = (int)hipEventRecord(lane->quantised, lane->side);
+      if (rc == MOE_OK)
+        rc = gemm1_launch(lane->side, w.xq, w.xs, T, H, shared_w13, shared_w13_scale, I_sh, 1, 1, nullptr, nullptr,
+                          nullptr, 0, w.sh_hq, w.sh_hs, nullptr, nullptr, nullptr, nullptr);
+      // whatever the launches returned, the caller's stream waits for the side stream: nothing of this call may still
+      // run there when the caller's stream has finished
+      const int rc_join = (int)hipEventRecord(lane->join, lane->side);
+      if (rc_join) return rc_join;
+      join = lane->join;
+      if (rc) {
+        (void)hipStreamWaitEvent(st, join, 0);
+        return rc;
+      }
+    } else {
+      rc = router_front_launch(st, x_bf16, T, H, router_w_bf16, E, d.partial, &n_slices, zero, n_zero);
     }
-    // the activations are quantised by extra workgroups of the routing launch
-    rc = route_from_partials_launch(st, d.partial, n_slices, router_bias, T, E, K, mode, n_groups, topk_groups, renorm,
-                                    scale, weights, ids, (const uint16_t *)x_bf16, H, w.xq, w.xs);
-    if (rc) return rc;
-    rc = permute_launch(st, ids, T, K, E, choose_tile_m(T, K, E), w.sorted_slot, w.expert_offsets, w.slot_to_row, pw);
-    if (rc) return rc;
+    if (rc == MOE_OK && logits_out_bf16) rc = sum_slices_launch(st, d.partial, n_slices, T, E, (uint16_t *)logits_out_bf16);
+    // the activations are quantised by extra workgroups of the routing launch (unless they already are)
+    if (rc == MOE_OK)
+      rc = route_from_partials_launch(st, d.partial, n_slices, router_bias, T, E, K, mode, n_groups, topk_groups, renorm,
+                                      scale, weights, ids, lane ? nullptr : (const uint16_t *)x_bf16, H, w.xq, w.xs,
+                                      zero);
+    if (rc == MOE_OK)
+      rc = permute_launch(st, ids, T, K, E, choose_tile_m(T, K, E), w.sorted_slot, w.expert_offsets, w.slot_to_row, pw,
+                          nullptr, 0, counted);
+    if (rc == MOE_OK && lane) rc = (int)hipStreamWaitEvent(st, lane->quantised, 0);
+    if (rc) {
+      if (join) (void)hipStreamWaitEvent(st, join, 0);
+      return rc;
+    }
   }
   return run_experts(stream, w, pw, T, H, w13, w13_scale, w2, w2_scale, I, E, K, weights, shared_w13, shared_w13_scale,
-                     shared_w2, shared_w2_scale, I_sh, out_bf16, 1);
+                     shared_w2, shared_w2_scale, I_sh, out_bf16, 1, join);
 }
 }  // namespace moe
 
@@ -308,8 +405,10 @@ extern "C" int moe_layer_fp8(void *stream, const void *x_bf16, int T, int H, con
   return moe::layer_fp8_run(stream, x_bf16, T, H, router_w_bf16, router_bias, E, K, mode, n_groups, topk_groups, renorm,
                             scale, w13, w13_scale, w2, w2_scale, I, shared_w13, shared_w13_scale, shared_w2,
                             shared_w2_scale, I_shared, out_bf16, logits_out_bf16, weights_out, ids_out, workspace,
-                            workspace_bytes);
+                            workspace_bytes, true);
 }
+
+extern "C" int moe_set_shared_overlap(int enabled) { return moe::g_overlap_enabled.exchange(enabled ? 1 : 0); }
 
 // ---- the same call for callers that cannot allocate: the workspace is an array that lives in the library ----
 //
@@ -371,7 +470,7 @@ extern "C" int moe_layer_fp8_static(void *stream, const void *x_bf16, int T, int
   if (rc) return rc;
   return layer_fp8_run(stream, x_bf16, T, H, router_w_bf16, router_bias, E, K, mode, n_groups, topk_groups, renorm, scale,
                        w13, w13_scale, w2, w2_scale, I, shared_w13, shared_w13_scale, shared_w2, shared_w2_scale, I_shared,
-                       out_bf16, logits_out_bf16, weights_out, ids_out, ws, (size_t)MOE_STATIC_SCRATCH_BYTES);
+                       out_bf16, logits_out_bf16, weights_out, ids_out, ws, (size_t)MOE_STATIC_SCRATCH_BYTES, false);
 }
 
 // The router product on its own: logits [T, E] bf16 = x [T, H] . Wr [E, H]^T (fp32 sums, rounded once).

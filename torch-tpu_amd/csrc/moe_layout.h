@@ -72,6 +72,8 @@ struct PermuteWs {
   int32_t *tile_prefix;    // [E + 1] first tile of each expert; [E] = number of tiles
   int32_t *tile_expert;    // [max_tiles]
   int32_t *tile_desc;      // [max_tiles][8]: expert, its first tile, its tiles, its first row, its rows, 0, 0, 0
+  int32_t *expert_count;   // [E] slots per expert (between the two halves of the scan kernel)
+  int32_t *arrivals;       // [1] workgroups of the scan kernel that have finished their first half
   int n_chunks;
   int max_tiles;
 };
@@ -89,7 +91,7 @@ static inline size_t permute_ws_bytes(int T, int K, int E) {
   long tk = (long)T * K;
   size_t n_chunks = (size_t)((tk + kChunk - 1) / kChunk);
   if (n_chunks == 0) n_chunks = 1;
-  size_t ints = n_chunks * (size_t)E + (size_t)(E + 1) + 9 * (size_t)permute_max_tiles(T, K, E) + 8;
+  size_t ints = n_chunks * (size_t)E + 2 * (size_t)(E + 1) + 9 * (size_t)permute_max_tiles(T, K, E) + 8;
   return align_up(ints * 4, 256);
 }
 
@@ -100,7 +102,9 @@ static inline PermuteWs permute_ws_layout(void *ws, int T, int K, int E) {
   if (p.n_chunks == 0) p.n_chunks = 1;
   p.max_tiles = permute_max_tiles(T, K, E);
   p.chunk_counts = (int32_t *)ws;
-  p.tile_prefix = p.chunk_counts + (size_t)p.n_chunks * E;
+  p.expert_count = p.chunk_counts + (size_t)p.n_chunks * E;
+  p.arrivals = p.expert_count + E;
+  p.tile_prefix = p.arrivals + 1;
   p.tile_expert = p.tile_prefix + (E + 1);
   // 32-byte aligned: one descriptor is fetched with a single scalar load
   p.tile_desc = (int32_t *)(((uintptr_t)(p.tile_expert + p.max_tiles) + 31) & ~(uintptr_t)31);

@@ -3,9 +3,10 @@
 // Three small kernels, no host round trip (the grouped GEMMs that follow read the expert
 // offsets and the tile list from device memory):
 //   count    one wavefront per chunk of kChunk consecutive slots: per-chunk histogram in LDS.
-//   scan     one workgroup: per expert, running sum over the chunks (turns the histogram into
-//            the chunk's starting rank inside its expert), then an exclusive scan over the
-//            experts -> expert_offsets, and the list of row tiles the GEMMs walk.
+//   scan     one wavefront per expert: running sum over the chunks (turns the histogram into
+//            the chunk's starting rank inside its expert); the workgroup that finishes last adds
+//            an exclusive scan over the experts -> expert_offsets, and the list of row tiles the
+//            GEMMs walk.
 //   scatter  one workgroup per chunk, one wavefront per 64 slots: ranks its slots in slot order
 //            with a ballot "match-any" loop, so equal experts keep their original order (stable),
 //            and writes sorted_slot / slot_to_row.
@@ -46,9 +47,11 @@ __device__ __forceinline__ void zero_slot_row(uint16_t *__restrict__ rows, int r
 }
 
 __global__ __launch_bounds__(64) void permute_count_kernel(const int32_t *__restrict__ ids, int TK, int E,
-                                                           int32_t *__restrict__ chunk_counts) {
+                                                           int32_t *__restrict__ chunk_counts,
+                                                           int32_t *__restrict__ arrivals) {
   __shared__ int hist[MOE_MAX_EXPERTS];
   const int lane = threadIdx.x, c = blockIdx.x;
+  if (c == 0 && lane == 0) *arrivals = 0;               // the scan kernel counts its workgroups here
   for (int e = lane; e < E; e += 64) hist[e] = 0;
   __syncthreads();
   const int lo = c * kChunk;
@@ -82,76 +85,100 @@ __device__ __forceinline__ int block_exclusive_scan(int x, int *lds_wave_sums, i
   return base + inc - x;
 }
 
-__global__ __launch_bounds__(1024) void permute_scan_kernel(int32_t *__restrict__ chunk_counts, int n_chunks, int E,
-                                                            int tile_m, int max_tiles,
-                                                            int32_t *__restrict__ expert_offsets,
-                                                            int32_t *__restrict__ tile_prefix,
-                                                            int32_t *__restrict__ tile_expert,
-                                                            int32_t *__restrict__ tile_desc) {
-  __shared__ int wave_sums[16];
-  __shared__ int partial[1024];                       // [part][expert]: slots of the expert in that part of the chunks
-  // The chunks are cut into P parts and thread (part, expert) walks one part: its sum first, then - once the sums of
-  // the parts before it are known - the running count that turns each chunk's histogram entry into the rank of the
-  // chunk's first slot inside the expert.  Sixteen independent loads at a time in both passes (a load-add-store chain
-  // per chunk would pay one memory round trip per chunk).
-  int epad = 1;
-  while (epad < E) epad <<= 1;
-  const int P = 1024 / epad, part = threadIdx.x / epad, pe = threadIdx.x % epad;
-  const int len = (n_chunks + P - 1) / P, c_lo = part * len, c_hi = min(n_chunks, c_lo + len);
-  constexpr int B = 16;
-  int sum = 0;
-  if (pe < E)
-    for (int c0 = c_lo; c0 < c_hi; c0 += B) {
+// Scan.  First half, one wavefront per expert: a running sum over the chunks turns each chunk's histogram entry into
+// the rank of the chunk's first slot inside the expert (64 lanes x 8 chunks at a time: every load of a round is
+// independent of the others), and leaves the expert's total.  Second half, by the workgroup that arrives last (a
+// counter the count kernel cleared): exclusive scan over the experts -> expert_offsets, and the list of row tiles the
+// GEMMs walk.  Workgroups of four wavefronts with a few registers each find room on a compute unit whatever else runs
+// there.
+constexpr int kScanWaves = 4;
+__global__ __launch_bounds__(64 * kScanWaves) void permute_scan_kernel(int32_t *__restrict__ chunk_counts, int n_chunks,
+                                                                       int E, int tile_m, int max_tiles,
+                                                                       int32_t *__restrict__ expert_offsets,
+                                                                       int32_t *__restrict__ tile_prefix,
+                                                                       int32_t *__restrict__ tile_expert,
+                                                                       int32_t *__restrict__ tile_desc,
+                                                                       int32_t *__restrict__ expert_count,
+                                                                       int32_t *__restrict__ arrivals) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int e_mine = blockIdx.x * kScanWaves + wave;
+  if (e_mine < E) {
+    constexpr int B = 8;
+    int running = 0;
+    for (int c0 = 0; c0 < n_chunks; c0 += 64 * B) {
+      const int c = c0 + lane * B;
       int x[B];
 #pragma unroll
-      for (int i = 0; i < B; i++) x[i] = c0 + i < c_hi ? chunk_counts[(size_t)(c0 + i) * E + pe] : 0;
+      for (int i = 0; i < B; i++) x[i] = c + i < n_chunks ? chunk_counts[(size_t)(c + i) * E + e_mine] : 0;
+      int sum = 0;
 #pragma unroll
       for (int i = 0; i < B; i++) sum += x[i];
-    }
-  partial[threadIdx.x] = sum;
-  __syncthreads();
-  if (pe < E) {
-    int run = 0;
-    for (int q = 0; q < part; q++) run += partial[q * epad + pe];
-    for (int c0 = c_lo; c0 < c_hi; c0 += B) {
-      int x[B];
+      int inc = sum;
 #pragma unroll
-      for (int i = 0; i < B; i++) x[i] = c0 + i < c_hi ? chunk_counts[(size_t)(c0 + i) * E + pe] : 0;
+      for (int off = 1; off < 64; off <<= 1) {
+        const int y = __shfl_up(inc, off, 64);
+        if (lane >= off) inc += y;
+      }
+      int rank = running + inc - sum;
 #pragma unroll
       for (int i = 0; i < B; i++) {
-        if (c0 + i < c_hi) chunk_counts[(size_t)(c0 + i) * E + pe] = run;   // rank of the chunk's first slot inside the expert
-        run += x[i];
+        if (c + i < n_chunks) chunk_counts[(size_t)(c + i) * E + e_mine] = rank;
+        rank += x[i];
       }
+      running += __shfl(inc, 63, 64);
     }
+    if (lane == 0) expert_count[e_mine] = running;
   }
-  const int e = threadIdx.x;
-  int count = 0;
-  if (e < E)
-    for (int q = 0; q < P; q++) count += partial[q * epad + e];
-  int total;
-  int off = block_exclusive_scan(count, wave_sums, total);
-  int tiles = (count + tile_m - 1) / tile_m;
-  int total_tiles;
-  int first_tile = block_exclusive_scan(tiles, wave_sums, total_tiles);
-  if (e < E) {
-    expert_offsets[e] = off;
-    tile_prefix[e] = first_tile;
+  __shared__ int is_last;
+  __threadfence();                      // this workgroup's totals are visible device-wide before its arrival is counted
+  __syncthreads();
+  if (threadIdx.x == 0) is_last = atomicAdd(arrivals, 1) == (int)gridDim.x - 1;
+  __syncthreads();
+  if (!is_last) return;
+  __threadfence();
+
+  __shared__ int wave_sums[16];
+  __shared__ int t_first[MOE_MAX_EXPERTS + 1], t_count[MOE_MAX_EXPERTS], t_off[MOE_MAX_EXPERTS];
+  // thread t owns experts 4 t .. 4 t + 3 (MOE_MAX_EXPERTS = 4 x 256 threads)
+  static_assert(MOE_MAX_EXPERTS <= 4 * 64 * kScanWaves, "four experts per thread");
+  int count[4], tiles[4], rows_mine = 0, tiles_mine = 0;
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int e = 4 * threadIdx.x + j;
+    count[j] = e < E ? __hip_atomic_load(expert_count + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0;
+    tiles[j] = (count[j] + tile_m - 1) / tile_m;
+    rows_mine += count[j];
+    tiles_mine += tiles[j];
   }
-  if (e == 0) {
+  int total, total_tiles;
+  int off = block_exclusive_scan(rows_mine, wave_sums, total);
+  int first_tile = block_exclusive_scan(tiles_mine, wave_sums, total_tiles);
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int e = 4 * threadIdx.x + j;
+    if (e < E) {
+      expert_offsets[e] = off;
+      tile_prefix[e] = first_tile;
+    }
+    if (e < MOE_MAX_EXPERTS) {
+      t_first[e] = e < E ? first_tile : total_tiles;
+      t_count[e] = count[j];
+      t_off[e] = off;
+    }
+    off += count[j];
+    first_tile += tiles[j];
+  }
+  if (threadIdx.x == 0) {
     expert_offsets[E] = total;
     tile_prefix[E] = total_tiles;
+    t_first[MOE_MAX_EXPERTS] = total_tiles;
   }
+  __syncthreads();
   // The tile list, one thread per tile: under a skewed load one expert holds hundreds of row tiles, and a loop over
   // them in that expert's thread would be the longest chain of the kernel.  A tile finds its expert by bisection of
   // the first-tile table (experts without a tile share their successor's entry and are never the answer).
-  __shared__ int t_first[1025], t_count[1024], t_off[1024];
-  t_first[e] = e < E ? first_tile : total_tiles;
-  t_count[e] = count;
-  t_off[e] = off;
-  if (e == 0) t_first[1024] = total_tiles;
-  __syncthreads();
   const int n_tiles = min(total_tiles, max_tiles);
-  for (int j = threadIdx.x; j < n_tiles; j += 1024) {
+  for (int j = threadIdx.x; j < n_tiles; j += 64 * kScanWaves) {
     int lo = 0, hi = E;                                 // t_first[lo] <= j < t_first[hi]
     while (hi - lo > 1) {
       const int mid = (lo + hi) >> 1;
@@ -254,17 +281,20 @@ int permute_quant_small_launch(hipStream_t st, const int32_t *ids, int T, int K,
 
 // zero_rows (may be null): a [T*K, row_len] bf16 tensor in slot order whose rows of slots WITHOUT an expert (id outside
 // [0, E)) are cleared here - the per-slot output form: nothing else ever writes those rows
+// counted: the routing launch has filled ws.chunk_counts and ws.arrivals is zero (more than kChunk slots only)
 int permute_launch(hipStream_t st, const int32_t *ids, int T, int K, int E, int tile_m, int32_t *sorted_slot,
-                   int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &ws, uint16_t *zero_rows, int row_len) {
+                   int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &ws, uint16_t *zero_rows, int row_len,
+                   bool counted) {
   const int TK = T * K;
   if (TK <= kChunk) {
     permute_small_kernel<<<1, kChunk, 0, st>>>(ids, TK, E, tile_m, ws.max_tiles, sorted_slot, expert_offsets, slot_to_row,
                                            ws.tile_prefix, ws.tile_expert, ws.tile_desc, zero_rows, row_len);
     return (int)hipGetLastError();
   }
-  permute_count_kernel<<<ws.n_chunks, 64, 0, st>>>(ids, TK, E, ws.chunk_counts);
-  permute_scan_kernel<<<1, 1024, 0, st>>>(ws.chunk_counts, ws.n_chunks, E, tile_m, ws.max_tiles, expert_offsets,
-                                          ws.tile_prefix, ws.tile_expert, ws.tile_desc);
+  if (!counted) permute_count_kernel<<<ws.n_chunks, 64, 0, st>>>(ids, TK, E, ws.chunk_counts, ws.arrivals);
+  permute_scan_kernel<<<(E + kScanWaves - 1) / kScanWaves, 64 * kScanWaves, 0, st>>>(
+      ws.chunk_counts, ws.n_chunks, E, tile_m, ws.max_tiles, expert_offsets, ws.tile_prefix, ws.tile_expert, ws.tile_desc,
+      ws.expert_count, ws.arrivals);
   permute_scatter_kernel<<<ws.n_chunks, kChunk, 0, st>>>(ids, TK, E, ws.chunk_counts, expert_offsets, sorted_slot,
                                                      slot_to_row, zero_rows, row_len);
   return (int)hipGetLastError();
@@ -290,5 +320,5 @@ extern "C" int moe_permute(void *stream, const int32_t *ids, int T, int K, int E
   if ((uintptr_t)workspace % 4) return MOE_E_ALIGN;
   PermuteWs ws = permute_ws_layout(workspace, T, K, E);
   return permute_launch((hipStream_t)stream, ids, T, K, E, choose_tile_m(T, K, E), sorted_slot, expert_offsets,
-                        slot_to_row, ws, nullptr, 0);
+                        slot_to_row, ws, nullptr, 0, false);
 }

@@ -212,7 +212,8 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const void *__restrict_
                                                           int n_groups, int topk_groups, int renorm, float scale,
                                                           float *__restrict__ weights_out, int32_t *__restrict__ ids_out,
                                                           float *__restrict__ scores_out, int n_slices = 0,
-                                                          const QuantRide ride = QuantRide{}) {
+                                                          const QuantRide ride = QuantRide{},
+                                                          int32_t *__restrict__ chunk_counts = nullptr) {
   if (ride.x != nullptr && (int)blockIdx.x >= ride.first_block) {
     act_quant_thread(ride.x, ride.n_groups, ride.groups_per_row, ride.pitch, ride.q, ride.s,
                      (size_t)(blockIdx.x - ride.first_block) * 256 + threadIdx.x);
@@ -287,6 +288,8 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const void *__restrict_
   if (lane < K) {
     weights_out[(size_t)t * K + lane] = w * scale;
     ids_out[(size_t)t * K + lane] = idx;
+    // the permutation's first pass on the way: slots per (chunk of kChunk slots, expert); the table starts at zero
+    if (chunk_counts != nullptr) atomicAdd(&chunk_counts[(size_t)((t * K + lane) / kChunk) * E + idx], 1);
   }
 }
 
@@ -344,9 +347,12 @@ int sum_slices_launch(hipStream_t st, const float *partial, int n_slices, int T,
 // routing straight from the partial sums of the router product
 // x / H / xq / xs: the activations [T, H] bf16 are quantised in the same launch (xq e4m3fn [T, H], xs fp32 with
 // pitch scale_pitch(H / 128)); x null: routing only.
+// chunk_counts (may be null): [ceil(T K / kChunk)][E], zero on entry; every slot is counted under its chunk and
+// expert, which is the first pass of the permutation.
 int route_from_partials_launch(hipStream_t st, const float *partial, int n_slices, const float *bias, int T, int E, int K,
                                int mode, int n_groups, int topk_groups, int renorm, float scale, float *weights_out,
-                               int32_t *ids_out, const uint16_t *x, int H, uint8_t *xq, float *xs) {
+                               int32_t *ids_out, const uint16_t *x, int H, uint8_t *xq, float *xs,
+                               int32_t *chunk_counts) {
   if (n_slices < 1 || n_slices > 8) return MOE_E_SHAPE;
   if (mode != MOE_ROUTE_SOFTMAX && mode != MOE_ROUTE_SIGMOID && mode != MOE_ROUTE_SOFTMAX_LOGIT_BIAS) return MOE_E_MODE;
   const int rc = check_route_shape(T, E, K, n_groups, topk_groups);
@@ -367,7 +373,7 @@ int route_from_partials_launch(hipStream_t st, const float *partial, int n_slice
   dim3 grid((unsigned)blocks), block(256);
 #define MOE_LAUNCH_ROUTE_PARTIALS(P)                                                                               \
   route_topk_kernel<P><<<grid, block, 0, st>>>(partial, 0, bias, T, E, K, mode, n_groups, topk_groups, renorm, scale, \
-                                               weights_out, ids_out, nullptr, n_slices, ride)
+                                               weights_out, ids_out, nullptr, n_slices, ride, chunk_counts)
   if (E <= 64) MOE_LAUNCH_ROUTE_PARTIALS(1);
   else if (E <= 128) MOE_LAUNCH_ROUTE_PARTIALS(2);
   else if (E <= 256) MOE_LAUNCH_ROUTE_PARTIALS(4);

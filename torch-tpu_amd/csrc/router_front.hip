@@ -32,9 +32,12 @@ __device__ __forceinline__ uint32_t rf_lds_offset(const void *p) { return (uint3
 __global__ __launch_bounds__(256) void router_logits_splitk_kernel(const uint8_t *__restrict__ x,
                                                                    const uint8_t *__restrict__ wr, int T, int H, int E,
                                                                    int n_slices, int blocks_per_slice, int n_eblocks,
-                                                                   float *__restrict__ partial) {
+                                                                   float *__restrict__ partial,
+                                                                   int32_t *__restrict__ zero, int n_zero) {
   __shared__ RfSmem sm;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // the counters of the permutation that follows start at zero (the routing kernel adds to them)
+  for (int i = blockIdx.x * 256 + tid; i < n_zero; i += gridDim.x * 256) zero[i] = 0;
   const int li = lane & 15, lg = lane >> 4;
   // workgroup id = ((token block) * n_eblocks + expert block) * n_slices + slice: the workgroups that share a token
   // block, and then an expert block, are neighbours in launch order
@@ -145,7 +148,9 @@ size_t router_front_partial_bytes(int T, int H, int E) {
 }
 
 // x [T, H] bf16, wr [E, H] bf16 -> partial [n_slices][T][E] fp32.  The caller has checked pointers and alignment.
-int router_front_launch(hipStream_t st, const void *x, int T, int H, const void *wr, int E, float *partial, int *n_slices_out) {
+// zero / n_zero: integers the launch clears on the way (may be null / 0).
+int router_front_launch(hipStream_t st, const void *x, int T, int H, const void *wr, int E, float *partial, int *n_slices_out,
+                        int32_t *zero, int n_zero) {
   if (T < 1 || E < 1 || E > MOE_MAX_EXPERTS || H % kBlock) return MOE_E_SHAPE;
   // per-lane source offsets are 32-bit
   if ((double)T * H * 2 >= 2147483648.0 || (double)E * H * 2 >= 2147483648.0) return MOE_E_SHAPE;
@@ -155,7 +160,7 @@ int router_front_launch(hipStream_t st, const void *x, int T, int H, const void 
   const long blocks = (long)((T + kRfTokens - 1) / kRfTokens) * n_eblocks * s;
   if (blocks > 0x7fffffffl) return MOE_E_SHAPE;
   router_logits_splitk_kernel<<<(unsigned)blocks, 256, 0, st>>>((const uint8_t *)x, (const uint8_t *)wr, T, H, E, s, per,
-                                                                n_eblocks, partial);
+                                                                n_eblocks, partial, zero, n_zero);
   *n_slices_out = s;
   return (int)hipGetLastError();
 }

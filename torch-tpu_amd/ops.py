@@ -241,6 +241,12 @@ def fused_experts_fp8(x, w13, w13_scale, w2, w2_scale, ids, routing_weights=None
     return out
 
 
+def set_shared_overlap(enabled: bool) -> bool:
+    """Batches of 512 tokens and more: `layer_fp8` runs the shared expert's first GEMM on a stream of the library's
+    own beside the router product, routing and permutation (same results bit for bit).  Returns the previous setting."""
+    return bool(lib.moe_set_shared_overlap(1 if enabled else 0))
+
+
 def layer_eligible(T: int, E: int, K: int) -> bool:
     """Shapes the one-call entry point takes (layer_fp8): any batch, up to 1024 experts."""
     return T >= 0 and 1 <= K <= E <= 1024
