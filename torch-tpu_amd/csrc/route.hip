@@ -3,7 +3,8 @@
 // A row of E <= 1024 scores lives in registers, element e in lane e % 64, register e / 64
 // (coalesced loads).  Every arg-max is a butterfly over the wave on (value, index) pairs with
 // "greater value, then lower index" as the order, so equal scores resolve to the lower index
-// on every lane identically and the K picks come out in descending order.
+// on every lane identically and the K picks come out in descending order.  (value, index) travels as one
+// 64-bit key, so a comparison is one instruction.
 #include "moe_common.h"
 #include "moe_layout.h"
 #include "act_quant.h"
@@ -13,55 +14,65 @@
 namespace moe {
 
 
-struct Best {
-  float v;
-  int i;   // element index, or INT_MAX when the lane has no candidate
-};
+// A candidate is one 64-bit key: the score's bits mapped monotonically onto unsigned integers in the upper half
+// (-0 counts as +0, NaN sorts below -inf: it never wins), the complement of the element index in the lower half.
+// "Greater value, then lower index" is then a single unsigned comparison, candidates of one row never compare equal,
+// and 0 - below every real candidate - stands for "no candidate".
+typedef unsigned long long cand_t;
 
-__device__ __forceinline__ bool better(float av, int ai, float bv, int bi) {
-  // candidates with i == INT_MAX lose to everything
-  if (bi == 0x7fffffff) return true;
-  if (ai == 0x7fffffff) return false;
-  return (av > bv) || (av == bv && ai < bi);
+__device__ __forceinline__ uint32_t ordered_bits(float x) {
+  uint32_t b = __float_as_uint(x);
+  if (x == 0.f) b = 0;
+  uint32_t u = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+  if (x != x) u = 1;
+  return u;
+}
+__device__ __forceinline__ cand_t make_cand(float v, int index) {
+  return ((cand_t)ordered_bits(v) << 32) | (uint32_t)~index;
+}
+__device__ __forceinline__ int cand_index(cand_t c) { return (int)~(uint32_t)c; }       // c != 0
+__device__ __forceinline__ float cand_value(cand_t c) {                                 // c != 0
+  const uint32_t u = (uint32_t)(c >> 32);
+  return __uint_as_float((u & 0x80000000u) ? (u & 0x7fffffffu) : ~u);
 }
 
 // Arg-max over the wavefront with data-parallel-primitive moves (no LDS round trips): an inclusive
 // scan inside each row of 16 lanes (row_shr 1, 2, 4, 8), then row 0 -> 1 and 2 -> 3 (row_bcast:15),
 // then rows 0-1 -> 2-3 (row_bcast:31); lane 63 ends up with the winner, which is broadcast.
-// Lanes that have no source in a move see a candidate that loses to everything.
+// Lanes that have no source in a move see "no candidate".
 template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ void argmax_step(Best &b) {
-  const float ov = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, b.v), CTRL, ROW_MASK, 0xf, false));
-  const int oi = __builtin_amdgcn_update_dpp(0x7fffffff, b.i, CTRL, ROW_MASK, 0xf, false);
-  if (!better(b.v, b.i, ov, oi)) { b.v = ov; b.i = oi; }
+__device__ __forceinline__ void argmax_step(cand_t &c) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)c, CTRL, ROW_MASK, 0xf, false);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(c >> 32), CTRL, ROW_MASK, 0xf, false);
+  const cand_t o = ((cand_t)hi << 32) | lo;
+  c = o > c ? o : c;
 }
 
-__device__ __forceinline__ Best wave_argmax(Best b) {
-  argmax_step<0x111, 0xf>(b);   // row_shr:1
-  argmax_step<0x112, 0xf>(b);   // row_shr:2
-  argmax_step<0x114, 0xf>(b);   // row_shr:4
-  argmax_step<0x118, 0xf>(b);   // row_shr:8
-  argmax_step<0x142, 0xa>(b);   // row_bcast:15 into rows 1 and 3
-  argmax_step<0x143, 0xc>(b);   // row_bcast:31 into rows 2 and 3
-  Best r;
-  r.v = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, b.v), 63));
-  r.i = __builtin_amdgcn_readlane(b.i, 63);
-  return r;
+__device__ __forceinline__ cand_t read_cand(cand_t c, int src_lane) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)c, src_lane);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(c >> 32), src_lane);
+  return ((cand_t)hi << 32) | lo;
+}
+
+__device__ __forceinline__ cand_t wave_argmax(cand_t c) {
+  argmax_step<0x111, 0xf>(c);   // row_shr:1
+  argmax_step<0x112, 0xf>(c);   // row_shr:2
+  argmax_step<0x114, 0xf>(c);   // row_shr:4
+  argmax_step<0x118, 0xf>(c);   // row_shr:8
+  argmax_step<0x142, 0xa>(c);   // row_bcast:15 into rows 1 and 3
+  argmax_step<0x143, 0xc>(c);   // row_bcast:31 into rows 2 and 3
+  return read_cand(c, 63);
 }
 
 // Arg-max inside each half of the wavefront (lanes 0-31 and 32-63 separately); every lane ends up with
 // the winner of its own half.
-__device__ __forceinline__ Best half_argmax(Best b, int lane) {
-  argmax_step<0x111, 0xf>(b);   // row_shr:1
-  argmax_step<0x112, 0xf>(b);   // row_shr:2
-  argmax_step<0x114, 0xf>(b);   // row_shr:4
-  argmax_step<0x118, 0xf>(b);   // row_shr:8
-  argmax_step<0x142, 0xa>(b);   // row_bcast:15 into rows 1 and 3: lanes 31 and 63 hold the halves' winners
-  Best lo, hi;
-  lo.v = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, b.v), 31));
-  lo.i = __builtin_amdgcn_readlane(b.i, 31);
-  hi.v = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, b.v), 63));
-  hi.i = __builtin_amdgcn_readlane(b.i, 63);
+__device__ __forceinline__ cand_t half_argmax(cand_t c, int lane) {
+  argmax_step<0x111, 0xf>(c);   // row_shr:1
+  argmax_step<0x112, 0xf>(c);   // row_shr:2
+  argmax_step<0x114, 0xf>(c);   // row_shr:4
+  argmax_step<0x118, 0xf>(c);   // row_shr:8
+  argmax_step<0x142, 0xa>(c);   // row_bcast:15 into rows 1 and 3: lanes 31 and 63 hold the halves' winners
+  const cand_t lo = read_cand(c, 31), hi = read_cand(c, 63);
   return lane < 32 ? lo : hi;
 }
 
@@ -100,10 +111,10 @@ __device__ __forceinline__ void select_row(float (&v)[PER_LANE], int E, int lane
       // group 2j+1, so both halves reduce at once and no range scan is needed.
 #pragma unroll
       for (int j = 0; j < PER_LANE; j++) {
-        const int e = lane + 64 * j;
-        Best b1 = half_argmax(Best{v[j], e}, lane);
-        Best b2 = half_argmax(Best{v[j], e == b1.i ? 0x7fffffff : e}, lane);
-        float sum = b1.v + (b2.i != 0x7fffffff ? b2.v : 0.f);
+        const cand_t mine = make_cand(v[j], lane + 64 * j);
+        const cand_t b1 = half_argmax(mine, lane);
+        const cand_t b2 = half_argmax(mine == b1 ? 0 : mine, lane);
+        float sum = cand_value(b1) + (b2 != 0 ? cand_value(b2) : 0.f);
         if (round_bf16) sum = round_to_bf16(sum);
         const float lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sum), 0));
         const float hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sum), 32));
@@ -114,18 +125,18 @@ __device__ __forceinline__ void select_row(float (&v)[PER_LANE], int E, int lane
       for (int g = 0; g < n_groups; g++) {
         const int lo = g * per, hi = lo + per;
         float sum = 0.f;
-        int first = -1;
+        cand_t first = 0;
         for (int pass = 0; pass < 2; pass++) {
-          Best b{0.f, 0x7fffffff};
+          cand_t b = 0;
 #pragma unroll
           for (int j = 0; j < PER_LANE; j++) {
-            int e = lane + 64 * j;
-            if (e >= lo && e < hi && e != first && !(dead >> j & 1))
-              if (better(v[j], e, b.v, b.i)) { b.v = v[j]; b.i = e; }
+            const int e = lane + 64 * j;
+            const cand_t c = make_cand(v[j], e);
+            if (e >= lo && e < hi && c != first && !(dead >> j & 1) && c > b) b = c;
           }
           b = wave_argmax(b);
-          if (b.i != 0x7fffffff) sum = (pass == 0) ? b.v : sum + b.v;
-          first = b.i;
+          if (b != 0) sum = (pass == 0) ? cand_value(b) : sum + cand_value(b);
+          first = b;
         }
         if (round_bf16) sum = round_to_bf16(sum);
         if (lane == g) gscore = sum;
@@ -148,20 +159,25 @@ __device__ __forceinline__ void select_row(float (&v)[PER_LANE], int E, int lane
 
   my_value = 0.f;
   my_index = -1;
-  for (int s = 0; s < top_k; s++) {
-    Best b{0.f, 0x7fffffff};
+  cand_t cand[PER_LANE];          // 0 once picked (and for elements beyond E)
 #pragma unroll
-    for (int j = 0; j < PER_LANE; j++) {
-      int e = lane + 64 * j;
-      if (!(dead >> j & 1))
-        if (better(v[j], e, b.v, b.i)) { b.v = v[j]; b.i = e; }
-    }
+  for (int j = 0; j < PER_LANE; j++) cand[j] = (dead >> j & 1) ? 0 : make_cand(v[j], lane + 64 * j);
+  for (int s = 0; s < top_k; s++) {
+    cand_t b = 0;
+#pragma unroll
+    for (int j = 0; j < PER_LANE; j++) b = cand[j] > b ? cand[j] : b;
     b = wave_argmax(b);
-    if (b.i == 0x7fffffff) break;           // fewer than top_k elements: cannot happen (K <= E)
+    if (b == 0) break;                      // fewer than top_k elements: cannot happen (K <= E)
 #pragma unroll
     for (int j = 0; j < PER_LANE; j++)
-      if (lane + 64 * j == b.i) dead |= 1u << j;
-    if (lane == s) { my_value = b.v; my_index = b.i; }
+      if (cand[j] == b) cand[j] = 0;
+    if (lane == s) my_index = cand_index(b);
+  }
+  // the value of pick `lane` as its owner holds it (element i lives in lane i % 64, register i / 64)
+#pragma unroll
+  for (int j = 0; j < PER_LANE; j++) {
+    const float held = __shfl(v[j], my_index >= 0 ? (my_index & 63) : 0, 64);
+    if (my_index >= 0 && (my_index >> 6) == j) my_value = held;
   }
 }
 

@@ -4,11 +4,12 @@
 // The product is short and wide (a few thousand tokens by at most 256 experts over a long reduction), so the
 // reduction is cut into slices: workgroup (block of 128 tokens, slice) leaves its fp32 partial sums, and the routing
 // kernel that follows adds the slices in a fixed order, rounds to bf16 (what a bf16 matmul leaves) and routes.
-// Four wavefronts; wavefront w owns experts 64w .. 64w+63 of the workgroup's block of 256 for all 128 tokens (8 x 4 tiles of 16 x 16: with fewer
-// tokens per workgroup the router rows, re-read by every token block, saturate the L2 -> LDS path before the matrix
-// pipe).  A step is 64 reduction elements = 128 bytes of a row = two v_mfma_f32_16x16x32_bf16 per tile pair.  Both
-// operands travel L2 -> LDS with direct loads, two steps ahead, through three stages: the token tile (shared, one
-// barrier per step) and each wavefront's own 64 router rows (loaded and read by the same wavefront).
+// Eight wavefronts, two per SIMD, so that one's LDS reads and barrier waits hide behind the other's matrix
+// instructions: wavefront (token half, expert quarter) owns 64 tokens x 64 experts of the workgroup's 128 tokens x
+// block of 256 experts (4 x 4 tiles of 16 x 16; with fewer tokens per workgroup the router rows, re-read by every
+// token block, saturate the L2 -> LDS path before the matrix pipe).  A step is 64 reduction elements = 128 bytes of a
+// row = two v_mfma_f32_16x16x32_bf16 per tile pair.  Both operands travel L2 -> LDS with direct loads, two steps
+// ahead, through three stages, one barrier per step.
 #include "moe_common.h"
 #include "moe_layout.h"
 #include "../../include/moe_hip.h"
@@ -29,7 +30,9 @@ struct RfSmem {
 typedef __attribute__((address_space(3))) uint8_t rf_lds_byte;
 __device__ __forceinline__ uint32_t rf_lds_offset(const void *p) { return (uint32_t)(uintptr_t)(rf_lds_byte *)p; }
 
-__global__ __launch_bounds__(256) void router_logits_splitk_kernel(const uint8_t *__restrict__ x,
+constexpr int kRfThreads = 512;
+
+__global__ __launch_bounds__(kRfThreads) void router_logits_splitk_kernel(const uint8_t *__restrict__ x,
                                                                    const uint8_t *__restrict__ wr, int T, int H, int E,
                                                                    int n_slices, int blocks_per_slice, int n_eblocks,
                                                                    float *__restrict__ partial,
@@ -37,8 +40,9 @@ __global__ __launch_bounds__(256) void router_logits_splitk_kernel(const uint8_t
   __shared__ RfSmem sm;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   // the counters of the permutation that follows start at zero (the routing kernel adds to them)
-  for (int i = blockIdx.x * 256 + tid; i < n_zero; i += gridDim.x * 256) zero[i] = 0;
+  for (int i = blockIdx.x * kRfThreads + tid; i < n_zero; i += gridDim.x * kRfThreads) zero[i] = 0;
   const int li = lane & 15, lg = lane >> 4;
+  const int wm = wave & 1, wn = wave >> 1;                // token half, expert quarter
   // workgroup id = ((token block) * n_eblocks + expert block) * n_slices + slice: the workgroups that share a token
   // block, and then an expert block, are neighbours in launch order
   const int slice = blockIdx.x % n_slices, eb = (blockIdx.x / n_slices) % n_eblocks, e0 = eb * 256;
@@ -54,29 +58,30 @@ __global__ __launch_bounds__(256) void router_logits_splitk_kernel(const uint8_t
   // direct-to-LDS loads: one instruction moves 8 rows x 128 bytes; lane l fetches row l/8 and the chunk that
   // belongs at position l%8 of the swizzled row
   const int sub = lane >> 3, chunk = (lane & 7) ^ sub;
-  constexpr int NX = kRfTokens / 32;              // token-tile instructions per wavefront and step
-  uint32_t x_src[NX], w_src[8];
+  constexpr int NX = kRfTokens / 64, NWR = 4;     // token-tile and router-row instructions per wavefront and step
+  uint32_t x_src[NX], w_src[NWR];
 #pragma unroll
   for (int u = 0; u < NX; u++) x_src[u] = (uint32_t)min(m0 + 8 * (NX * wave + u) + sub, T - 1) * (uint32_t)row_bytes + chunk * 16;
 #pragma unroll
-  for (int u = 0; u < 8; u++) w_src[u] = (uint32_t)min(e0 + 64 * wave + 8 * u + sub, E - 1) * (uint32_t)row_bytes + chunk * 16;
+  for (int u = 0; u < NWR; u++) w_src[u] = (uint32_t)min(e0 + 8 * (NWR * wave + u) + sub, E - 1) * (uint32_t)row_bytes + chunk * 16;
   const uint32_t x_lds = __builtin_amdgcn_readfirstlane(rf_lds_offset(&sm.x[0][0])) + (NX * wave) * 1024;
-  const uint32_t w_lds = __builtin_amdgcn_readfirstlane(rf_lds_offset(&sm.w[0][0])) + (8 * wave) * 1024;
+  const uint32_t w_lds = __builtin_amdgcn_readfirstlane(rf_lds_offset(&sm.w[0][0])) + (NWR * wave) * 1024;
   auto request = [&](int step) {
     const uint8_t *xb = xbase + (size_t)step * 128, *wb = wbase + (size_t)step * 128;
-    const uint32_t xm = x_lds + (step % kRfXStages) * (kRfTokens * 128), wm = w_lds + (step % kRfWStages) * (256 * 128);
+    const uint32_t xm = x_lds + (step % kRfXStages) * (kRfTokens * 128), wst = w_lds + (step % kRfWStages) * (256 * 128);
 #pragma unroll
     for (int u = 0; u < NX; u++)
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(xm + u * 1024), "v"(x_src[u]), "s"(xb) : "memory", "m0");
 #pragma unroll
-    for (int u = 0; u < 8; u++)
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(wm + u * 1024), "v"(w_src[u]), "s"(wb) : "memory", "m0");
+    for (int u = 0; u < NWR; u++)
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(wst + u * 1024), "v"(w_src[u]), "s"(wb) : "memory", "m0");
   };
-  constexpr int kLoadsPerStep = NX + 8;
+  constexpr int kLoadsPerStep = NX + NWR;
+  constexpr int kWaveMT = kRfMT / 2;              // row tiles of a wavefront
 
-  v4f acc[kRfMT][4];
+  v4f acc[kWaveMT][4];
 #pragma unroll
-  for (int i = 0; i < kRfMT; i++)
+  for (int i = 0; i < kWaveMT; i++)
 #pragma unroll
     for (int j = 0; j < 4; j++) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
 
@@ -85,44 +90,44 @@ __global__ __launch_bounds__(256) void router_logits_splitk_kernel(const uint8_t
   request(min(1, last));
   const int o0 = (lg ^ (li & 7)) << 4, o1 = ((lg + 4) ^ (li & 7)) << 4;
   for (int t = 0; t < n_steps; t++) {
-    // step t has landed (step t + 1 may still be in flight); everybody has left step t - 1, whose token stage the
+    // step t has landed (step t + 1 may still be in flight); everybody has left step t - 1, whose stages the
     // request below overwrites
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoadsPerStep) : "memory");
     __syncthreads();
     request(min(t + 2, last));          // past the end: the last step again, so that the count in flight stays the same
-    const uint8_t *xs = sm.x[t % kRfXStages] + li * 128;
-    const uint8_t *ws = sm.w[t % kRfWStages] + (64 * wave + li) * 128;
-    v4i xa[kRfMT][2], wb[4][2];
+    const uint8_t *xs = sm.x[t % kRfXStages] + (64 * wm + li) * 128;
+    const uint8_t *ws = sm.w[t % kRfWStages] + (64 * wn + li) * 128;
+    v4i xa[kWaveMT][2], wb[4][2];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       wb[i][0] = *(const v4i *)(ws + i * 2048 + o0);
       wb[i][1] = *(const v4i *)(ws + i * 2048 + o1);
     }
 #pragma unroll
-    for (int i = 0; i < kRfMT; i++) {
+    for (int i = 0; i < kWaveMT; i++) {
       xa[i][0] = *(const v4i *)(xs + i * 2048 + o0);
       xa[i][1] = *(const v4i *)(xs + i * 2048 + o1);
     }
 #pragma unroll
     for (int h = 0; h < 2; h++)
 #pragma unroll
-      for (int i = 0; i < kRfMT; i++)
+      for (int i = 0; i < kWaveMT; i++)
 #pragma unroll
         for (int j = 0; j < 4; j++)
           acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf_t, xa[i][h]),
                                                               __builtin_bit_cast(v8bf_t, wb[j][h]), acc[i][j], 0, 0, 0);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  // c[r] of tile (i, j): token m0 + 16 i + 4 (l / 16) + r, expert e0 + 64 w + 16 j + l % 16
+  // c[r] of tile (i, j): token m0 + 64 wm + 16 i + 4 (l / 16) + r, expert e0 + 64 wn + 16 j + l % 16
   float *const out = partial + (size_t)slice * T * E;
 #pragma unroll
-  for (int i = 0; i < kRfMT; i++)
+  for (int i = 0; i < kWaveMT; i++)
 #pragma unroll
     for (int r = 0; r < 4; r++) {
-      const int tok = m0 + 16 * i + 4 * lg + r;
+      const int tok = m0 + 64 * wm + 16 * i + 4 * lg + r;
 #pragma unroll
       for (int j = 0; j < 4; j++) {
-        const int e = e0 + 64 * wave + 16 * j + li;
+        const int e = e0 + 64 * wn + 16 * j + li;
         if (tok < T && e < E) out[(size_t)tok * E + e] = acc[i][j][r];
       }
     }
@@ -159,7 +164,7 @@ int router_front_launch(hipStream_t st, const void *x, int T, int H, const void 
   const int n_eblocks = (E + 255) / 256;
   const long blocks = (long)((T + kRfTokens - 1) / kRfTokens) * n_eblocks * s;
   if (blocks > 0x7fffffffl) return MOE_E_SHAPE;
-  router_logits_splitk_kernel<<<(unsigned)blocks, 256, 0, st>>>((const uint8_t *)x, (const uint8_t *)wr, T, H, E, s, per,
+  router_logits_splitk_kernel<<<(unsigned)blocks, kRfThreads, 0, st>>>((const uint8_t *)x, (const uint8_t *)wr, T, H, E, s, per,
                                                                 n_eblocks, partial, zero, n_zero);
   *n_slices_out = s;
   return (int)hipGetLastError();
