@@ -16,6 +16,7 @@
 #include <hip/hip_runtime_api.h>
 #include <torch/library.h>
 
+#include <array>
 #include <cstdio>
 #include <map>
 #include <mutex>
@@ -42,33 +43,37 @@ void *stream_of(const Tensor &t) { return (void *)c10::hip::getCurrentHIPStream(
 // dead and is dropped the next time the table is walked, so new weights that land on a recycled address never meet
 // an old copy.  An in-place write that does not move the version counter cannot be seen from here
 // (my_ops::_invalidate_weight_cache after such an update).
+// (three dimensions: the callers of identify() have checked that)
 struct SourceId {
   const c10::StorageImpl *storage;
   const void *data;
   int64_t offset;
   uint32_t version;
   c10::ScalarType dtype;
-  std::vector<int64_t> sizes, strides;
+  int64_t sizes[3], strides[3];
   bool operator==(const SourceId &o) const {
-    return storage == o.storage && data == o.data && offset == o.offset && version == o.version && dtype == o.dtype &&
-           sizes == o.sizes && strides == o.strides;
+    bool same = storage == o.storage && data == o.data && offset == o.offset && version == o.version && dtype == o.dtype;
+    for (int i = 0; i < 3; i++) same = same && sizes[i] == o.sizes[i] && strides[i] == o.strides[i];
+    return same;
   }
 };
 
 SourceId identify(const Tensor &t) {
   SourceId s;
-  s.storage = t.storage().unsafeGetStorageImpl();
+  s.storage = t.unsafeGetTensorImpl()->unsafe_storage().unsafeGetStorageImpl();
   s.data = t.data_ptr();
   s.offset = t.storage_offset();
   s.version = t.is_inference() ? 0u : (uint32_t)t._version();
   s.dtype = t.scalar_type();
-  s.sizes = t.sizes().vec();
-  s.strides = t.strides().vec();
+  for (int i = 0; i < 3; i++) {
+    s.sizes[i] = t.size(i);
+    s.strides[i] = t.stride(i);
+  }
   return s;
 }
 
 struct PackedEntry {
-  std::vector<SourceId> ids;
+  std::array<SourceId, 6> ids;
   std::vector<c10::weak_intrusive_ptr<c10::StorageImpl>> alive;
   Tensor w13, w13s, w2, w2s;
 };
@@ -93,9 +98,8 @@ Tensor tile_block(const Tensor &w) {
 const PackedEntry &packed_weights(const Tensor &gate, const Tensor &up, const Tensor &down, const Tensor &gs,
                                   const Tensor &us, const Tensor &ds) {
   const Tensor *src[6] = {&gate, &up, &down, &gs, &us, &ds};
-  std::vector<SourceId> ids;
-  ids.reserve(6);
-  for (const Tensor *t : src) ids.push_back(identify(*t));
+  std::array<SourceId, 6> ids;
+  for (int i = 0; i < 6; i++) ids[i] = identify(*src[i]);
   for (size_t i = 0; i < g_packed.size();) {
     bool dead = false;
     for (auto &w : g_packed[i].alive) dead = dead || w.expired();
@@ -108,7 +112,7 @@ const PackedEntry &packed_weights(const Tensor &gate, const Tensor &up, const Te
     i++;
   }
   PackedEntry e;
-  e.ids = std::move(ids);
+  e.ids = ids;
   for (const Tensor *t : src) e.alive.push_back(t->storage().getWeakStorageImpl());
   e.w13 = tile_block(at::cat({gate, up}, 1).contiguous());
   e.w13s = at::cat({gs, us}, 1).to(at::kFloat).contiguous();
