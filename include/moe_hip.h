@@ -176,6 +176,22 @@ int moe_fused_experts_fp8(void *stream,
                           const uint8_t *shared_w2, const float *shared_w2_scale, int I_shared,
                           void *out_bf16, int out_mode,
                           void *workspace, size_t workspace_bytes);
+/*
+ * The same with the routing weights in the dtype the caller holds them in: routing_weights_dtype MOE_DTYPE_F32 or
+ * MOE_DTYPE_BF16 (the reference's callers hand the op bf16 routing weights,
+ * python/regression/test_llm/test_moe.py:263; torch_tpu/csrc/ops/my_ops/fusedMoE.cpp:117-131 takes the tensor as it is).  bf16 weights are widened inside the weighted sum (exact), so no
+ * conversion kernel runs in front of the call, and the result equals that of moe_fused_experts_fp8 on the widened
+ * weights bit for bit.
+ */
+int moe_fused_experts_fp8_rw(void *stream,
+                             const void *x_bf16, int T, int H,
+                             const uint8_t *w13, const float *w13_scale,
+                             const uint8_t *w2, const float *w2_scale, int I, int E,
+                             const int32_t *ids, const void *routing_weights, int routing_weights_dtype, int K,
+                             const uint8_t *shared_w13, const float *shared_w13_scale,
+                             const uint8_t *shared_w2, const float *shared_w2_scale, int I_shared,
+                             void *out_bf16, int out_mode,
+                             void *workspace, size_t workspace_bytes);
 
 /*
  * Stages of the above, exposed for tests and for timing one kernel at a time.  All take

@@ -524,6 +524,11 @@ def test_my_ops_registered_from_cpp_keeps_one_packed_copy_per_weight_set(pkg, or
     ops.fused_moe_fused_experts(red, x, None, None, gate, up, down, gs, us, ds, ids, w16, *tail)
     want_red = pkg.fused_experts_fp8(x, *packed, ids, w16.float())
     assert torch.equal(red.view(torch.int16), want_red.view(torch.int16))
+    # fp32 weights are taken as they are, any other dtype or layout goes through a widened copy: same bits
+    for other in (w16.float(), w16.to(torch.float16), w16.t().contiguous().t()):
+        red2 = torch.empty_like(red)
+        ops.fused_moe_fused_experts(red2, x, None, None, gate, up, down, gs, us, ds, ids, other, *tail)
+        assert torch.equal(red2.view(torch.int16), want_red.view(torch.int16)), (other.dtype, other.stride())
     # a recorded in-place change re-packs; so do new tensors
     gs.mul_(2.0)
     ops.fused_moe_fused_experts(out2, x, None, None, gate, up, down, gs, us, ds, ids, w16, *tail)

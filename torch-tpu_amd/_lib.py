@@ -28,6 +28,9 @@ SIGNATURES = {
     "moe_scale_pitch": (c_int, [c_int]),
     "moe_act_quant": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p]),
     "moe_fused_experts_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
+    "moe_fused_experts_fp8_rw": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                         c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
+                                         c_void_p, c_int, c_void_p, c_int, c_void_p, c_size_t]),
     "moe_fused_experts_fp8": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                       c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                                       c_void_p, c_int, c_void_p, c_int, c_void_p, c_size_t]),

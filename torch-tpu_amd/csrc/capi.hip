@@ -27,8 +27,8 @@ int decode_prep_launch(hipStream_t st, const uint16_t *x, int T, int H, const ui
                        int32_t *ids, int *arrivals, uint8_t *xq, float *xs, int tile_m, int32_t *sorted_slot,
                        int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &pw);
 
-int weighted_reduce_launch(hipStream_t st, const uint16_t *y, const float *w, const uint16_t *shared_y,
-                           const int32_t *slot_to_row, int T, int K, int H, uint16_t *out);
+int weighted_reduce_launch(hipStream_t st, const uint16_t *y, const void *w, const uint16_t *shared_y,
+                           const int32_t *slot_to_row, int T, int K, int H, uint16_t *out, int w_bf16 = 0);
 size_t router_front_partial_bytes(int T, int H, int E);
 int router_front_launch(hipStream_t st, const void *x, int T, int H, const void *wr, int E, float *partial, int *n_slices_out,
                         int32_t *zero = nullptr, int n_zero = 0);
@@ -140,9 +140,9 @@ static const SideLane *side_lane(hipStream_t st) {
 // join: the shared expert's first GEMM has been launched elsewhere and this event marks its end.
 static int run_experts(void *stream, const FusedWs &w, const PermuteWs &pw, int T, int H, const uint8_t *w13,
                        const float *w13_scale, const uint8_t *w2, const float *w2_scale, int I, int E, int K,
-                       const float *routing_weights, const uint8_t *shared_w13, const float *shared_w13_scale,
+                       const void *routing_weights, const uint8_t *shared_w13, const float *shared_w13_scale,
                        const uint8_t *shared_w2, const float *shared_w2_scale, int I_sh, void *out_bf16, int out_mode,
-                       hipEvent_t join = nullptr) {
+                       hipEvent_t join = nullptr, int weights_bf16 = 0) {
   hipStream_t st = (hipStream_t)stream;
   const bool has_shared = shared_w13 != nullptr;
   // a shared expert of the routed experts' width rides in the routed launches (its tiles fill the
@@ -172,7 +172,7 @@ static int run_experts(void *stream, const FusedWs &w, const PermuteWs &pw, int 
     if (rc) return rc;
   }
   return weighted_reduce_launch(st, y, routing_weights, has_shared ? w.sh_y : nullptr, w.slot_to_row, T, K, H,
-                                (uint16_t *)out_bf16);
+                                (uint16_t *)out_bf16, weights_bf16);
 }
 
 // moe_layer_fp8: the fused-experts workspace followed by the router's own pieces
@@ -245,7 +245,19 @@ extern "C" int moe_fused_experts_fp8(void *stream, const void *x_bf16, int T, in
                                      const uint8_t *shared_w13, const float *shared_w13_scale,
                                      const uint8_t *shared_w2, const float *shared_w2_scale, int I_shared,
                                      void *out_bf16, int out_mode, void *workspace, size_t workspace_bytes) {
+  return moe_fused_experts_fp8_rw(stream, x_bf16, T, H, w13, w13_scale, w2, w2_scale, I, E, ids, routing_weights,
+                                  MOE_DTYPE_F32, K, shared_w13, shared_w13_scale, shared_w2, shared_w2_scale, I_shared,
+                                  out_bf16, out_mode, workspace, workspace_bytes);
+}
+
+extern "C" int moe_fused_experts_fp8_rw(void *stream, const void *x_bf16, int T, int H, const uint8_t *w13,
+                                        const float *w13_scale, const uint8_t *w2, const float *w2_scale, int I, int E,
+                                        const int32_t *ids, const void *routing_weights, int routing_weights_dtype,
+                                        int K, const uint8_t *shared_w13, const float *shared_w13_scale,
+                                        const uint8_t *shared_w2, const float *shared_w2_scale, int I_shared,
+                                        void *out_bf16, int out_mode, void *workspace, size_t workspace_bytes) {
   using namespace moe;
+  if (routing_weights_dtype != MOE_DTYPE_F32 && routing_weights_dtype != MOE_DTYPE_BF16) return MOE_E_MODE;
   // per-token pointers may be NULL for an empty batch (T == 0): nothing is read or written through them
   if (!w13 || !w13_scale || !w2 || !w2_scale || !workspace) return MOE_E_NULL;
   if (T != 0 && (!x_bf16 || !ids || !out_bf16)) return MOE_E_NULL;
@@ -288,7 +300,8 @@ extern "C" int moe_fused_experts_fp8(void *stream, const void *x_bf16, int T, in
     if (rc) return rc;
   }
   return run_experts(stream, w, pw, T, H, w13, w13_scale, w2, w2_scale, I, E, K, routing_weights, shared_w13,
-                     shared_w13_scale, shared_w2, shared_w2_scale, I_sh, out_bf16, out_mode);
+                     shared_w13_scale, shared_w2, shared_w2_scale, I_sh, out_bf16, out_mode, nullptr,
+                     routing_weights_dtype == MOE_DTYPE_BF16);
 }
 
 extern "C" size_t moe_layer_fp8_workspace_bytes(int T, int H, int I, int E, int K, int I_shared) {

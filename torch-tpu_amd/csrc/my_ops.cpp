@@ -237,26 +237,32 @@ Tensor fused_moe_fused_experts(const Tensor &output, const Tensor &input, const 
   void *st = stream_of(input);
   ProfileScope prof("fused_moe_fused_experts", st);
   const PackedEntry &w = packed_weights(gate_weights, up_weights, down_weights, *gate_scales, *up_scales, *down_scales);
-  const float *rw = nullptr;
+  const void *rw = nullptr;
+  int rw_dtype = MOE_DTYPE_F32;
   if (out_mode) {
-    // [T,H] form: the fp32 weighted sum over the slots; the reference's callers hold the weights in bf16
+    // [T,H] form: the fp32 weighted sum over the slots; the reference's callers hold the weights in bf16, which the
+    // library widens inside the sum
     TORCH_CHECK(routing_weights.dim() == 2 && routing_weights.size(0) == T && routing_weights.size(1) == K &&
                 routing_weights.is_cuda(), "routing_weights must be [T, K]");
     if (routing_weights.scalar_type() == at::kFloat && routing_weights.is_contiguous()) {
-      rw = routing_weights.data_ptr<float>();
+      rw = routing_weights.data_ptr();
+    } else if (routing_weights.scalar_type() == at::kBFloat16 && routing_weights.is_contiguous()) {
+      rw = routing_weights.data_ptr();
+      rw_dtype = MOE_DTYPE_BF16;
     } else {
       Tensor &buf = scratch(g_rw, input, st, (size_t)(T * K) * 4, 16384);
       Tensor view = buf.narrow(0, 0, T * K * 4).view(at::kFloat).view({T, K});
       view.copy_(routing_weights);
-      rw = view.data_ptr<float>();
+      rw = view.data_ptr();
     }
   }
   const size_t need = moe_fused_experts_workspace_bytes((int)T, (int)H, (int)I, (int)E, (int)K, 0);
   Tensor &ws = scratch(g_workspace, input, st, need, (size_t)1 << 20);
-  check_rc(moe_fused_experts_fp8(st, input.data_ptr(), (int)T, (int)H, (const uint8_t *)w.w13.data_ptr(),
-                                 w.w13s.data_ptr<float>(), (const uint8_t *)w.w2.data_ptr(), w.w2s.data_ptr<float>(),
-                                 (int)I, (int)E, select_experts.data_ptr<int32_t>(), rw, (int)K, nullptr, nullptr, nullptr,
-                                 nullptr, 0, output.data_ptr(), out_mode, ws.data_ptr(), (size_t)ws.numel()),
+  check_rc(moe_fused_experts_fp8_rw(st, input.data_ptr(), (int)T, (int)H, (const uint8_t *)w.w13.data_ptr(),
+                                    w.w13s.data_ptr<float>(), (const uint8_t *)w.w2.data_ptr(), w.w2s.data_ptr<float>(),
+                                    (int)I, (int)E, select_experts.data_ptr<int32_t>(), rw, rw_dtype, (int)K, nullptr,
+                                    nullptr, nullptr, nullptr, 0, output.data_ptr(), out_mode, ws.data_ptr(),
+                                    (size_t)ws.numel()),
            "fused_moe_fused_experts");
   return output;
 }

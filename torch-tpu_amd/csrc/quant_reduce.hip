@@ -21,7 +21,7 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const uint16_t *__restri
 // faster there; a small batch, whose rows the second GEMM has just left in the cache, keeps the plain loads.
 template <bool STREAM>
 __global__ __launch_bounds__(256) void weighted_reduce_kernel(const uint16_t *__restrict__ y,
-                                                              const float *__restrict__ w,
+                                                              const void *__restrict__ w, int w_bf16,
                                                               const uint16_t *__restrict__ shared_y,
                                                               const int32_t *__restrict__ slot_to_row, int T, int K,
                                                               int H, uint16_t *__restrict__ out) {
@@ -41,7 +41,8 @@ __global__ __launch_bounds__(256) void weighted_reduce_kernel(const uint16_t *__
     for (int i = 0; i < 8; i++) {
       const size_t slot = (size_t)t * K + min(k0 + i, K - 1);
       const bool live = k0 + i < K && (slot_to_row == nullptr || slot_to_row[slot] >= 0);
-      wk[i] = live ? w[slot] : 0.f;
+      // weights kept in bf16 by the caller are widened here (exact), fp32 ones taken as they are
+      wk[i] = !live ? 0.f : w_bf16 ? bf16_to_f32(((const uint16_t *)w)[slot]) : ((const float *)w)[slot];
       raw[i] = STREAM ? __builtin_nontemporal_load((const v4i *)(y + slot * H + c)) : *(const v4i *)(y + slot * H + c);
       if (!live) raw[i] = (v4i){0, 0, 0, 0};
     }
@@ -106,18 +107,18 @@ static int repack_launch(hipStream_t st, const void *src, int64_t rows, int row_
   return (int)hipGetLastError();
 }
 
-// slot_to_row (may be null): slots with a negative entry are left out of the sum
-int weighted_reduce_launch(hipStream_t st, const uint16_t *y, const float *w, const uint16_t *shared_y,
-                           const int32_t *slot_to_row, int T, int K, int H, uint16_t *out) {
+// slot_to_row (may be null): slots with a negative entry are left out of the sum; w: [T, K] fp32, or bf16 with w_bf16
+int weighted_reduce_launch(hipStream_t st, const uint16_t *y, const void *w, const uint16_t *shared_y,
+                           const int32_t *slot_to_row, int T, int K, int H, uint16_t *out, int w_bf16) {
   const size_t n = (size_t)T * (H / 8);
   if (n == 0) return MOE_OK;
   const size_t blocks = (n + 255) / 256;
   if (blocks > 0x7fffffffull) return MOE_E_SHAPE;
   // 256 MB of last-level cache on this GPU
   if ((size_t)T * K * H * 2 > ((size_t)256 << 20))
-    weighted_reduce_kernel<true><<<(unsigned)blocks, 256, 0, st>>>(y, w, shared_y, slot_to_row, T, K, H, out);
+    weighted_reduce_kernel<true><<<(unsigned)blocks, 256, 0, st>>>(y, w, w_bf16, shared_y, slot_to_row, T, K, H, out);
   else
-    weighted_reduce_kernel<false><<<(unsigned)blocks, 256, 0, st>>>(y, w, shared_y, slot_to_row, T, K, H, out);
+    weighted_reduce_kernel<false><<<(unsigned)blocks, 256, 0, st>>>(y, w, w_bf16, shared_y, slot_to_row, T, K, H, out);
   return (int)hipGetLastError();
 }
 
@@ -157,5 +158,5 @@ extern "C" int moe_weighted_reduce(void *stream, const void *y_bf16, const float
   if (((uintptr_t)y_bf16 % 16) || ((uintptr_t)out_bf16 % 16) || (shared_y_bf16 && ((uintptr_t)shared_y_bf16 % 16)))
     return MOE_E_ALIGN;
   return weighted_reduce_launch((hipStream_t)stream, (const uint16_t *)y_bf16, routing_weights,
-                                (const uint16_t *)shared_y_bf16, nullptr, T, K, H, (uint16_t *)out_bf16);
+                                (const uint16_t *)shared_y_bf16, nullptr, T, K, H, (uint16_t *)out_bf16, 0);
 }
