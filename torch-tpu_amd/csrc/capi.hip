@@ -88,13 +88,13 @@ static FusedWs fused_layout(void *base, int T, int H, int I, int E, int K, int I
 
 // ---- the shared expert's first GEMM beside the front end ----
 // The shared expert's first GEMM needs the quantised activations and nothing of the routing.  The router product,
-// the routing and the three permutation launches are short chains that leave most of the chip idle, so for batches
+// the routing and the permutation launches are short chains that leave most of the chip idle, so for batches
 // beyond the decode size moe_layer_fp8 runs the quantisation and that GEMM on a stream of its own while the caller's
 // stream goes through the front end: an event on the caller's stream lets the side stream start, the caller's stream
 // waits for the quantised activations before the first grouped GEMM and for the shared expert's first GEMM before
 // the second (which carries the shared expert's tiles as before).  The router product comes first on the caller's
 // stream: its workgroups need most of a compute unit's LDS, which a GEMM workgroup would not leave them.
-// To the caller the call is still work on its one stream.  One side stream and one pair of events per (device,
+// To the caller the call is still work on its one stream.  One side stream and three events per (device,
 // caller's stream), created at the first call that uses them and kept until the process ends; streams of the default
 // priority, no implicit synchronisation with the null stream.  Not used while the caller's stream is being captured
 // into a graph, nor by the entry point that allocates nothing.
