@@ -254,7 +254,9 @@ def test_permutation_reference_tables(pkg, oracle, dev, ref_fixtures, name):
 
 
 @pytest.mark.parametrize("T,E,K", [(1, 1, 1), (1, 256, 8), (32, 256, 8), (33, 8, 2), (4096, 256, 8), (1000, 1024, 32),
-                                   (5000, 3, 2), (16384, 128, 8)])
+                                   (5000, 3, 2), (16384, 128, 8),
+                                   # more than 512 chunks of 256 slots: the scan walks them in more than one round
+                                   (30000, 7, 7), (70000, 1000, 2)])
 def test_permutation_random(pkg, oracle, dev, T, E, K):
     say("permute random", T, E, K)
     sel, _ = distinct_ids(T, E, K, seed=T + E + K)
