@@ -193,5 +193,8 @@ def check_sample(pkg, oracle, x_s, ids_s, layer_dev, w_s=None, shared_dev=None, 
         assert rep.get(k, 0.0) <= MAX_WORST, f"{what}: {k} = {rep[k]:.2f}"
     # the reference's own gate is 1e-4 (python/regression/test_llm/test_moe.py:308); measured 2e-6 to 4e-6 at full layer
     # size and up to 1.0e-5 on a 50-row sample of a layer whose intermediate is 256 wide (fewer terms per output)
-    assert rep["cos_diff"] < MAX_COS_DIFF, f"{what}: cos_diff {rep['cos_diff']:.2e}"
+    # A sample of a handful of slot rows is one neighbouring code away from several times that (measured 6.9e-5 on a
+    # single row of a 256-wide layer): below eight rows the reference's gate itself is the cap.
+    cap = MAX_COS_DIFF if n * K >= 8 else 1e-4
+    assert rep["cos_diff"] < cap, f"{what}: cos_diff {rep['cos_diff']:.2e}"
     return rep
