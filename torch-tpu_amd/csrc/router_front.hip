@@ -22,9 +22,10 @@ constexpr int kRfTokens = 128;                // tokens per workgroup
 constexpr int kRfMT = kRfTokens / 16;
 constexpr int kRfXStages = 3, kRfWStages = 3;
 
+template <int EB>
 struct RfSmem {
   alignas(1024) uint8_t x[kRfXStages][kRfTokens * 128];   // [row][16-byte chunk, XOR-swizzled by row % 8]
-  alignas(1024) uint8_t w[kRfWStages][256 * 128];
+  alignas(1024) uint8_t w[kRfWStages][EB * 128];
 };
 
 typedef __attribute__((address_space(3))) uint8_t rf_lds_byte;
@@ -32,12 +33,17 @@ __device__ __forceinline__ uint32_t rf_lds_offset(const void *p) { return (uint3
 
 constexpr int kRfThreads = 512;
 
+// EB: experts per workgroup (256; 128 or 64 for a layer with no more experts than that, so that nothing is loaded or
+// multiplied for rows that do not exist); a wavefront owns EB / 4 of them
+template <int EB>
 __global__ __launch_bounds__(kRfThreads) void router_logits_splitk_kernel(const uint8_t *__restrict__ x,
                                                                    const uint8_t *__restrict__ wr, int T, int H, int E,
                                                                    int n_slices, int blocks_per_slice, int n_eblocks,
                                                                    float *__restrict__ partial,
                                                                    int32_t *__restrict__ zero, int n_zero) {
-  __shared__ RfSmem sm;
+  constexpr int EQ = EB / 4;                              // experts of a wavefront
+  constexpr int NJ = EQ / 16;                             // its expert tiles
+  __shared__ RfSmem<EB> sm;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   // the counters of the permutation that follows start at zero (the routing kernel adds to them)
   for (int i = blockIdx.x * kRfThreads + tid; i < n_zero; i += gridDim.x * kRfThreads) zero[i] = 0;
@@ -45,7 +51,7 @@ __global__ __launch_bounds__(kRfThreads) void router_logits_splitk_kernel(const 
   const int wm = wave & 1, wn = wave >> 1;                // token half, expert quarter
   // workgroup id = ((token block) * n_eblocks + expert block) * n_slices + slice: the workgroups that share a token
   // block, and then an expert block, are neighbours in launch order
-  const int slice = blockIdx.x % n_slices, eb = (blockIdx.x / n_slices) % n_eblocks, e0 = eb * 256;
+  const int slice = blockIdx.x % n_slices, eb = (blockIdx.x / n_slices) % n_eblocks, e0 = eb * EB;
   const int m0 = (blockIdx.x / (n_slices * n_eblocks)) * kRfTokens;
   const int nblk = H >> 7;
   const int b0 = slice * blocks_per_slice, b1 = min(nblk, b0 + blocks_per_slice);
@@ -58,17 +64,18 @@ __global__ __launch_bounds__(kRfThreads) void router_logits_splitk_kernel(const 
   // direct-to-LDS loads: one instruction moves 8 rows x 128 bytes; lane l fetches row l/8 and the chunk that
   // belongs at position l%8 of the swizzled row
   const int sub = lane >> 3, chunk = (lane & 7) ^ sub;
-  constexpr int NX = kRfTokens / 64, NWR = 4;     // token-tile and router-row instructions per wavefront and step
+  constexpr int NX = kRfTokens / 64, NWR = (EB / 8 + 7) / 8;   // token-tile and router-row instructions per wavefront and step
   uint32_t x_src[NX], w_src[NWR];
 #pragma unroll
   for (int u = 0; u < NX; u++) x_src[u] = (uint32_t)min(m0 + 8 * (NX * wave + u) + sub, T - 1) * (uint32_t)row_bytes + chunk * 16;
 #pragma unroll
-  for (int u = 0; u < NWR; u++) w_src[u] = (uint32_t)min(e0 + 8 * (NWR * wave + u) + sub, E - 1) * (uint32_t)row_bytes + chunk * 16;
+  for (int u = 0; u < NWR; u++)      // (64 experts: eight pieces, one per wavefront)
+    w_src[u] = (uint32_t)min(e0 + 8 * min(NWR * wave + u, EB / 8 - 1) + sub, E - 1) * (uint32_t)row_bytes + chunk * 16;
   const uint32_t x_lds = __builtin_amdgcn_readfirstlane(rf_lds_offset(&sm.x[0][0])) + (NX * wave) * 1024;
-  const uint32_t w_lds = __builtin_amdgcn_readfirstlane(rf_lds_offset(&sm.w[0][0])) + (NWR * wave) * 1024;
+  const uint32_t w_lds = __builtin_amdgcn_readfirstlane(rf_lds_offset(&sm.w[0][0])) + min(NWR * wave, EB / 8 - 1) * 1024;
   auto request = [&](int step) {
     const uint8_t *xb = xbase + (size_t)step * 128, *wb = wbase + (size_t)step * 128;
-    const uint32_t xm = x_lds + (step % kRfXStages) * (kRfTokens * 128), wst = w_lds + (step % kRfWStages) * (256 * 128);
+    const uint32_t xm = x_lds + (step % kRfXStages) * (kRfTokens * 128), wst = w_lds + (step % kRfWStages) * (EB * 128);
 #pragma unroll
     for (int u = 0; u < NX; u++)
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(xm + u * 1024), "v"(x_src[u]), "s"(xb) : "memory", "m0");
@@ -79,11 +86,11 @@ __global__ __launch_bounds__(kRfThreads) void router_logits_splitk_kernel(const 
   constexpr int kLoadsPerStep = NX + NWR;
   constexpr int kWaveMT = kRfMT / 2;              // row tiles of a wavefront
 
-  v4f acc[kWaveMT][4];
+  v4f acc[kWaveMT][NJ];
 #pragma unroll
   for (int i = 0; i < kWaveMT; i++)
 #pragma unroll
-    for (int j = 0; j < 4; j++) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < NJ; j++) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
 
   const int last = n_steps - 1;
   request(0);
@@ -96,10 +103,10 @@ __global__ __launch_bounds__(kRfThreads) void router_logits_splitk_kernel(const 
     __syncthreads();
     request(min(t + 2, last));          // past the end: the last step again, so that the count in flight stays the same
     const uint8_t *xs = sm.x[t % kRfXStages] + (64 * wm + li) * 128;
-    const uint8_t *ws = sm.w[t % kRfWStages] + (64 * wn + li) * 128;
-    v4i xa[kWaveMT][2], wb[4][2];
+    const uint8_t *ws = sm.w[t % kRfWStages] + (EQ * wn + li) * 128;
+    v4i xa[kWaveMT][2], wb[NJ][2];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < NJ; i++) {
       wb[i][0] = *(const v4i *)(ws + i * 2048 + o0);
       wb[i][1] = *(const v4i *)(ws + i * 2048 + o1);
     }
@@ -113,12 +120,12 @@ __global__ __launch_bounds__(kRfThreads) void router_logits_splitk_kernel(const 
 #pragma unroll
       for (int i = 0; i < kWaveMT; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int j = 0; j < NJ; j++)
           acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf_t, xa[i][h]),
                                                               __builtin_bit_cast(v8bf_t, wb[j][h]), acc[i][j], 0, 0, 0);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  // c[r] of tile (i, j): token m0 + 64 wm + 16 i + 4 (l / 16) + r, expert e0 + 64 wn + 16 j + l % 16
+  // c[r] of tile (i, j): token m0 + 64 wm + 16 i + 4 (l / 16) + r, expert e0 + EQ wn + 16 j + l % 16
   float *const out = partial + (size_t)slice * T * E;
 #pragma unroll
   for (int i = 0; i < kWaveMT; i++)
@@ -126,8 +133,8 @@ __global__ __launch_bounds__(kRfThreads) void router_logits_splitk_kernel(const 
     for (int r = 0; r < 4; r++) {
       const int tok = m0 + 64 * wm + 16 * i + 4 * lg + r;
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const int e = e0 + 64 * wn + 16 * j + li;
+      for (int j = 0; j < NJ; j++) {
+        const int e = e0 + EQ * wn + 16 * j + li;
         if (tok < T && e < E) out[(size_t)tok * E + e] = acc[i][j][r];
       }
     }
@@ -167,8 +174,13 @@ int router_front_launch(hipStream_t st, const void *x, int T, int H, const void 
   const int n_eblocks = (E + 255) / 256;
   const long blocks = (long)((T + kRfTokens - 1) / kRfTokens) * n_eblocks * s;
   if (blocks > 0x7fffffffl) return MOE_E_SHAPE;
-  router_logits_splitk_kernel<<<(unsigned)blocks, kRfThreads, 0, st>>>((const uint8_t *)x, (const uint8_t *)wr, T, H, E, s, per,
-                                                                n_eblocks, partial, zero, n_zero);
+#define MOE_ROUTER_PRODUCT(EB)                                                                                         \
+  router_logits_splitk_kernel<EB><<<(unsigned)blocks, kRfThreads, 0, st>>>((const uint8_t *)x, (const uint8_t *)wr, T, H, E, \
+                                                                           s, per, n_eblocks, partial, zero, n_zero)
+  if (E <= 64) MOE_ROUTER_PRODUCT(64);
+  else if (E <= 128) MOE_ROUTER_PRODUCT(128);
+  else MOE_ROUTER_PRODUCT(256);
+#undef MOE_ROUTER_PRODUCT
   *n_slices_out = s;
   return (int)hipGetLastError();
 }
