@@ -291,7 +291,7 @@ int moe_mlp_fp8(void *stream, const void *x_bf16, int M, int H, const uint8_t *w
  * Decode-size batches (T * K <= 256 slots, E <= 256): two launches stand in front of the grouped GEMMs - the router
  * logits together with the activation quantisation, then routing and permutation.  Larger batches: the
  * router product runs on the matrix cores with its reduction cut into slices, the routing kernel adds
- * the slices, and the activations are quantised by extra workgroups of that launch.  Either way the logits
+ * the slices, and the activations are quantised by extra workgroups of the permutation's scan launch.  Either way the logits
  * are fp32 sums rounded once to bf16.
  * router_w_bf16 [E, H] bf16; router_bias [E] fp32 or NULL (selection only, or part of the logits with
  * MOE_ROUTE_SOFTMAX_LOGIT_BIAS, as in moe_route_topk);

@@ -36,4 +36,15 @@ __device__ __forceinline__ void act_quant_thread(const uint16_t *__restrict__ x,
   if (sub == 0) s[(g / groups_per_row) * pitch + g % groups_per_row] = sc;
 }
 
+// A quantisation job that rides in another kernel's launch as extra workgroups of 256 threads (x null: none).
+struct QuantJob {
+  const uint16_t *x;      // [rows, groups_per_row * 128] bf16
+  uint8_t *q;             // e4m3fn, same shape
+  float *s;               // [rows, pitch] fp32
+  size_t n_groups;
+  int groups_per_row;
+  int pitch;
+  __host__ __device__ unsigned blocks() const { return x ? (unsigned)((n_groups * 16 + 255) / 256) : 0u; }
+};
+
 }  // namespace moe

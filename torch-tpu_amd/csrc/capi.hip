@@ -3,13 +3,14 @@
 #include <mutex>
 #include "moe_common.h"
 #include "moe_layout.h"
+#include "act_quant.h"
 #include "../../include/moe_hip.h"
 
 namespace moe {
 
 int permute_launch(hipStream_t st, const int32_t *ids, int T, int K, int E, int tile_m, int32_t *sorted_slot,
                    int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &ws, uint16_t *zero_rows = nullptr,
-                   int row_len = 0, bool counted = false);
+                   int row_len = 0, bool counted = false, const QuantJob *ride = nullptr);
 int permute_quant_small_launch(hipStream_t st, const int32_t *ids, int T, int K, int E, int tile_m, int32_t *sorted_slot,
                                int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &ws, uint16_t *zero_rows,
                                int row_len, const uint16_t *x, int H, uint8_t *xq, float *xs);
@@ -293,10 +294,10 @@ extern "C" int moe_fused_experts_fp8_rw(void *stream, const void *x_bf16, int T,
                                     w.slot_to_row, pw, zero_rows, H, (const uint16_t *)x_bf16, H, w.xq, w.xs);
     if (rc) return rc;
   } else {
+    // the activations are quantised by extra workgroups of the permutation's scan launch
+    const QuantJob job{(const uint16_t *)x_bf16, w.xq, w.xs, (size_t)T * (H / kBlock), H / kBlock, scale_pitch(H / kBlock)};
     rc = permute_launch(st, ids, T, K, E, choose_tile_m(T, K, E), w.sorted_slot, w.expert_offsets, w.slot_to_row, pw,
-                        zero_rows, H);
-    if (rc) return rc;
-    rc = moe_act_quant(stream, x_bf16, T, H, w.xq, w.xs);
+                        zero_rows, H, false, &job);
     if (rc) return rc;
   }
   return run_experts(stream, w, pw, T, H, w13, w13_scale, w2, w2_scale, I, E, K, routing_weights, shared_w13,
@@ -389,14 +390,18 @@ static int layer_fp8_run(void *stream, const void *x_bf16, int T, int H, const v
       rc = router_front_launch(st, x_bf16, T, H, router_w_bf16, E, d.partial, &n_slices, zero, n_zero);
     }
     if (rc == MOE_OK && logits_out_bf16) rc = sum_slices_launch(st, d.partial, n_slices, T, E, (uint16_t *)logits_out_bf16);
-    // the activations are quantised by extra workgroups of the routing launch (unless they already are)
+    // Unless the side stream quantises the activations, extra workgroups do: of the permutation's scan launch (a
+    // few dozen workgroups of its own), or - up to kChunk slots, where the permutation is one workgroup - of the
+    // routing launch.
+    const bool ride_in_scan = !lane && (long)T * K > kChunk;
     if (rc == MOE_OK)
       rc = route_from_partials_launch(st, d.partial, n_slices, router_bias, T, E, K, mode, n_groups, topk_groups, renorm,
-                                      scale, weights, ids, lane ? nullptr : (const uint16_t *)x_bf16, H, w.xq, w.xs,
-                                      zero);
+                                      scale, weights, ids, lane || ride_in_scan ? nullptr : (const uint16_t *)x_bf16, H,
+                                      w.xq, w.xs, zero);
+    const QuantJob job{(const uint16_t *)x_bf16, w.xq, w.xs, (size_t)T * (H / kBlock), H / kBlock, scale_pitch(H / kBlock)};
     if (rc == MOE_OK)
       rc = permute_launch(st, ids, T, K, E, choose_tile_m(T, K, E), w.sorted_slot, w.expert_offsets, w.slot_to_row, pw,
-                          nullptr, 0, counted);
+                          nullptr, 0, counted, ride_in_scan ? &job : nullptr);
     if (rc == MOE_OK && lane) rc = (int)hipStreamWaitEvent(st, lane->quantised, 0);
     if (rc) {
       if (join) (void)hipStreamWaitEvent(st, join, 0);

@@ -99,7 +99,15 @@ __global__ __launch_bounds__(64 * kScanWaves) void permute_scan_kernel(int32_t *
                                                                        int32_t *__restrict__ tile_expert,
                                                                        int32_t *__restrict__ tile_desc,
                                                                        int32_t *__restrict__ expert_count,
-                                                                       int32_t *__restrict__ arrivals) {
+                                                                       int32_t *__restrict__ arrivals, int n_scan,
+                                                                       const QuantJob ride) {
+  // The scan is a few dozen workgroups and a chain of latencies; workgroups past its own quantise the activations
+  // (pure streaming, needed only by the GEMM after the permutation) in the shadow of it.
+  if ((int)blockIdx.x >= n_scan) {
+    act_quant_thread(ride.x, ride.n_groups, ride.groups_per_row, ride.pitch, ride.q, ride.s,
+                     (size_t)(blockIdx.x - n_scan) * (64 * kScanWaves) + threadIdx.x);
+    return;
+  }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int e_mine = blockIdx.x * kScanWaves + wave;
   if (e_mine < E) {
@@ -132,7 +140,7 @@ __global__ __launch_bounds__(64 * kScanWaves) void permute_scan_kernel(int32_t *
   __shared__ int is_last;
   __threadfence();                      // this workgroup's totals are visible device-wide before its arrival is counted
   __syncthreads();
-  if (threadIdx.x == 0) is_last = atomicAdd(arrivals, 1) == (int)gridDim.x - 1;
+  if (threadIdx.x == 0) is_last = atomicAdd(arrivals, 1) == n_scan - 1;
   __syncthreads();
   if (!is_last) return;
   __threadfence();
@@ -282,9 +290,10 @@ int permute_quant_small_launch(hipStream_t st, const int32_t *ids, int T, int K,
 // zero_rows (may be null): a [T*K, row_len] bf16 tensor in slot order whose rows of slots WITHOUT an expert (id outside
 // [0, E)) are cleared here - the per-slot output form: nothing else ever writes those rows
 // counted: the routing launch has filled ws.chunk_counts and ws.arrivals is zero (more than kChunk slots only)
+// ride (may be null; more than kChunk slots only): activations quantised by extra workgroups of the scan launch
 int permute_launch(hipStream_t st, const int32_t *ids, int T, int K, int E, int tile_m, int32_t *sorted_slot,
                    int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &ws, uint16_t *zero_rows, int row_len,
-                   bool counted) {
+                   bool counted, const QuantJob *ride) {
   const int TK = T * K;
   if (TK <= kChunk) {
     permute_small_kernel<<<1, kChunk, 0, st>>>(ids, TK, E, tile_m, ws.max_tiles, sorted_slot, expert_offsets, slot_to_row,
@@ -292,9 +301,12 @@ int permute_launch(hipStream_t st, const int32_t *ids, int T, int K, int E, int 
     return (int)hipGetLastError();
   }
   if (!counted) permute_count_kernel<<<ws.n_chunks, 64, 0, st>>>(ids, TK, E, ws.chunk_counts, ws.arrivals);
-  permute_scan_kernel<<<(E + kScanWaves - 1) / kScanWaves, 64 * kScanWaves, 0, st>>>(
+  static_assert(64 * kScanWaves == 256, "a quantising workgroup has 256 threads");
+  const int n_scan = (E + kScanWaves - 1) / kScanWaves;
+  const QuantJob job = ride ? *ride : QuantJob{};
+  permute_scan_kernel<<<n_scan + job.blocks(), 64 * kScanWaves, 0, st>>>(
       ws.chunk_counts, ws.n_chunks, E, tile_m, ws.max_tiles, expert_offsets, ws.tile_prefix, ws.tile_expert, ws.tile_desc,
-      ws.expert_count, ws.arrivals);
+      ws.expert_count, ws.arrivals, n_scan, job);
   permute_scatter_kernel<<<ws.n_chunks, kChunk, 0, st>>>(ids, TK, E, ws.chunk_counts, expert_offsets, sorted_slot,
                                                      slot_to_row, zero_rows, row_len);
   return (int)hipGetLastError();
@@ -320,5 +332,5 @@ extern "C" int moe_permute(void *stream, const int32_t *ids, int T, int K, int E
   if ((uintptr_t)workspace % 4) return MOE_E_ALIGN;
   PermuteWs ws = permute_ws_layout(workspace, T, K, E);
   return permute_launch((hipStream_t)stream, ids, T, K, E, choose_tile_m(T, K, E), sorted_slot, expert_offsets,
-                        slot_to_row, ws, nullptr, 0, false);
+                        slot_to_row, ws, nullptr, 0, false, nullptr);
 }
