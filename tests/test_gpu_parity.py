@@ -47,6 +47,38 @@ def test_act_quant_bit_exact(pkg, oracle, dev, R, C):
     assert torch.equal(q.cpu().view(torch.uint8), q_ref.view(torch.uint8))
 
 
+def test_act_quant_every_value_under_every_scale(pkg, oracle, dev):
+    """The quantiser divides by its scale through a refined reciprocal instead of the IEEE division sequence.  Its
+    domain is small enough to visit completely: every finite bf16 value x under the scale of every bf16 amax >= |x|
+    (a group holds its amax first and 127 candidates after it; candidates above the amax are replaced by zero).
+    Codes and scales must equal the oracle's, which divides (oracle/moe_oracle.py: x / scale, round to nearest even)."""
+    say("act_quant, exhaustive")
+    pos = torch.arange(0, 0x7F80, dtype=torch.int32)                   # +0, denormals, normals up to the largest finite
+    vals = torch.cat([pos, pos | 0x8000]).to(torch.int16).view(torch.bfloat16)        # all 65280 finite bf16 values
+    n_groups = -(-vals.numel() // 127)
+    cand = torch.zeros(n_groups * 127, dtype=torch.bfloat16)
+    cand[:vals.numel()] = vals
+    cand = cand.view(n_groups, 127)
+    cand_abs = cand.float().abs()
+    amaxes = pos[1:].to(torch.int16).view(torch.bfloat16)              # every positive finite bf16
+    step = 96
+    for lo in range(0, amaxes.numel(), step):
+        a = amaxes[lo:lo + step]
+        x = torch.empty(a.numel(), n_groups, 128, dtype=torch.bfloat16)
+        x[:, :, 0] = a[:, None]
+        x[:, :, 1:] = torch.where(cand_abs[None] <= a.float()[:, None, None], cand[None], torch.zeros((), dtype=torch.bfloat16))
+        x = x.view(-1, 128)
+        q, sc = pkg.act_quant(x.to(dev))
+        q_ref, s_ref = oracle.act_quant_group128(x)
+        assert torch.equal(sc.cpu(), s_ref), lo
+        same = q.cpu().view(torch.uint8) == q_ref.view(torch.uint8)
+        if not bool(same.all()):
+            bad = (~same).nonzero()[0]
+            raise AssertionError(f"amax {float(x[bad[0], 0])}: x = {float(x[bad[0], bad[1]])} quantises to "
+                                 f"{int(q.cpu().view(torch.uint8)[bad[0], bad[1]])}, the oracle's code is "
+                                 f"{int(q_ref.view(torch.uint8)[bad[0], bad[1]])}")
+
+
 # ----------------------------------------------------------------------------- weight layout
 def tile_blocked_reference(w):
     """The tile-blocked byte order written as an index permutation: [tile, row, step, half, chunk, byte] ->

@@ -1,38 +1,48 @@
-// Activation quantisation of one 128-column group by 16 neighbouring lanes, as a device function:
+// Activation quantisation of one 128-column group by a few neighbouring lanes, as a device function:
 // shared by the stand-alone kernel and by the decode-size kernel that also computes the router logits.
 #pragma once
 #include "moe_common.h"
 
 namespace moe {
 
-// Thread `index` of a flat launch: group index / 16, 8 bf16 (16 bytes) per lane.  Every lane of a
-// wavefront must call it (the maximum is taken with cross-lane moves); lanes past the end do nothing.
+// A group is quantised by kQuantLanes neighbouring lanes, 16 bf16 (32 bytes) per lane: a wavefront reads 2 KB and
+// writes 1 KB of consecutive memory.
+constexpr int kQuantLanes = 8;
+// threads of a flat launch that quantises n_groups groups
+__host__ __device__ inline size_t quant_threads(size_t n_groups) { return n_groups * kQuantLanes; }
+
+// Thread `index` of such a launch.  Every lane of a wavefront must call it (the maximum is taken with cross-lane
+// moves); lanes past the end do nothing.
 __device__ __forceinline__ void act_quant_thread(const uint16_t *__restrict__ x, size_t n_groups, int groups_per_row,
                                                  int pitch, uint8_t *__restrict__ q, float *__restrict__ s,
                                                  size_t index) {
-  const size_t g = index >> 4;
-  const int sub = (int)(index & 15);
+  const size_t g = index / kQuantLanes;
+  const int sub = (int)(index % kQuantLanes);
   const bool live = g < n_groups;
-  float f[8];
+  float f[16];
   float amax = 0.f;
   if (live) {
-    v4i raw = *(const v4i *)(x + g * kBlock + sub * 8);
+    const v4i *src = (const v4i *)(x + g * kBlock + sub * 16);
+    const v4i raw[2] = {src[0], src[1]};
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      uint32_t w = (uint32_t)raw[i];
+    for (int i = 0; i < 8; i++) {
+      uint32_t w = (uint32_t)raw[i >> 2][i & 3];
       f[2 * i] = bf16_to_f32((uint16_t)(w & 0xffff));
       f[2 * i + 1] = bf16_to_f32((uint16_t)(w >> 16));
     }
 #pragma unroll
-    for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(f[i]));
+    for (int i = 0; i < 16; i++) amax = fmaxf(amax, fabsf(f[i]));
   }
-  amax = max_over_row16(amax);
+  amax = max_over_row8(amax);
   if (!live) return;
   const float sc = group_scale(amax);
-  v2i out;
-  out[0] = (int)pack4_fp8(f[0] / sc, f[1] / sc, f[2] / sc, f[3] / sc);
-  out[1] = (int)pack4_fp8(f[4] / sc, f[5] / sc, f[6] / sc, f[7] / sc);
-  *(v2i *)(q + g * kBlock + sub * 8) = out;
+  const ScaleRecip r = scale_recip(sc);
+  v4i out;
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+    out[i] = (int)pack4_fp8(div_by_scale(f[4 * i], r), div_by_scale(f[4 * i + 1], r), div_by_scale(f[4 * i + 2], r),
+                            div_by_scale(f[4 * i + 3], r));
+  *(v4i *)(q + g * kBlock + sub * 16) = out;
   if (sub == 0) s[(g / groups_per_row) * pitch + g % groups_per_row] = sc;
 }
 
@@ -44,7 +54,7 @@ struct QuantJob {
   size_t n_groups;
   int groups_per_row;
   int pitch;
-  __host__ __device__ unsigned blocks() const { return x ? (unsigned)((n_groups * 16 + 255) / 256) : 0u; }
+  __host__ __device__ unsigned blocks() const { return x ? (unsigned)((quant_threads(n_groups) + 255) / 256) : 0u; }
 };
 
 }  // namespace moe

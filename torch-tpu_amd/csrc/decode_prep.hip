@@ -138,7 +138,7 @@ int decode_prep_launch(hipStream_t st, const uint16_t *x, int T, int H, const ui
   if (rc) return rc;
   const int n_logit_blocks = E * ((T + kLogitTokens - 1) / kLogitTokens);
   const size_t groups = (size_t)T * (H / kBlock);
-  const int quant_blocks = (int)((groups * 16 + 255) / 256);
+  const int quant_blocks = (int)((quant_threads(groups) + 255) / 256);
   router_logits_quant_kernel<<<n_logit_blocks + quant_blocks, 256, 0, st>>>(x, wr, T, H, E, logits, n_logit_blocks, groups,
                                                                            H / kBlock, scale_pitch(H / kBlock), xq, xs,
                                                                            arrivals);

@@ -254,7 +254,7 @@ __global__ __launch_bounds__(kChunk) void permute_small_kernel(const int32_t *__
 }
 
 // The same with the activation quantisation in the launch: workgroup 0 permutes, the workgroups after it quantise x
-// (16 lanes per 128-column group).  At this size either is one short dependent chain; side by side they cost one launch.
+// (eight lanes per 128-column group).  At this size either is one short dependent chain; side by side they cost one launch.
 __global__ __launch_bounds__(kChunk) void permute_small_quant_kernel(
     const int32_t *__restrict__ ids, int TK, int E, int tile_m, int max_tiles, int32_t *__restrict__ sorted_slot,
     int32_t *__restrict__ expert_offsets, int32_t *__restrict__ slot_to_row, int32_t *__restrict__ tile_prefix,
@@ -279,7 +279,7 @@ int permute_quant_small_launch(hipStream_t st, const int32_t *ids, int T, int K,
                                int32_t *expert_offsets, int32_t *slot_to_row, const PermuteWs &ws, uint16_t *zero_rows,
                                int row_len, const uint16_t *x, int H, uint8_t *xq, float *xs) {
   const size_t groups = (size_t)T * (H / kBlock);
-  const unsigned quant_blocks = (unsigned)((groups * 16 + kChunk - 1) / kChunk);
+  const unsigned quant_blocks = (unsigned)((quant_threads(groups) + kChunk - 1) / kChunk);
   permute_small_quant_kernel<<<1 + quant_blocks, kChunk, 0, st>>>(ids, T * K, E, tile_m, ws.max_tiles, sorted_slot,
                                                                   expert_offsets, slot_to_row, ws.tile_prefix,
                                                                   ws.tile_expert, ws.tile_desc, zero_rows, row_len, x,

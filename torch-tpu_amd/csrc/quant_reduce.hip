@@ -139,10 +139,10 @@ extern "C" int moe_act_quant(void *stream, const void *x_bf16, int R, int C, uin
   if (R != 0 && (!x_bf16 || !q || !s)) return MOE_E_NULL;
   if (R < 0 || C < 1) return MOE_E_SHAPE;
   if (C % kBlock) return MOE_E_ALIGN;
-  if (((uintptr_t)x_bf16 % 16) || ((uintptr_t)q % 8) || ((uintptr_t)s % 64)) return MOE_E_ALIGN;
+  if (((uintptr_t)x_bf16 % 16) || ((uintptr_t)q % 16) || ((uintptr_t)s % 64)) return MOE_E_ALIGN;
   const size_t groups = (size_t)R * (C / kBlock);
   if (groups == 0) return MOE_OK;
-  const size_t blocks = (groups * 16 + 255) / 256;
+  const size_t blocks = (quant_threads(groups) + 255) / 256;
   if (blocks > 0x7fffffffull) return MOE_E_SHAPE;
   act_quant_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>((const uint16_t *)x_bf16, groups, C / kBlock,
                                                                       scale_pitch(C / kBlock), q, s);

@@ -209,7 +209,7 @@ __global__ __launch_bounds__(256) void noaux_tc_topk_kernel(const void *__restri
   }
 }
 
-// Activation quantisation riding in the routing launch: the workgroups from `first_block` on quantise x (16 lanes
+// Activation quantisation riding in the routing launch: the workgroups from `first_block` on quantise x (eight lanes
 // per 128-column group) instead of routing.  Routing is a chain of cross-lane steps per token and leaves the memory
 // system idle; the quantiser is pure streaming, so the two share the chip instead of following one another.
 struct QuantRide {
@@ -383,7 +383,7 @@ int route_from_partials_launch(hipStream_t st, const float *partial, int n_slice
     ride.groups_per_row = H / kBlock;
     ride.pitch = scale_pitch(H / kBlock);
     ride.first_block = route_blocks;
-    blocks += (long)((ride.n_groups * 16 + 255) / 256);
+    blocks += (long)((quant_threads(ride.n_groups) + 255) / 256);
   }
   if (blocks > 0x7fffffffl) return MOE_E_SHAPE;
   dim3 grid((unsigned)blocks), block(256);
