@@ -1,5 +1,6 @@
 // Host-side layout of the caller-provided workspaces (shared by the launchers).
 #pragma once
+#include <cmath>
 #include <stddef.h>
 #include <stdint.h>
 
@@ -35,9 +36,13 @@ static inline int choose_tile_m(int T, int K, int E) {
   // T=3072 2.993 / 2.404 / 2.410, T=4096 (128 rows) 3.627 / 2.924 / 2.651; Mixtral shape, T=96 (24 rows) 0.252 / 0.290 / 0.298,
   // T=192 (48 rows) 0.297 / 0.312 / 0.319, T=256 (64 rows) 0.338 / 0.319 / 0.325; Qwen3 shape under a skewed load, T=512
   // (32 rows) 0.130 / 0.140, T=768 (48 rows) 0.148 / 0.144, T=1024 0.172 / 0.156.
+  // The rule those crossovers follow: under balanced routing an expert's row count is binomial (T*K draws, 1/E each);
+  // take the smallest tile that holds mean + 2.4 standard deviations - an expert's rows with about 99 % probability.
+  // That puts the 64 | 128 boundary at 47 rows per expert on average and the 128 | 192 boundary at 103.
   const double mean = (double)T * K / E;
-  if (mean <= 40.0) return 64;
-  return mean > 104.0 ? 192 : 128;
+  const double reach = mean + 2.4 * std::sqrt(mean * (1.0 - 1.0 / E));
+  if (reach <= 64.0) return 64;
+  return reach <= 128.0 ? 128 : 192;
 }
 
 // Row tile of the dense layers (one "expert" owns every row; M > 128 rows, `items_per_row_tile` strips of the output,
