@@ -6,6 +6,7 @@
 // everything in registers (no LDS, no barrier, operands loaded straight into matrix-instruction
 // layout), and several wavefronts per SIMD hide each other's load latency.  Slices of the
 // reduction are summed by a second, tiny kernel in a fixed order, so results are reproducible.
+#include <type_traits>
 #include "moe_common.h"
 #include "moe_layout.h"
 #include "../../include/moe_hip.h"
@@ -36,12 +37,16 @@ __device__ __forceinline__ v8i cat8(v4i a, v4i b) {
 // NTW  weight tiles of 16 rows per work item: every token operand loaded from L2 serves NTW matrix
 //      instructions (wide layers), or 1 to get the most work items out of a narrow layer
 // STREAM  the weights are read once and are too many for the caches: non-temporal loads
+// a workgroup is one wavefront: the dispatcher then spreads the work items over the compute units one by one (with
+// four per workgroup a 7168 x 36864 layer put 8 wavefronts on some units and 12 on others, and ran 6 % longer)
+constexpr int kDsWaves = 1;
 template <int MT, int NTW, bool STREAM>
-__global__ __launch_bounds__(256) void dense_small_kernel(const SmallArgs a) {
-  constexpr int U = NTW == 1 ? 4 : 2;                    // reduction steps loaded together
+__global__ __launch_bounds__(64 * kDsWaves) void dense_small_kernel(const SmallArgs a) {
+  constexpr int U = NTW == 1 ? 4 : 1;                    // reduction steps of one load batch
+  constexpr int NB = NTW == 1 ? 1 : 2;                   // batches held in registers
   const int lane = threadIdx.x & 63, li = lane & 15, lg = lane >> 4;
   const int n_tiles = a.N / (16 * NTW);
-  long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);  // (row chunk, slice, weight tile group), the last fastest
+  long item = (long)blockIdx.x * kDsWaves + (threadIdx.x >> 6);  // (row chunk, slice, weight tile group), the last fastest
   const int nt = (int)(item % n_tiles);
   item /= n_tiles;
   const int sp = (int)(item % a.n_splits);
@@ -67,9 +72,15 @@ __global__ __launch_bounds__(256) void dense_small_kernel(const SmallArgs a) {
   for (int j = 0; j < NTW; j++)
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) acc[j][mt] = (v4f){0.f, 0.f, 0.f, 0.f};
-  for (int kb = kb0; kb < kb1; kb += U) {
-    v4i wl[U][NTW], wh[U][NTW], xl[U][MT], xh[U][MT];
-    float f[U][MT];
+  // Wide layers (NTW = 4): two batches of one step in registers; the loads of the next batch are issued before the
+  // matrix work of the current one, so a wavefront always has a batch in flight (with one batch, loaded and then
+  // consumed, only the other wavefronts of the SIMD cover its load latency: the weight stream of a 7168 x 36864 layer
+  // ran at 3.9 TB/s, now 5 TB/s).  Narrow layers (NTW = 1): slices of a few steps, one batch of four steps per pass -
+  // most items are a single round trip to memory.  The sums are formed in the same order either way.
+  v4i wl[NB][U][NTW], wh[NB][U][NTW], xl[NB][U][MT], xh[NB][U][MT];
+  float f[NB][U][MT];
+  auto load = [&](auto buf_c, int kb) {
+    constexpr int B = decltype(buf_c)::value;
 #pragma unroll
     for (int u = 0; u < U; u++) {
       const int kk = min(kb + u, kb1 - 1);               // past the slice: the last step again, times zero
@@ -79,29 +90,49 @@ __global__ __launch_bounds__(256) void dense_small_kernel(const SmallArgs a) {
         const v4i *lo = (const v4i *)(wp + j * wtile + (size_t)kk * 2048), *hi = lo + 64;
         // a large matrix whose rows fit one work item per weight tile is read once, every byte: streamed with the
         // non-temporal hint (7 % faster on a 7168 x 18432 gated MLP at 32 rows)
-        if (STREAM) { wl[u][j] = __builtin_nontemporal_load(lo); wh[u][j] = __builtin_nontemporal_load(hi); }
-        else { wl[u][j] = *lo; wh[u][j] = *hi; }
+        if (STREAM) { wl[B][u][j] = __builtin_nontemporal_load(lo); wh[B][u][j] = __builtin_nontemporal_load(hi); }
+        else { wl[B][u][j] = *lo; wh[B][u][j] = *hi; }
       }
 #pragma unroll
       for (int mt = 0; mt < MT; mt++) {
-        xl[u][mt] = *(const v4i *)(xp[mt] + (size_t)kk * 128);
-        xh[u][mt] = *(const v4i *)(xp[mt] + (size_t)kk * 128 + 64);
-        f[u][mt] = sap[mt][kk] * sb;
+        xl[B][u][mt] = *(const v4i *)(xp[mt] + (size_t)kk * 128);
+        xh[B][u][mt] = *(const v4i *)(xp[mt] + (size_t)kk * 128 + 64);
+        f[B][u][mt] = sap[mt][kk] * sb;
       }
     }
+  };
+  auto compute = [&](auto buf_c) {
+    constexpr int B = decltype(buf_c)::value;
 #pragma unroll
     for (int u = 0; u < U; u++) {
 #pragma unroll
       for (int mt = 0; mt < MT; mt++) {
-        const v8i xc = cat8(xl[u][mt], xh[u][mt]);
+        const v8i xc = cat8(xl[B][u][mt], xh[B][u][mt]);
 #pragma unroll
         for (int j = 0; j < NTW; j++) {
           const v4f zero = {0.f, 0.f, 0.f, 0.f};
-          const v4f p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(cat8(wl[u][j], wh[u][j]), xc, zero, 0, 0, 0, 0, 0, 0);
+          const v4f p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(cat8(wl[B][u][j], wh[B][u][j]), xc, zero, 0, 0, 0, 0, 0, 0);
 #pragma unroll
-          for (int r = 0; r < 4; r++) acc[j][mt][r] = fmaf(p[r], f[u][mt], acc[j][mt][r]);
+          for (int r = 0; r < 4; r++) acc[j][mt][r] = fmaf(p[r], f[B][u][mt], acc[j][mt][r]);
         }
       }
+    }
+  };
+  using buf0 = std::integral_constant<int, 0>;
+  if constexpr (NB == 1) {
+    for (int kb = kb0; kb < kb1; kb += U) {
+      load(buf0{}, kb);
+      compute(buf0{});
+    }
+  } else {
+    load(buf0{}, kb0);
+    for (int kb = kb0; kb < kb1; kb += 2 * U) {
+      // a batch past the end of the slice is the last step again with factor zero: loaded (from cache), never computed
+      load(std::integral_constant<int, NB - 1>{}, kb + U);
+      compute(buf0{});
+      if (kb + U >= kb1) break;
+      load(buf0{}, kb + 2 * U);
+      compute(std::integral_constant<int, NB - 1>{});
     }
   }
   // a lane holds output columns (tile)*16 + 4*lg .. +3 of token row li of each m-tile
@@ -194,7 +225,13 @@ void dense_small_plan(int M, int K, int N, int *n_splits, int *split_len, int *r
   const int ntw = (N % 64 == 0 && (long)(N / 64) * chunks * (NKB / 8) >= 1024) ? 4 : 1;
   *tiles_per_item = ntw;
   const long tiles = (long)(N / (16 * ntw)) * chunks;
-  long want = (2048 + tiles - 1) / tiles;                // ~2 wavefronts per SIMD over 256 CUs
+  // wavefront-sized work items: about two per SIMD for a narrow layer; fewer and longer for a wide one, whose items keep
+  // a load batch in flight on their own.  Measured on 7168 x 36864, product alone, 4096 / 2048 / 1536 / 1024 / 576
+  // items wanted: 32 rows - / 62 / 62 / 60 / - us (gated MLP 18432: 0.118 / 0.101 / - / 0.096 / 0.125 ms), 128 rows
+  // - / 159 / 159 / 129 us; up to 16 rows (little matrix work between the loads) 1 row 46.8 / 46.2 / 50.3 us,
+  // 16 rows 51.7 / 50.3 / 48.3 us
+  const int target = ntw == 1 ? 2048 : (mt == 1 ? 1536 : 1024);
+  long want = (target + tiles - 1) / tiles;
   if (want < 1) want = 1;
   int len = (int)((NKB + want - 1) / want);
   len = (len + 3) / 4 * 4;                               // whole load batches
@@ -223,13 +260,13 @@ int dense_small_launch(hipStream_t st, const uint8_t *xq, const float *xs, int M
   a.M = M; a.K = K; a.N = N; a.NKB = K / kBlock;
   const bool stream_w = a.n_mchunks == 1 && (size_t)N * K >= ((size_t)64 << 20);
   const long items = (long)(N / (16 * ntw)) * a.n_splits * a.n_mchunks;
-  const long blocks = (items + 3) / 4;
+  const long blocks = (items + kDsWaves - 1) / kDsWaves;
   if (blocks > 0x7fffffffl) return MOE_E_SHAPE;
   const unsigned g = (unsigned)blocks;
 #define MOE_DENSE_SMALL(MT, NTW)                                                          \
   do {                                                                                    \
-    if (stream_w) dense_small_kernel<MT, NTW, true><<<g, 256, 0, st>>>(a);                 \
-    else dense_small_kernel<MT, NTW, false><<<g, 256, 0, st>>>(a);                         \
+    if (stream_w) dense_small_kernel<MT, NTW, true><<<g, 64 * kDsWaves, 0, st>>>(a);                 \
+    else dense_small_kernel<MT, NTW, false><<<g, 64 * kDsWaves, 0, st>>>(a);                         \
   } while (0)
   if (ntw == 1) {
     if (rows == 16) MOE_DENSE_SMALL(1, 1);
