@@ -44,6 +44,13 @@ int dense_small_launch(hipStream_t st, const uint8_t *xq, const float *xs, int M
                        int N, uint16_t *out, float *partial, int *n_splits_out);
 int swiglu_quant_reduce_launch(hipStream_t st, const float *partial, int n_splits, int M, int I, uint8_t *hq, float *hs);
 constexpr int kDenseSmallRows = 128;        // up to this many rows the per-wavefront dense kernel is used
+// A single product of few rows: the per-wavefront kernel slices the reduction over the chip, which is what a narrow
+// layer with a long reduction needs (16384 -> 1024 at 64 rows: 28 us against 67 us for the grouped kernel's 16 strips).
+// A wide layer gives the grouped kernel's 64-column strips enough workgroups by itself, and they stream through the
+// deeper LDS ring (7168 -> 36864 at 32 / 64 / 128 rows: 57 / 71 / 59 us against 61 / 88 / 129 us; the boundary lies
+// between 7168 and 12288 columns for reductions of 4096 and 7168), and under a short reduction both are a couple of
+// launch latencies, of which the grouped path has one fewer (no slices to add).
+static inline bool mm_uses_small_kernel(int M, int K, int N) { return M <= kDenseSmallRows && N < 12288 && K > 2048; }
 
 // Carves the caller's workspace.  Every piece starts on a 256-byte boundary.
 struct FusedWs {
@@ -543,7 +550,7 @@ static DenseWs dense_layout(void *base, int M, int K, int I, int N = 0) {
     if (I > 0) {      // MLP: K = H, N = H; first product [M, 2I] over H, second [M, H] over I
       w.partial1 = (float *)take(dense_small_partial_bytes(M, K, 2 * I, true));
       w.partial = (float *)take(dense_small_partial_bytes(M, I, N, false));
-    } else {
+    } else if (mm_uses_small_kernel(M, K, N)) {
       w.partial = (float *)take(dense_small_partial_bytes(M, K, N, false));
     }
   }
@@ -572,7 +579,7 @@ extern "C" int moe_mm_fp8(void *stream, const void *x_bf16, int M, int K, const 
   if (M == 0) return MOE_OK;
   int rc = moe_act_quant(stream, x_bf16, M, K, d.xq, d.xs);
   if (rc) return rc;
-  if (M <= kDenseSmallRows)
+  if (mm_uses_small_kernel(M, K, N))
     return dense_small_launch((hipStream_t)stream, d.xq, d.xs, M, K, w, w_scale, N, (uint16_t *)out_bf16, d.partial, nullptr);
   return gemm2_launch((hipStream_t)stream, d.xq, d.xs, M, M, N, w, w_scale, K, 1, 1, nullptr, nullptr, nullptr, 0,
                       (uint16_t *)out_bf16, nullptr, nullptr, 0, nullptr, nullptr, nullptr);

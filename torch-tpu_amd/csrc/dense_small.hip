@@ -222,7 +222,9 @@ void dense_small_plan(int M, int K, int N, int *n_splits, int *split_len, int *r
   const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
   const int chunks = M > 0 ? (M + 16 * mt - 1) / (16 * mt) : 1;        // an empty batch plans like one row
   // four weight tiles per item when the layer is wide enough to still fill the chip with short slices
-  const int ntw = (N % 64 == 0 && (long)(N / 64) * chunks * (NKB / 8) >= 1024) ? 4 : 1;
+  // (with two or four m-tiles per item a lone weight tile would have the item load 2 to 4 token tiles per matrix
+  // instruction: 7168 x 7168 at 64 rows 49.5 -> 26.4 us, 4096 x 14336 52.0 -> 30.3 us with four tiles from 128 such items on)
+  const int ntw = (N % 64 == 0 && (long)(N / 64) * chunks * (NKB / 8) >= (mt == 1 ? 1024 : 128)) ? 4 : 1;
   *tiles_per_item = ntw;
   const long tiles = (long)(N / (16 * ntw)) * chunks;
   // wavefront-sized work items: about two per SIMD for a narrow layer; fewer and longer for a wide one, whose items keep
