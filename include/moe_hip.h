@@ -251,8 +251,8 @@ int moe_fused_experts_w8a16(void *stream, const void *x_bf16, int T, int H, cons
  * transpose of w [N, K] fp8 with fp32 scales [ceil(N/128), K/128].  K a multiple of 128, N a
  * multiple of 16.  Up to 128 rows a per-wavefront kernel slices the reduction over the chip and a
  * second kernel adds the slices in a fixed order (for the MLP the SwiGLU and re-quantisation ride in that
- * reduction) - for a single product only where that pays: N < 12288 under K > 2048; otherwise, and above
- * 128 rows, the grouped kernel runs with one expert.  Which of the two ran changes the order of the sums, not
+ * reduction) - for a single product only where that pays (K > 2048 and N < 12288; narrow layers keep it
+ * further: N <= 2048 up to 384 rows, N <= 1024 up to 512); otherwise the grouped kernel runs with one expert.  Which of the two ran changes the order of the sums, not
  * the arithmetic: a result is reproducible for a given (M, K, N).
  * moe_mlp_fp8 replaces at::mlp_w8a16_dq_forward -> tpudnnMlpW8A16DqAsync
  * (torch_tpu/csrc/ops/my_ops/MlpW8A16Dq.cpp:189-241): out [M, H] bf16 =

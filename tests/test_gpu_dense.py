@@ -24,7 +24,9 @@ def normalised_outside(got, ref):
 MM_SHAPES = [(32, 7168, 1536), (32, 7168, 576), (32, 2048, 7168), (64, 4096, 2048), (128, 7168, 1536),
              (256, 4096, 1024), (1, 256, 16), (200, 384, 272), (100, 4096, 8192), (128, 1024, 64),
              # few rows, wide layer or short reduction: the grouped kernels' strips instead of the per-wavefront kernel
-             (32, 4096, 14336), (1, 2304, 12288), (128, 1024, 16384), (17, 7168, 12288), (64, 2048, 7168)]
+             (32, 4096, 14336), (1, 2304, 12288), (128, 1024, 16384), (17, 7168, 12288), (64, 2048, 7168),
+             # more than 128 rows of a narrow layer under a long reduction: the per-wavefront kernel, several row chunks
+             (256, 7168, 1536), (384, 16384, 1024), (512, 7168, 512), (385, 7168, 1536), (513, 7168, 512)]
 
 
 @pytest.mark.parametrize("M,K,N", MM_SHAPES)

@@ -43,14 +43,21 @@ size_t dense_small_partial_bytes(int M, int K, int N, bool keep_partial);
 int dense_small_launch(hipStream_t st, const uint8_t *xq, const float *xs, int M, int K, const uint8_t *w, const float *ws,
                        int N, uint16_t *out, float *partial, int *n_splits_out);
 int swiglu_quant_reduce_launch(hipStream_t st, const float *partial, int n_splits, int M, int I, uint8_t *hq, float *hs);
-constexpr int kDenseSmallRows = 128;        // up to this many rows the per-wavefront dense kernel is used
+constexpr int kDenseSmallRows = 128;        // up to this many rows the gated MLP uses the per-wavefront dense kernel
 // A single product of few rows: the per-wavefront kernel slices the reduction over the chip, which is what a narrow
 // layer with a long reduction needs (16384 -> 1024 at 64 rows: 28 us against 67 us for the grouped kernel's 16 strips).
 // A wide layer gives the grouped kernel's 64-column strips enough workgroups by itself, and they stream through the
 // deeper LDS ring (7168 -> 36864 at 32 / 64 / 128 rows: 57 / 71 / 59 us against 61 / 88 / 129 us; the boundary lies
 // between 7168 and 12288 columns for reductions of 4096 and 7168), and under a short reduction both are a couple of
-// launch latencies, of which the grouped path has one fewer (no slices to add).
-static inline bool mm_uses_small_kernel(int M, int K, int N) { return M <= kDenseSmallRows && N < 12288 && K > 2048; }
+// launch latencies, of which the grouped path has one fewer (no slices to add).  A layer of at most 2048 columns keeps
+// the sliced kernel up to 384 rows, one of at most 1024 up to 512: the grouped kernel has a handful of strips there
+// (7168 -> 1536 at 129 / 256 / 384 rows: 24 / 27 / 29 us against 34 / 35 / 36 us; 16384 -> 1024: 27 / 31 / 40 against
+// 67 / 69 / 70 us; 4096 -> 4096 is already the grouped kernel's).
+static inline bool mm_uses_small_kernel(int M, int K, int N) {
+  if (K <= 2048) return false;
+  if (M <= 128) return N < 12288;
+  return (M <= 384 && N <= 2048) || (M <= 512 && N <= 1024);
+}
 
 // Carves the caller's workspace.  Every piece starts on a 256-byte boundary.
 struct FusedWs {
@@ -546,11 +553,11 @@ static DenseWs dense_layout(void *base, int M, int K, int I, int N = 0) {
     w.hq = (uint8_t *)take((size_t)M * I);
     w.hs = (float *)take((size_t)M * scale_pitch(I / kBlock) * 4);
   }
-  if (N > 0 && M <= kDenseSmallRows) {
+  if (N > 0 && (I > 0 ? M <= kDenseSmallRows : mm_uses_small_kernel(M, K, N))) {
     if (I > 0) {      // MLP: K = H, N = H; first product [M, 2I] over H, second [M, H] over I
       w.partial1 = (float *)take(dense_small_partial_bytes(M, K, 2 * I, true));
       w.partial = (float *)take(dense_small_partial_bytes(M, I, N, false));
-    } else if (mm_uses_small_kernel(M, K, N)) {
+    } else {
       w.partial = (float *)take(dense_small_partial_bytes(M, K, N, false));
     }
   }
