@@ -452,8 +452,8 @@ def bench_dense(pkg, dev, steps, warmup):
     dense tests at a decode and a prefill batch."""
     res = []
     g = torch.Generator(device=dev).manual_seed(7)
-    for kind, M, K, N in (("mm", 32, 7168, 1536), ("mm", 4096, 7168, 1536), ("mm", 4096, 2048, 7168),
-                          ("mlp", 32, 7168, 18432), ("mlp", 4096, 7168, 18432)):
+    for kind, M, K, N in (("mm", 32, 7168, 1536), ("mm", 256, 7168, 1536), ("mm", 4096, 7168, 1536), ("mm", 4096, 2048, 7168),
+                          ("mlp", 32, 7168, 18432), ("mlp", 256, 7168, 18432), ("mlp", 4096, 7168, 18432)):
         x = torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16)
         if kind == "mm":
             w, ws = make_weights(pkg, 1, N, K, dev, 31)
@@ -470,7 +470,8 @@ def bench_dense(pkg, dev, steps, warmup):
             wsp = torch.empty(_lib().moe_mlp_fp8_workspace_bytes(M, K, I), dtype=torch.uint8, device=dev)
             fn = lambda: pkg.mlp_fp8(x, w13[0], w13s[0], w2[0], w2s[0], out=out, workspace=wsp)
             flops, nbytes = 6.0 * M * K * I, 3 * K * I + 4 * M * K
-        sec = time_steps(fn, max(steps, 10), warmup)
+        # the small ones are tens of microseconds: more of them, so that a host hiccup does not show
+        sec = time_steps(fn, max(steps, 10) * (10 if M <= 256 else 1), max(warmup, 5))
         res.append(dict(op=kind, M=M, K=K, N=N, ms=sec * 1e3, tflops=flops / sec / 1e12, hbm_gbs=nbytes / sec / 1e9))
     return res
 
@@ -614,6 +615,8 @@ def main():
     ap.add_argument("--cpu-sample", type=int, default=32)
     ap.add_argument("--decode-only", type=int, default=0, metavar="T",
                     help="run only the decode leg at this batch size and print its record (for profiling one batch size)")
+    ap.add_argument("--dense-only", action="store_true",
+                    help="run only the dense layers (mm / gated MLP at 32, 256 and 4096 rows) and print their records")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures ONE GPU: the path is single-device by design (sharding the experts over several "
@@ -624,6 +627,9 @@ def main():
         sys.exit(2)
     pkg = entry.load_package()
     dev = "cuda:0"
+    if args.dense_only:
+        print(json.dumps(bench_dense(pkg, dev, args.steps, args.warmup)))
+        return
     cfg = WORKLOADS[args.workload]
     moe = build_layer(pkg, cfg, dev)
     if args.decode_only:
