@@ -843,8 +843,12 @@ static int launch_gemm(hipStream_t st, GemmArgs &a, int tile_m, int routed_tiles
   // Second GEMM with small row tiles: strips of 64 output columns instead of 256 - four times the workgroups,
   // three of them resident per compute unit, so that one's start and end hide behind the others' streams (and a
   // batch with few experts still reaches every compute unit: a workgroup alone streams at most ~37 GB/s).  The
-  // order of every sum is the same.  With 64-row tiles it only pays while the wide strips would leave units idle.
-  const bool narrow = !GATED && (km <= 32 || (km == 64 && row_tiles * ((a.N + 255) / 256) < 192));
+  // order of every sum is the same.  With 64-row tiles it only pays while the wide strips would leave units idle: two
+  // such workgroups fit a compute unit (60 KB of LDS each), so up to 128 wide work items = 512 narrow ones run in one
+  // round (a dense 7168 -> 7168 product at 288-384 rows, 140-168 wide items: 64 us in narrow strips, 46 us in wide ones).
+  // (a dense layer knows its row tiles; the tile list's entries are an upper bound, a few more than the real ones -
+  // Mixtral shape at 48-96 tokens: 9-11 entries for 8 real tiles of 16 strips each - hence the wider margin there)
+  const bool narrow = !GATED && (km <= 32 || (km == 64 && row_tiles * ((a.N + 255) / 256) < (a.fixed_expert >= 0 ? 129 : 193)));
   a.n_strips = GATED ? a.N / 128 : narrow ? (a.N + 63) / 64 : (a.N + 255) / 256;
   a.max_mtiles = routed_tiles;
   long total = row_tiles * a.n_strips;
