@@ -112,9 +112,13 @@ __global__ __launch_bounds__(kRouteBlock) void route_permute_small_kernel(
   if (gridDim.x == 1) {
     v = s < TK ? rs.isel[s] : -1;       // one token: its picks are still in LDS
   } else {
-    __threadfence();                    // this token's picks are visible device-wide before the arrival is counted
+    // this token's picks are visible device-wide before the arrival is counted: one fence per workgroup, by the
+    // thread that counts, after the barrier that orders the other wavefronts' stores before it
     __syncthreads();
-    if (threadIdx.x == 0) is_last = atomicAdd(arrivals, 1) == (int)gridDim.x - 1;
+    if (threadIdx.x == 0) {
+      __threadfence();
+      is_last = atomicAdd(arrivals, 1) == (int)gridDim.x - 1;
+    }
     __syncthreads();
     if (!is_last) return;
     __threadfence();

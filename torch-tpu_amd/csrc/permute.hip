@@ -138,9 +138,14 @@ __global__ __launch_bounds__(64 * kScanWaves) void permute_scan_kernel(int32_t *
     if (lane == 0) expert_count[e_mine] = running;
   }
   __shared__ int is_last;
-  __threadfence();                      // this workgroup's totals are visible device-wide before its arrival is counted
+  // This workgroup's totals are visible device-wide before its arrival is counted.  One fence per workgroup, by the
+  // thread that counts, after the barrier that orders the other wavefronts' stores before it: on this chip a
+  // device-scope fence writes back and invalidates the whole L2 of its XCD, so they are worth counting.
   __syncthreads();
-  if (threadIdx.x == 0) is_last = atomicAdd(arrivals, 1) == n_scan - 1;
+  if (threadIdx.x == 0) {
+    __threadfence();
+    is_last = atomicAdd(arrivals, 1) == n_scan - 1;
+  }
   __syncthreads();
   if (!is_last) return;
   __threadfence();
